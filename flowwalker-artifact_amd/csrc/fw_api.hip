@@ -1,0 +1,548 @@
+// C ABI of libflowwalker_hip.so: errors, device buffers, graph mirror, walk drivers.
+// Host-side counterpart of src/walk.cu (walk_test, walk_batch, timing_batch_async/sync),
+// include/gpu_graph.cuh (device CSR mirror) and adjust_flags' autobatch rule (src/main.cu:244-272).
+
+#include <limits.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <chrono>
+#include <new>
+#include <vector>
+
+#include "fw_internal.h"
+
+// ---- errors --------------------------------------------------------------------------------------
+
+static thread_local char g_err[512] = "";
+
+void fw_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int fw_check_hip(hipError_t e, const char* what, const char* file, int line) {
+  if (e == hipSuccess) return FW_OK;
+  fw_set_error("%s:%d HIP call \"%s\" failed with %s (%d)", file, line, what, hipGetErrorString(e), (int)e);
+  (void)hipGetLastError();
+  return FW_ERR_HIP;
+}
+
+extern "C" const char* fw_last_error(void) { return g_err; }
+
+extern "C" int fw_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+static int require_device() {
+  if (fw_device_count() <= 0) {
+    fw_set_error("no HIP device is visible; the walk engine has no CPU fallback");
+    return FW_ERR_NO_DEVICE;
+  }
+  return FW_OK;
+}
+
+extern "C" int fw_device_mem_info(size_t* free_bytes, size_t* total_bytes) {
+  int rc = require_device();
+  if (rc != FW_OK) return rc;
+  size_t f = 0, t = 0;
+  FW_HIP(hipMemGetInfo(&f, &t));
+  if (free_bytes) *free_bytes = f;
+  if (total_bytes) *total_bytes = t;
+  return FW_OK;
+}
+
+extern "C" void fw_walk_params_default(fw_walk_params* p) {
+  if (!p) return;
+  memset(p, 0, sizeof(*p));
+  p->app = FW_APP_DEEPWALK;
+  p->sampler = FW_SAMPLER_ZPRS;
+  p->max_depth = 81;
+  p->wg_threads = 512;
+  p->hub_threshold = 16384;
+  p->schema_len = 5;
+  for (int i = 0; i < 5; ++i) p->schema[i] = i;
+  p->tp = 0.2f;
+  p->p = 2.0f;
+  p->q = 0.5f;
+  p->walker_base = 0;
+  p->seed = 1337;
+  p->grid = 0;
+}
+
+extern "C" uint32_t fw_autobatch_size(size_t free_bytes, int32_t headroom_mb, int32_t max_depth, int sync,
+                                      uint32_t n_queries) {
+  const size_t headroom = (size_t)(headroom_mb > 0 ? headroom_mb : 0) * 1024u * 1024u;
+  if (max_depth < 1 || free_bytes <= headroom) return 0;
+  const int d = max_depth - 1;
+  size_t bs = (free_bytes - headroom) / (4u * (size_t)(d + 2));
+  if (bs > (size_t)INT_MAX) bs = (size_t)INT_MAX;
+  if (!sync) bs /= 2;
+  if (bs > (size_t)n_queries) bs = n_queries;
+  return (uint32_t)bs;
+}
+
+// ---- device buffers ------------------------------------------------------------------------------
+
+extern "C" int fw_dev_alloc(size_t bytes, void** d_ptr) {
+  if (!d_ptr) { fw_set_error("fw_dev_alloc: d_ptr is NULL"); return FW_ERR_INVALID; }
+  *d_ptr = nullptr;
+  int rc = require_device();
+  if (rc != FW_OK) return rc;
+  FW_HIP(hipMalloc(d_ptr, bytes ? bytes : 1));
+  return FW_OK;
+}
+extern "C" int fw_dev_free(void* d_ptr) {
+  if (!d_ptr) return FW_OK;
+  FW_HIP(hipFree(d_ptr));
+  return FW_OK;
+}
+extern "C" int fw_dev_upload(void* d_dst, const void* h_src, size_t bytes) {
+  if (bytes == 0) return FW_OK;
+  FW_HIP(hipMemcpy(d_dst, h_src, bytes, hipMemcpyHostToDevice));
+  return FW_OK;
+}
+extern "C" int fw_dev_download(void* h_dst, const void* d_src, size_t bytes) {
+  if (bytes == 0) return FW_OK;
+  FW_HIP(hipMemcpy(h_dst, d_src, bytes, hipMemcpyDeviceToHost));
+  return FW_OK;
+}
+
+__global__ void fw_fill_i32_kernel(int32_t* dst, int32_t value, size_t count) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) dst[i] = value;
+}
+extern "C" int fw_dev_fill_i32(int32_t* d_dst, int32_t value, size_t count) {
+  if (count == 0) return FW_OK;
+  size_t blocks = (count + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(fw_fill_i32_kernel, dim3((unsigned)blocks), dim3(256), 0, 0, d_dst, value, count);
+  FW_HIP(hipGetLastError());
+  FW_HIP(hipDeviceSynchronize());
+  return FW_OK;
+}
+extern "C" int fw_dev_sync(void) {
+  FW_HIP(hipDeviceSynchronize());
+  return FW_OK;
+}
+
+extern "C" int fw_host_alloc_pinned(size_t bytes, void** h_ptr) {
+  if (!h_ptr) { fw_set_error("fw_host_alloc_pinned: h_ptr is NULL"); return FW_ERR_INVALID; }
+  *h_ptr = nullptr;
+  int rc = require_device();
+  if (rc != FW_OK) return rc;
+  FW_HIP(hipHostMalloc(h_ptr, bytes ? bytes : 1, hipHostMallocDefault));
+  return FW_OK;
+}
+extern "C" int fw_host_free_pinned(void* h_ptr) {
+  if (!h_ptr) return FW_OK;
+  FW_HIP(hipHostFree(h_ptr));
+  return FW_OK;
+}
+
+// ---- graph ---------------------------------------------------------------------------------------
+
+static int validate_csr_host(int32_t V, uint64_t E, const uint32_t* xadj, const int32_t* adjncy, const float* weight) {
+  if (V <= 0) { fw_set_error("V must be positive (got %d)", V); return FW_ERR_INVALID; }
+  if (E == 0 || E > 0xFFFFFFF0ull) { fw_set_error("E must be in [1, 2^32-16] (got %llu)", (unsigned long long)E); return FW_ERR_INVALID; }
+  if (!xadj || !adjncy) { fw_set_error("xadj and adjncy are required"); return FW_ERR_INVALID; }
+  if (xadj[0] != 0u) { fw_set_error("xadj[0] must be 0"); return FW_ERR_INVALID; }
+  if ((uint64_t)xadj[V] != E) {  // include/graph.cuh:135-136
+    fw_set_error("xadj[V] = %u does not match E = %llu", xadj[V], (unsigned long long)E);
+    return FW_ERR_INVALID;
+  }
+  for (int32_t v = 0; v < V; ++v) {
+    if (xadj[v + 1] < xadj[v]) { fw_set_error("xadj is not non-decreasing at vertex %d", v); return FW_ERR_INVALID; }
+  }
+  for (uint64_t i = 0; i < E; ++i) {
+    if ((uint32_t)adjncy[i] >= (uint32_t)V) {
+      fw_set_error("adjncy[%llu] = %d is outside [0, V)", (unsigned long long)i, adjncy[i]);
+      return FW_ERR_INVALID;
+    }
+  }
+  if (weight) {
+    for (uint64_t i = 0; i < E; ++i) {
+      const float w = weight[i];
+      if (!(w >= 0.0f) || isinf(w)) {
+        fw_set_error("weight[%llu] = %g is not a finite non-negative number", (unsigned long long)i, (double)w);
+        return FW_ERR_INVALID;
+      }
+    }
+  }
+  return FW_OK;
+}
+
+template <typename T>
+static int alloc_edge_array(T** out, uint64_t E) {
+  const size_t bytes = (size_t)(E + FW_EDGE_PAD) * sizeof(T);
+  FW_HIP(hipMalloc(reinterpret_cast<void**>(out), bytes));
+  FW_HIP(hipMemset(reinterpret_cast<char*>(*out) + (size_t)E * sizeof(T), 0, FW_EDGE_PAD * sizeof(T)));
+  return FW_OK;
+}
+
+extern "C" int fw_graph_destroy(fw_graph* g) {
+  if (!g) return FW_OK;
+  int rc = FW_OK;
+  if (g->owns) {
+    void* ptrs[4] = {g->xadj, g->adjncy, g->weight, g->label};
+    for (void* p : ptrs) {
+      if (p && hipFree(p) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
+    }
+  }
+  delete g;
+  return rc;
+}
+
+extern "C" int fw_graph_create(int32_t V, uint64_t E, const uint32_t* h_xadj, const int32_t* h_adjncy,
+                               const float* h_weight, const int32_t* h_label, fw_graph** out) {
+  if (!out) { fw_set_error("fw_graph_create: out is NULL"); return FW_ERR_INVALID; }
+  *out = nullptr;
+  int rc = validate_csr_host(V, E, h_xadj, h_adjncy, h_weight);
+  if (rc != FW_OK) return rc;
+  rc = require_device();
+  if (rc != FW_OK) return rc;
+  fw_graph* g = new (std::nothrow) fw_graph();
+  if (!g) { fw_set_error("out of host memory"); return FW_ERR_NOMEM; }
+  g->V = V;
+  g->E = E;
+  g->owns = 1;
+  auto fail = [&](int code) { fw_graph_destroy(g); return code; };
+  if (hipGetDevice(&g->device) != hipSuccess) return fail(FW_ERR_HIP);
+  const size_t xbytes = (size_t)(V + 1) * sizeof(uint32_t);
+  if ((rc = fw_check_hip(hipMalloc(reinterpret_cast<void**>(&g->xadj), xbytes), "hipMalloc(xadj)", __FILE__, __LINE__))) return fail(rc);
+  if ((rc = fw_check_hip(hipMemcpy(g->xadj, h_xadj, xbytes, hipMemcpyHostToDevice), "hipMemcpy(xadj)", __FILE__, __LINE__))) return fail(rc);
+  if ((rc = alloc_edge_array(&g->adjncy, E))) return fail(rc);
+  if ((rc = fw_check_hip(hipMemcpy(g->adjncy, h_adjncy, (size_t)E * 4, hipMemcpyHostToDevice), "hipMemcpy(adjncy)", __FILE__, __LINE__))) return fail(rc);
+  if (h_weight) {
+    if ((rc = alloc_edge_array(&g->weight, E))) return fail(rc);
+    if ((rc = fw_check_hip(hipMemcpy(g->weight, h_weight, (size_t)E * 4, hipMemcpyHostToDevice), "hipMemcpy(weight)", __FILE__, __LINE__))) return fail(rc);
+  }
+  if (h_label) {
+    if ((rc = alloc_edge_array(&g->label, E))) return fail(rc);
+    if ((rc = fw_check_hip(hipMemcpy(g->label, h_label, (size_t)E * 4, hipMemcpyHostToDevice), "hipMemcpy(label)", __FILE__, __LINE__))) return fail(rc);
+  }
+  *out = g;
+  return FW_OK;
+}
+
+extern "C" int fw_graph_adopt_device(int32_t V, uint64_t E, uint32_t* d_xadj, int32_t* d_adjncy, float* d_weight,
+                                     int32_t* d_label, int take_ownership, fw_graph** out) {
+  if (!out) { fw_set_error("fw_graph_adopt_device: out is NULL"); return FW_ERR_INVALID; }
+  *out = nullptr;
+  if (V <= 0 || E == 0 || E > 0xFFFFFFF0ull || !d_xadj || !d_adjncy) {
+    fw_set_error("fw_graph_adopt_device: need V > 0, 0 < E <= 2^32-16, xadj and adjncy");
+    return FW_ERR_INVALID;
+  }
+  if ((((uintptr_t)d_adjncy) | ((uintptr_t)d_weight) | ((uintptr_t)d_label)) & 15u) {
+    fw_set_error("fw_graph_adopt_device: edge arrays must be 16-byte aligned");
+    return FW_ERR_INVALID;
+  }
+  int rc = require_device();
+  if (rc != FW_OK) return rc;
+  fw_graph* g = new (std::nothrow) fw_graph();
+  if (!g) { fw_set_error("out of host memory"); return FW_ERR_NOMEM; }
+  g->V = V; g->E = E;
+  g->xadj = d_xadj; g->adjncy = d_adjncy; g->weight = d_weight; g->label = d_label;
+  g->owns = take_ownership ? 1 : 0;
+  if (hipGetDevice(&g->device) != hipSuccess) { (void)hipGetLastError(); }
+  *out = g;
+  return FW_OK;
+}
+
+// max degree with the smallest vertex among ties: key = degree << 32 | ~vertex
+__global__ void fw_max_degree_kernel(const uint32_t* __restrict__ xadj, int32_t V, unsigned long long* best) {
+  unsigned long long local = 0ull;
+  const int stride = gridDim.x * blockDim.x;
+  for (int v = blockIdx.x * blockDim.x + threadIdx.x; v < V; v += stride) {
+    const unsigned long long d = xadj[v + 1] - xadj[v];
+    const unsigned long long key = (d << 32) | (unsigned long long)(0xFFFFFFFFu - (uint32_t)v);
+    local = key > local ? key : local;
+  }
+  atomicMax(best, local);
+}
+
+__global__ void fw_sorted_kernel(const uint32_t* __restrict__ xadj, const int32_t* __restrict__ adjncy, int32_t V,
+                                 int* unsorted) {
+  const int stride = gridDim.x * blockDim.x;
+  for (int v = blockIdx.x * blockDim.x + threadIdx.x; v < V; v += stride) {
+    const uint32_t b = xadj[v], e = xadj[v + 1];
+    for (uint32_t i = b + 1; i < e; ++i) {
+      if (adjncy[i] <= adjncy[i - 1]) { *unsorted = 1; break; }
+    }
+  }
+}
+
+extern "C" int fw_graph_info(const fw_graph* g, int32_t* V, uint64_t* E, int32_t* max_degree,
+                             int32_t* max_degree_vertex) {
+  if (!g) { fw_set_error("fw_graph_info: graph is NULL"); return FW_ERR_INVALID; }
+  if (V) *V = g->V;
+  if (E) *E = g->E;
+  if (max_degree || max_degree_vertex) {
+    fw_graph* mg = const_cast<fw_graph*>(g);
+    if (mg->max_degree < 0) {
+      unsigned long long* d_best = nullptr;
+      FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_best), sizeof(unsigned long long)));
+      FW_HIP(hipMemset(d_best, 0, sizeof(unsigned long long)));
+      hipLaunchKernelGGL(fw_max_degree_kernel, dim3(1024), dim3(256), 0, 0, g->xadj, g->V, d_best);
+      unsigned long long best = 0;
+      FW_HIP(hipMemcpy(&best, d_best, sizeof(best), hipMemcpyDeviceToHost));
+      FW_HIP(hipFree(d_best));
+      mg->max_degree = (int32_t)(best >> 32);
+      mg->max_degree_vertex = (int32_t)(0xFFFFFFFFu - (uint32_t)(best & 0xFFFFFFFFull));
+    }
+    if (max_degree) *max_degree = mg->max_degree;
+    if (max_degree_vertex) *max_degree_vertex = mg->max_degree_vertex;
+  }
+  return FW_OK;
+}
+
+extern "C" int fw_graph_is_sorted(const fw_graph* g, int* sorted) {
+  if (!g || !sorted) { fw_set_error("fw_graph_is_sorted: NULL argument"); return FW_ERR_INVALID; }
+  fw_graph* mg = const_cast<fw_graph*>(g);
+  if (mg->sorted < 0) {
+    int* d_flag = nullptr;
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_flag), sizeof(int)));
+    FW_HIP(hipMemset(d_flag, 0, sizeof(int)));
+    hipLaunchKernelGGL(fw_sorted_kernel, dim3(2048), dim3(256), 0, 0, g->xadj, g->adjncy, g->V, d_flag);
+    int flag = 0;
+    FW_HIP(hipMemcpy(&flag, d_flag, sizeof(flag), hipMemcpyDeviceToHost));
+    FW_HIP(hipFree(d_flag));
+    mg->sorted = flag ? 0 : 1;
+  }
+  *sorted = mg->sorted;
+  return FW_OK;
+}
+
+extern "C" int fw_graph_download(const fw_graph* g, uint32_t* h_xadj, int32_t* h_adjncy, float* h_weight,
+                                 int32_t* h_label) {
+  if (!g) { fw_set_error("fw_graph_download: graph is NULL"); return FW_ERR_INVALID; }
+  if (h_xadj) FW_HIP(hipMemcpy(h_xadj, g->xadj, (size_t)(g->V + 1) * 4, hipMemcpyDeviceToHost));
+  if (h_adjncy) FW_HIP(hipMemcpy(h_adjncy, g->adjncy, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+  if (h_weight) {
+    if (!g->weight) { fw_set_error("graph has no weights"); return FW_ERR_INVALID; }
+    FW_HIP(hipMemcpy(h_weight, g->weight, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+  }
+  if (h_label) {
+    if (!g->label) { fw_set_error("graph has no labels"); return FW_ERR_INVALID; }
+    FW_HIP(hipMemcpy(h_label, g->label, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+  }
+  return FW_OK;
+}
+
+// ---- walks ---------------------------------------------------------------------------------------
+
+static int check_walk_args(const fw_graph* g, const fw_walk_params* p, const void* starts, int32_t n,
+                           const void* paths) {
+  if (!g || !p || !starts || !paths) { fw_set_error("walk: NULL argument"); return FW_ERR_INVALID; }
+  if (n <= 0) { fw_set_error("walk: n must be positive (got %d)", n); return FW_ERR_INVALID; }
+  if (p->max_depth < 1) { fw_set_error("walk: max_depth must be >= 1 (got %d)", p->max_depth); return FW_ERR_INVALID; }
+  if (p->hub_threshold < 0) { fw_set_error("walk: hub_threshold must be >= 0"); return FW_ERR_INVALID; }
+  switch (p->app) {
+    case FW_APP_DEEPWALK:
+    case FW_APP_PPR:
+    case FW_APP_NODE2VEC:
+      if (!g->weight) { fw_set_error("walk: this application needs edge weights"); return FW_ERR_INVALID; }
+      break;
+    case FW_APP_METAPATH:
+      if (!g->label) { fw_set_error("walk: metapath needs edge labels"); return FW_ERR_INVALID; }
+      if (p->schema_len < 1 || p->schema_len > FW_MAX_SCHEMA) {
+        fw_set_error("walk: schema_len must be in [1, %d] (got %d)", FW_MAX_SCHEMA, p->schema_len);
+        return FW_ERR_INVALID;
+      }
+      break;
+    default:
+      fw_set_error("walk: unknown app %d", p->app);
+      return FW_ERR_INVALID;
+  }
+  if (p->app == FW_APP_PPR && !(p->tp >= 0.0f && p->tp <= 1.0f)) {
+    fw_set_error("walk: tp must be in [0,1]");
+    return FW_ERR_INVALID;
+  }
+  if (p->app == FW_APP_NODE2VEC && !(p->p > 0.0f && p->q > 0.0f)) {
+    fw_set_error("walk: p and q must be positive");
+    return FW_ERR_INVALID;
+  }
+  return FW_OK;
+}
+
+static void fill_kargs(fw_kargs* a, const fw_graph* g, const fw_walk_params* p) {
+  memset(a, 0, sizeof(*a));
+  a->xadj = g->xadj;
+  a->adjncy = g->adjncy;
+  a->weight = g->weight;
+  a->label = g->label;
+  a->V = g->V;
+  a->max_depth = p->max_depth;
+  a->hub_threshold = p->hub_threshold;
+  a->seed_lo = (uint32_t)p->seed;
+  a->seed_hi = (uint32_t)(p->seed >> 32);
+  a->walker_base = p->walker_base;
+  a->tp = p->tp;
+  a->inv_p = 1.0f / p->p;
+  a->inv_q = 1.0f / p->q;
+  a->schema_len = p->schema_len;
+  for (int i = 0; i < FW_MAX_SCHEMA; ++i) a->schema[i] = (i < p->schema_len) ? p->schema[i] : 0;
+}
+
+struct Scratch {  // dispenser word + two 64-bit counters, 32 bytes per launch slot
+  uint32_t dispenser;
+  uint32_t pad;
+  unsigned long long counters[2];
+  unsigned long long pad2;
+};
+
+static double now_ms() {
+  using clk = std::chrono::steady_clock;
+  return std::chrono::duration<double, std::milli>(clk::now().time_since_epoch()).count();
+}
+
+extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const int32_t* d_starts, int32_t n,
+                              int32_t* d_paths, void* stream_v, fw_walk_stats* stats) {
+  int rc = check_walk_args(g, p, d_starts, n, d_paths);
+  if (rc != FW_OK) return rc;
+  hipStream_t stream = reinterpret_cast<hipStream_t>(stream_v);
+  const double t0 = now_ms();
+
+  Scratch* d_scr = nullptr;
+  FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_scr), sizeof(Scratch)));
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  auto cleanup = [&]() {
+    if (ev0) (void)hipEventDestroy(ev0);
+    if (ev1) (void)hipEventDestroy(ev1);
+    if (d_scr) (void)hipFree(d_scr);
+  };
+#define FW_TRY(call)                                                 \
+  do {                                                               \
+    int rc_ = fw_check_hip((call), #call, __FILE__, __LINE__);       \
+    if (rc_ != FW_OK) { cleanup(); return rc_; }                     \
+  } while (0)
+  FW_TRY(hipEventCreate(&ev0));
+  FW_TRY(hipEventCreate(&ev1));
+  FW_TRY(hipMemsetAsync(d_scr, 0, sizeof(Scratch), stream));
+  // -1 fill of the path matrix: src/walk.cu:398, :536
+  FW_TRY(hipMemsetAsync(d_paths, 0xFF, (size_t)n * (size_t)p->max_depth * sizeof(int32_t), stream));
+
+  fw_kargs a;
+  fill_kargs(&a, g, p);
+  a.starts = d_starts;
+  a.paths = d_paths;
+  a.n = n;
+  a.dispenser = &d_scr->dispenser;
+  a.counters = d_scr->counters;
+  int grid_used = 0;
+  FW_TRY(hipEventRecord(ev0, stream));
+  rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, &grid_used);
+  if (rc != FW_OK) { cleanup(); return rc; }
+  FW_TRY(hipEventRecord(ev1, stream));
+  FW_TRY(hipStreamSynchronize(stream));
+  float ms = 0.0f;
+  FW_TRY(hipEventElapsedTime(&ms, ev0, ev1));
+  Scratch h;
+  FW_TRY(hipMemcpy(&h, d_scr, sizeof(h), hipMemcpyDeviceToHost));
+  cleanup();
+  if (stats) {
+    stats->kernel_ms = ms;
+    stats->total_ms = now_ms() - t0;
+    stats->steps = h.counters[0];
+    stats->sampled_edges = h.counters[1];
+    stats->launches = 1;
+    stats->grid = grid_used;
+  }
+  return FW_OK;
+}
+
+extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const int32_t* h_starts, int32_t n,
+                             uint32_t batch_size, int sync, int32_t* h_paths, fw_walk_stats* stats) {
+  int rc = check_walk_args(g, p, h_starts, n, h_paths);
+  if (rc != FW_OK) return rc;
+  if (batch_size == 0) {  // autobatch, src/main.cu:259-271 with the default 512 MB headroom
+    size_t free_b = 0, total_b = 0;
+    rc = fw_device_mem_info(&free_b, &total_b);
+    if (rc != FW_OK) return rc;
+    batch_size = fw_autobatch_size(free_b, 512, p->max_depth, sync, (uint32_t)n);
+    if (batch_size == 0) { fw_set_error("autobatch: not enough free device memory"); return FW_ERR_NOMEM; }
+  }
+  if (batch_size > (uint32_t)n) batch_size = (uint32_t)n;
+  const int nbuf = sync ? 1 : 2;
+  const size_t bs = batch_size;
+  const size_t md = (size_t)p->max_depth;
+
+  int32_t* d_starts = nullptr;
+  int32_t* d_paths = nullptr;
+  Scratch* d_scr = nullptr;
+  hipStream_t streams[2] = {nullptr, nullptr};
+  std::vector<hipEvent_t> events;
+  auto cleanup = [&]() {
+    for (hipEvent_t e : events) (void)hipEventDestroy(e);
+    for (int i = 0; i < 2; ++i) if (streams[i]) (void)hipStreamDestroy(streams[i]);
+    if (d_starts) (void)hipFree(d_starts);
+    if (d_paths) (void)hipFree(d_paths);
+    if (d_scr) (void)hipFree(d_scr);
+  };
+  FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_starts), bs * nbuf * sizeof(int32_t)));
+  FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_paths), bs * nbuf * md * sizeof(int32_t)));
+  const int nbatch = (int)(((size_t)n + bs - 1) / bs);
+  FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_scr), sizeof(Scratch) * (size_t)nbatch));
+  FW_TRY(hipMemset(d_scr, 0, sizeof(Scratch) * (size_t)nbatch));
+  for (int i = 0; i < nbuf; ++i) FW_TRY(hipStreamCreate(&streams[i]));
+  events.resize((size_t)nbatch * 2, nullptr);
+  for (auto& e : events) FW_TRY(hipEventCreate(&e));
+
+  fw_kargs a;
+  fill_kargs(&a, g, p);
+  int grid_used = 0;
+  const double t0 = now_ms();
+  for (int b = 0; b < nbatch; ++b) {
+    const int s = b % nbuf;
+    const size_t first = (size_t)b * bs;
+    const int32_t cnt = (int32_t)(((size_t)n - first) < bs ? ((size_t)n - first) : bs);
+    int32_t* ds = d_starts + (size_t)s * bs;
+    int32_t* dp = d_paths + (size_t)s * bs * md;
+    FW_TRY(hipMemcpyAsync(ds, h_starts + first, (size_t)cnt * sizeof(int32_t), hipMemcpyHostToDevice, streams[s]));
+    FW_TRY(hipMemsetAsync(dp, 0xFF, (size_t)cnt * md * sizeof(int32_t), streams[s]));
+    a.starts = ds;
+    a.paths = dp;
+    a.n = cnt;
+    a.walker_base = p->walker_base + (uint32_t)first;
+    a.dispenser = &d_scr[b].dispenser;
+    a.counters = d_scr[b].counters;
+    FW_TRY(hipEventRecord(events[2 * b], streams[s]));
+    rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, streams[s], &grid_used);
+    if (rc != FW_OK) { cleanup(); return rc; }
+    FW_TRY(hipEventRecord(events[2 * b + 1], streams[s]));
+    FW_TRY(hipMemcpyAsync(h_paths + first * md, dp, (size_t)cnt * md * sizeof(int32_t), hipMemcpyDeviceToHost, streams[s]));
+    if (sync) FW_TRY(hipStreamSynchronize(streams[s]));
+  }
+  for (int i = 0; i < nbuf; ++i) FW_TRY(hipStreamSynchronize(streams[i]));
+  const double total = now_ms() - t0;
+
+  double kernel_ms = 0.0;
+  for (int b = 0; b < nbatch; ++b) {
+    float ms = 0.0f;
+    FW_TRY(hipEventElapsedTime(&ms, events[2 * b], events[2 * b + 1]));
+    kernel_ms += ms;
+  }
+  std::vector<Scratch> h((size_t)nbatch);
+  FW_TRY(hipMemcpy(h.data(), d_scr, sizeof(Scratch) * (size_t)nbatch, hipMemcpyDeviceToHost));
+  cleanup();
+  if (stats) {
+    stats->kernel_ms = kernel_ms;
+    stats->total_ms = total;
+    stats->steps = 0;
+    stats->sampled_edges = 0;
+    for (const Scratch& s : h) { stats->steps += s.counters[0]; stats->sampled_edges += s.counters[1]; }
+    stats->launches = nbatch;
+    stats->grid = grid_used;
+  }
+  return FW_OK;
+}
+#undef FW_TRY

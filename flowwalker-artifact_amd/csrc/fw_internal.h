@@ -1,0 +1,59 @@
+// Internal declarations shared by the translation units of libflowwalker_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "flowwalker.h"
+
+// Device CSR mirror (include/gpu_graph.cuh:28-36 in the reference).  Edge arrays are allocated with
+// FW_EDGE_PAD extra elements so that aligned 16-byte loads of the last quartet stay in bounds.
+struct fw_graph {
+  int32_t V = 0;
+  uint64_t E = 0;
+  uint32_t* xadj = nullptr;
+  int32_t* adjncy = nullptr;
+  float* weight = nullptr;
+  int32_t* label = nullptr;
+  int owns = 1;
+  int device = 0;
+  int32_t max_degree = -1;  // lazily computed
+  int32_t max_degree_vertex = -1;
+  int sorted = -1;          // lazily computed
+};
+
+constexpr int FW_EDGE_PAD = 4;
+
+// Arguments of one walk-kernel launch.
+struct fw_kargs {
+  const uint32_t* xadj;
+  const int32_t* adjncy;
+  const float* weight;
+  const int32_t* label;
+  const int32_t* starts;
+  int32_t* paths;
+  uint32_t* dispenser;          // one zeroed word per launch: the global query dispenser
+  unsigned long long* counters; // [0] steps, [1] sum of source degrees
+  int32_t V;
+  int32_t n;
+  int32_t max_depth;
+  int32_t hub_threshold;
+  uint32_t seed_lo, seed_hi;
+  uint32_t walker_base;
+  float tp, inv_p, inv_q;
+  int32_t schema_len;
+  int32_t schema[FW_MAX_SCHEMA];
+};
+
+void fw_set_error(const char* fmt, ...);
+int fw_check_hip(hipError_t e, const char* what, const char* file, int line);
+#define FW_HIP(call)                                                  \
+  do {                                                                \
+    int fw_rc_ = fw_check_hip((call), #call, __FILE__, __LINE__);     \
+    if (fw_rc_ != FW_OK) return fw_rc_;                               \
+  } while (0)
+
+// Launches the walk kernel for (app, sampler, wg_threads) on `stream`.  grid = 0: fill the device.
+// Returns the grid used through *grid_used.
+int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, hipStream_t stream,
+                   int* grid_used);

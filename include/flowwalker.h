@@ -1,0 +1,187 @@
+/*
+ * flowwalker.h -- C ABI of libflowwalker_hip.so, the MI355X (gfx950) walk engine.
+ *
+ * The reference (junyimei/flowwalker-artifact) has no FFI; its seam is the pair of in-process host
+ * entry points walk_test / walk_batch (include/walker.cuh:49-57) that src/main.cu:346-357 calls
+ * with a device graph (include/gpu_graph.cuh:28-78) and gflags globals for the application
+ * parameters (src/walk.cu:36-44).  Every function below names the reference interface it replaces.
+ *
+ * Conventions: plain pointers and sizes; every function returns an fw_status (0 = ok) and never
+ * calls exit(); fw_last_error() describes the last failure on the calling thread.  "d_" pointers
+ * are device memory of the current HIP device, "h_" pointers are host memory.  Output buffers are
+ * caller-owned (the reference allocates result_pool inside the callee and never frees it:
+ * src/walk.cu:536, :586).
+ */
+#ifndef FLOWWALKER_H_
+#define FLOWWALKER_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FW_MAX_SCHEMA 64
+#define FW_WAVE 64
+
+typedef enum {
+  FW_OK = 0,
+  FW_ERR_INVALID = 1,   /* bad argument (message says which) */
+  FW_ERR_HIP = 2,       /* a HIP runtime call failed */
+  FW_ERR_NO_DEVICE = 3, /* no gfx950 device visible */
+  FW_ERR_IO = 4,        /* file missing / short / inconsistent */
+  FW_ERR_NOMEM = 5
+} fw_status;
+
+/* Application selector: --deepwalk / --ppr / --node2vec / --metapath (src/main.cu:50-53);
+ * functors of include/app.cuh:58-152. */
+typedef enum { FW_APP_DEEPWALK = 0, FW_APP_PPR = 1, FW_APP_NODE2VEC = 2, FW_APP_METAPATH = 3 } fw_app;
+
+/* Sampler selector: ZPRS kernel (include/walker.cuh:1307) or DPRS kernel (:1444, --dprs). */
+typedef enum { FW_SAMPLER_ZPRS = 0, FW_SAMPLER_DPRS = 1 } fw_sampler;
+
+/*
+ * Walk parameters.  Replaces the gflags globals read by src/walk.cu:36-44 (FLAGS_tp, FLAGS_p,
+ * FLAGS_q, app booleans) and the schema / schema_len / max_depth arguments of walk_test /
+ * walk_batch.  Fill with fw_walk_params_default() and override.
+ */
+typedef struct {
+  int32_t app;           /* fw_app */
+  int32_t sampler;       /* fw_sampler */
+  int32_t max_depth;     /* path row length = --d + 1 (src/main.cu:342) */
+  int32_t wg_threads;    /* lanes of the workgroup sampler: 256, 512 or 1024 */
+  int32_t hub_threshold; /* degree > hub_threshold uses the workgroup sampler (THRESHOLD, include/walker.cuh:29) */
+  int32_t schema_len;    /* metapath: number of labels in the schema (src/main.cu:226-242) */
+  int32_t schema[FW_MAX_SCHEMA];
+  float tp;              /* PPR termination probability (--tp) */
+  float p;               /* node2vec return parameter (--p) */
+  float q;               /* node2vec in-out parameter (--q) */
+  uint32_t walker_base;  /* global walker id of query 0: keys the RNG, so batches do not repeat streams */
+  uint64_t seed;         /* RNG seed (the reference hard-codes 1337: include/walker.cuh:1324) */
+  int32_t grid;          /* workgroups to launch; 0 = library default (src/walk.cu:84-92 analogue) */
+  int32_t reserved;
+} fw_walk_params;
+
+/* What src/main.cu:82-113 (calculate_workload) and the timing code of src/walk.cu report. */
+typedef struct {
+  double kernel_ms;       /* sum of walk-kernel durations (HIP events on the launch stream) */
+  double total_ms;        /* wall time of the call, transfers included (src/walk.cu:388,459,465) */
+  uint64_t steps;         /* "Total sampled vertex" */
+  uint64_t sampled_edges; /* "Total sampled edge": sum over steps of deg(source) */
+  int32_t launches;       /* kernel launches (= batches) */
+  int32_t grid;           /* workgroups per launch actually used */
+} fw_walk_stats;
+
+typedef struct fw_graph fw_graph; /* device CSR mirror: include/gpu_graph.cuh:28-78 */
+
+/* ---- library ---------------------------------------------------------------------------------- */
+
+/* Thread-local text of the last error; replaces the print-and-exit of CUDA_RT_CALL (include/util.cuh:56-68). */
+const char* fw_last_error(void);
+
+/* Number of usable devices (0 when there is no GPU); never fails. */
+int fw_device_count(void);
+
+/* Free / total device memory in bytes: get_avail_mem (src/util.cu:50-65). */
+int fw_device_mem_info(size_t* free_bytes, size_t* total_bytes);
+
+/* Fills defaults: app DeepWalk, d = 80, tp 0.2, p 2.0, q 0.5, schema 0,1,2,3,4, seed 1337 (src/main.cu:40-80). */
+void fw_walk_params_default(fw_walk_params* p);
+
+/*
+ * Autobatch rule of adjust_flags (src/main.cu:259-271):
+ *   bs = min((free - headroom_mb * 2^20) / (4 * (d + 2)), INT_MAX); halved unless sync; min(bs, n_queries).
+ * d = max_depth - 1.  Returns 0 on invalid input (free <= headroom).
+ */
+uint32_t fw_autobatch_size(size_t free_bytes, int32_t headroom_mb, int32_t max_depth, int sync, uint32_t n_queries);
+
+/* ---- device buffers (so hosts without a HIP binding can keep inputs resident) ------------------ */
+
+int fw_dev_alloc(size_t bytes, void** d_ptr);
+int fw_dev_free(void* d_ptr);
+int fw_dev_upload(void* d_dst, const void* h_src, size_t bytes);
+int fw_dev_download(void* h_dst, const void* d_src, size_t bytes);
+int fw_dev_fill_i32(int32_t* d_dst, int32_t value, size_t count);
+int fw_dev_sync(void);
+
+/* ---- graph ------------------------------------------------------------------------------------ */
+
+/*
+ * Uploads a host CSR: replaces gpu_graph::gpu_graph(graph*) (include/gpu_graph.cuh:39-78).
+ * xadj: uint32[V+1], xadj[0] = 0, xadj[V] = E; adjncy: int32[E]; weight: float32[E] or NULL;
+ * label: int32[E] or NULL (the reference uploads weights XOR labels, :50-76; here both may be given).
+ * Weights must be finite and >= 0 (checked).  Fails with FW_ERR_INVALID on inconsistent input.
+ */
+int fw_graph_create(int32_t V, uint64_t E, const uint32_t* h_xadj, const int32_t* h_adjncy,
+                    const float* h_weight, const int32_t* h_label, fw_graph** out);
+
+/*
+ * Adopts device arrays that already hold a CSR (e.g. produced by fw_gen_rmat).  The arrays must
+ * stay valid until fw_graph_destroy and must be readable 12 bytes past their last element
+ * (the kernels use aligned 16-byte loads).  take_ownership != 0: destroy frees them with hipFree.
+ */
+int fw_graph_adopt_device(int32_t V, uint64_t E, uint32_t* d_xadj, int32_t* d_adjncy, float* d_weight,
+                          int32_t* d_label, int take_ownership, fw_graph** out);
+
+int fw_graph_destroy(fw_graph* g);
+
+/* V, E and the maximum degree / its vertex (graph::print_max_degree, include/graph.cuh:209-220). */
+int fw_graph_info(const fw_graph* g, int32_t* V, uint64_t* E, int32_t* max_degree, int32_t* max_degree_vertex);
+
+/* 1 when every neighbour list is strictly ascending (needed by node2vec: include/gpu_graph.cuh:97-118). */
+int fw_graph_is_sorted(const fw_graph* g, int* sorted);
+
+/* Copies the device CSR back (any output pointer may be NULL). */
+int fw_graph_download(const fw_graph* g, uint32_t* h_xadj, int32_t* h_adjncy, float* h_weight, int32_t* h_label);
+
+/* ---- walks ------------------------------------------------------------------------------------ */
+
+/*
+ * One kernel launch over device-resident queries: replaces walk_test + timing<App>() for
+ * walk_mode wb_dynamic (src/walk.cu:527-574, :222-248), i.e. kernels walker_wb_dynamic_zprs /
+ * _dprs (include/walker.cuh:1307, :1444).
+ * d_starts: int32[n]; d_paths: int32[n][max_depth], written completely (-1 padded; the caller does
+ * not have to pre-fill it, unlike src/walk.cu:536).  stream: hipStream_t or NULL.  Synchronous:
+ * returns after the kernel has finished; stats may be NULL.
+ */
+int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const int32_t* d_starts, int32_t n,
+                   int32_t* d_paths, void* stream, fw_walk_stats* stats);
+
+/*
+ * Batched walk over host queries: replaces walk_batch (src/walk.cu:576-649) with
+ * timing_batch_async (two streams, double-buffered H2D / kernel / D2H, :373-466) or, when
+ * sync != 0, timing_batch_sync (:468-523).  h_starts: int32[n]; h_paths: int32[n][max_depth],
+ * caller-owned (pinned memory gives overlap, pageable works).  batch_size = 0: autobatch.
+ * Walker ids are walker_base + query index, whatever the batch size.
+ */
+int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const int32_t* h_starts, int32_t n,
+                  uint32_t batch_size, int sync, int32_t* h_paths, fw_walk_stats* stats);
+
+/* Pinned host memory for start points / paths: cudaMallocHost in src/main.cu:275, src/walk.cu:586. */
+int fw_host_alloc_pinned(size_t bytes, void** h_ptr);
+int fw_host_free_pinned(void* h_ptr);
+
+/* ---- synthetic graphs (the build's own generator; output format of data/EdgeListToCSR.cpp:216-251) */
+
+typedef struct {
+  int32_t scale;        /* V = 2^scale */
+  int32_t edge_factor;  /* generated edges = edge_factor * V (before dedupe) */
+  float a, b, c;        /* R-MAT quadrant probabilities; d = 1 - a - b - c.  a = b = c = 0.25: uniform */
+  int32_t symmetrise;   /* insert both directions */
+  float w_lo, w_hi;     /* weights uniform in [w_lo, w_hi), equal on both directions */
+  int32_t n_labels;     /* labels uniform in [0, n_labels); 0 = no labels */
+  int32_t make_weights; /* 0 = no weights */
+  uint64_t seed;
+} fw_rmat_params;
+
+/*
+ * Generates a deduplicated, self-loop-free R-MAT CSR with ascending neighbour lists directly in
+ * device memory.  Deterministic in (params).  The CSR has V = 2^scale vertices (isolated vertices kept).
+ */
+int fw_gen_rmat(const fw_rmat_params* rp, fw_graph** out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLOWWALKER_H_ */

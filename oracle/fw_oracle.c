@@ -1,0 +1,448 @@
+/*
+ * fw_oracle.c -- CPU oracle for the FlowWalker walk path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file is the checker, not the product: only tests/, __graft_entry__.smoke() and the
+ * cpu_baseline leg of bench.py may build, load or call it.  The shipped library never links it
+ * and has no CPU fallback.
+ *
+ * It restates, in plain C, the algorithm of the reference's sampler-centric walk engine and fixes
+ * every detail the reference leaves to thread scheduling, so that the HIP kernels can be compared
+ * bit for bit.  The reference itself cannot be built here (CUDA + CUB + cuRAND + gflags) and is not
+ * a bitwise oracle anyway: its RNG streams belong to threads and its query->slot assignment is an
+ * atomic race (include/walker.cuh:1323-1324, :1339).
+ *
+ * What follows the reference, and where:
+ *   - walk control flow (start write, step commit, dead end, stop, -1 padded rows):
+ *       include/walker.cuh:1338-1350, :1357-1438; include/gpu_task.cuh:52-77
+ *   - sampler: weighted reservoir sampling whose winner is "the last accepted element in
+ *       lane-major order" over lane-strided elements, lane totals combined with a prefix scan and
+ *       a max over accepted lanes: include/sampler.cuh:46-85 (warp), :87-127 (block);
+ *       sequential ground truth include/sampler.cuh:26-44
+ *   - DPRS (natural order, chunked inclusive scan, one Bernoulli per element):
+ *       include/sampler.cuh:129-155, :157-200
+ *   - bias functors and stop rules: include/app.cuh:58-71 (DeepWalk), :73-95 (PPR),
+ *       :97-127 (node2vec), :129-152 (MetaPath); adjacency test include/gpu_graph.cuh:97-118
+ *   - workload counters (steps, sum of source degrees): src/main.cu:82-113
+ *
+ * What this build defines differently from the reference (documented, deliberate):
+ *   - RNG: Philox4x32-10 (Salmon et al., SC'11), keyed by the 64-bit seed, counter =
+ *       (walker id, step, stream, block).  Replaces the stateful XORWOW of include/myrand.cuh.
+ *       Pinned by the Random123 known-answer vectors (tests/golden/philox4x32_10_kat.json).
+ *   - ZPRS is one pass: every lane runs a sequential reservoir over its own elements starting
+ *       from 0 (not from the exclusive lane prefix), and lanes are then combined by one Bernoulli
+ *       per lane against the inclusive lane prefix.  The law of the winner is unchanged
+ *       (w_i / sum w); the second pass over the weights of include/sampler.cuh:70-80 disappears.
+ *   - acceptance inside a lane uses the telescoping identity
+ *       P(no accept in (j,k]) = prod S_{i-1}/S_i = S_j/S_k,
+ *       so one uniform u decides the NEXT accepted element (first k with S_k*u > S_j) instead of one
+ *       uniform per element.  Same law as include/sampler.cuh:76, O(log n) draws per lane.
+ *   - no division anywhere: tests are u*S < w-shaped products, never FMA-contracted.
+ *   - uniforms are (x >> 8) * 2^-24 in [0,1), exact in f32.
+ *   - elements are grouped in 4-element quartets aligned to the absolute CSR index (16-byte
+ *       aligned vector loads on the GPU); quartet k of a list belongs to lane k mod P.
+ *   - PPR stop draw is made once per completed step of a live walk, from its own stream
+ *       (the reference also draws for empty slots, include/walker.cuh:1422-1431).
+ *   - node2vec multiplies by host-computed f32 reciprocals 1/p and 1/q instead of dividing.
+ *
+ * Build: make -C oracle   (gcc -O2 -ffp-contract=off -fopenmp)
+ */
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define FW_WAVE 64
+#define FW_QUAD 4
+#define FW_MAX_SCHEMA 64
+#define FW_MAX_GROUP 1024
+
+enum { FW_APP_DEEPWALK = 0, FW_APP_PPR = 1, FW_APP_NODE2VEC = 2, FW_APP_METAPATH = 3 };
+enum { FW_SAMPLER_ZPRS = 0, FW_SAMPLER_DPRS = 1 };
+
+#define FW_STREAM_WAVE 0x40000000u /* | wave index : workgroup-level combine draws */
+#define FW_STREAM_STOP 0x80000000u /* PPR stop draw */
+#define FW_STREAM_DPRS 0xC0000000u /* DPRS: block index carries the element quartet */
+
+typedef struct {
+  int32_t app;           /* FW_APP_* */
+  int32_t sampler;       /* FW_SAMPLER_* */
+  int32_t max_depth;     /* path row length = steps + 1 */
+  int32_t wg_threads;    /* lanes of the workgroup sampler (multiple of 64, <= 1024) */
+  int32_t hub_threshold; /* degree > hub_threshold -> workgroup sampler */
+  int32_t schema_len;
+  int32_t schema[FW_MAX_SCHEMA];
+  float tp;
+  float inv_p;
+  float inv_q;
+  uint32_t walker_base; /* global walker id of query 0 */
+  uint64_t seed;
+} fw_oracle_params;
+
+typedef struct {
+  int32_t V;
+  const uint32_t* xadj;
+  const int32_t* adjncy;
+  const float* weight;  /* NULL for metapath */
+  const int32_t* label; /* NULL unless metapath */
+} fw_oracle_graph;
+
+/* ---- Philox4x32-10 ------------------------------------------------------------------------ */
+
+void fw_oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+  uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3];
+  uint32_t k0 = key[0], k1 = key[1];
+  for (int r = 0; r < 10; ++r) {
+    uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    uint32_t n1 = (uint32_t)p1;
+    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    uint32_t n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+/* n-th 32-bit draw of stream `stream` at (walker, step): word n&3 of Philox block n>>2. */
+static uint32_t draw_bits(uint64_t seed, uint32_t walker, uint32_t step, uint32_t stream, uint32_t n) {
+  uint32_t ctr[4] = {walker, step, stream, n >> 2};
+  uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  uint32_t out[4];
+  fw_oracle_philox4x32_10(ctr, key, out);
+  return out[n & 3];
+}
+
+static float u24(uint32_t bits) { return (float)(bits >> 8) * 0x1p-24f; }
+
+float fw_oracle_uniform(uint64_t seed, uint32_t walker, uint32_t step, uint32_t stream, uint32_t n) {
+  return u24(draw_bits(seed, walker, step, stream, n));
+}
+
+/* ---- scan trees (mirror of the wave64 DPP scan: row_shr 1,2,4,8; row_bcast15; row_bcast31) - */
+
+/* In-place inclusive scan of 64 floats with the exact association order of the GPU wave scan. */
+void fw_oracle_wave_scan(float x[FW_WAVE]) {
+  float t[FW_WAVE];
+  for (int off = 1; off < 16; off <<= 1) {
+    for (int l = 0; l < FW_WAVE; ++l) t[l] = ((l & 15) >= off) ? x[l] + x[l - off] : x[l];
+    memcpy(x, t, sizeof(t));
+  }
+  /* row_bcast:15, rows 1 and 3 */
+  {
+    float r0 = x[15], r2 = x[47];
+    for (int l = 16; l < 32; ++l) x[l] = x[l] + r0;
+    for (int l = 48; l < 64; ++l) x[l] = x[l] + r2;
+  }
+  /* row_bcast:31, rows 2 and 3 */
+  {
+    float h = x[31];
+    for (int l = 32; l < 64; ++l) x[l] = x[l] + h;
+  }
+}
+
+/* Inclusive scan of m <= 16 floats: one DPP row (row_shr 1,2,4,8). */
+static void row_scan(float* x, int m) {
+  float t[16];
+  for (int off = 1; off < 16; off <<= 1) {
+    for (int l = 0; l < m; ++l) t[l] = (l >= off) ? x[l] + x[l - off] : x[l];
+    memcpy(x, t, sizeof(float) * m);
+  }
+}
+
+/* ---- bias functors (include/app.cuh) -------------------------------------------------------- */
+
+typedef struct {
+  const fw_oracle_graph* g;
+  const fw_oracle_params* p;
+  int32_t prev;       /* -1 on the first step */
+  uint32_t prev_off;  /* CSR range of prev (node2vec) */
+  int32_t prev_deg;
+  int32_t want_label; /* metapath: schema[step % schema_len] */
+} bias_ctx;
+
+/* include/gpu_graph.cuh:97-112 */
+static int sorted_contains(const int32_t* arr, int32_t size, int32_t target) {
+  int32_t l = 0, r = size - 1;
+  while (l <= r) {
+    int32_t m = l + (r - l) / 2;
+    if (arr[m] == target) return 1;
+    if (arr[m] < target) l = m + 1; else r = m - 1;
+  }
+  return 0;
+}
+
+/* Bias of CSR entry `a` (absolute index).  include/app.cuh:64-66, :86-88, :108-123, :141-146. */
+static float bias_at(const bias_ctx* c, uint64_t a) {
+  switch (c->p->app) {
+    case FW_APP_METAPATH:
+      return c->g->label[a] == c->want_label ? 1.0f : 0.0f;
+    case FW_APP_NODE2VEC: {
+      float w = c->g->weight[a];
+      if (c->prev == -1) return w;
+      int32_t post = c->g->adjncy[a];
+      if (post == c->prev) return w * c->p->inv_p;
+      if (!sorted_contains(c->g->adjncy + c->prev_off, c->prev_deg, post)) return w * c->p->inv_q;
+      return w;
+    }
+    default:
+      return c->g->weight[a];
+  }
+}
+
+/* ---- ZPRS: one-pass zero-preprocessing parallel reservoir sampler ---------------------------- */
+
+/*
+ * Samples one local index in [0,deg) with probability bias_i / sum(bias), or -1 when no bias is
+ * positive.  P lanes (64 = wave, wg_threads = workgroup).  Follows the lane-strided / prefix /
+ * max structure of include/sampler.cuh:46-127 with the one-pass and jump changes listed on top.
+ */
+static int32_t zprs_sample(const bias_ctx* c, uint32_t off, int32_t deg, int P, uint32_t walker,
+                           uint32_t step) {
+  if (deg <= 0) return -1;
+  const uint64_t seed = c->p->seed;
+  const uint64_t a0 = (uint64_t)off & ~(uint64_t)(FW_QUAD - 1);
+  const uint64_t end = (uint64_t)off + (uint64_t)deg;
+  const uint64_t nq = (end - a0 + FW_QUAD - 1) / FW_QUAD;
+
+  float L[FW_MAX_GROUP];
+  int32_t sel[FW_MAX_GROUP];
+
+  for (int t = 0; t < P; ++t) {
+    float S = 0.0f, Sj = 0.0f, u = 1.0f;
+    int32_t s = -1;
+    uint32_t ndraw = 0;
+    for (uint64_t k = (uint64_t)t; k < nq; k += (uint64_t)P) {
+      for (int j = 0; j < FW_QUAD; ++j) {
+        uint64_t a = a0 + FW_QUAD * k + j;
+        if (a < off || a >= end) continue;
+        float w = bias_at(c, a);
+        S = S + w;
+        float lhs = S * u;
+        if (lhs > Sj) {
+          s = (int32_t)(a - off);
+          Sj = S;
+          u = u24(draw_bits(seed, walker, step, (uint32_t)t, 1u + ndraw));
+          ++ndraw;
+        }
+      }
+    }
+    L[t] = S;
+    sel[t] = s;
+  }
+
+  const int nw = P / FW_WAVE;
+  float W[16];
+  int32_t wsel[16];
+  for (int wv = 0; wv < nw; ++wv) {
+    float I[FW_WAVE];
+    for (int l = 0; l < FW_WAVE; ++l) I[l] = L[wv * FW_WAVE + l];
+    fw_oracle_wave_scan(I);
+    int32_t pick = -1;
+    for (int l = 0; l < FW_WAVE; ++l) {
+      int t = wv * FW_WAVE + l;
+      if (L[t] > 0.0f) {
+        float ub = u24(draw_bits(seed, walker, step, (uint32_t)t, 0u));
+        float lhs = ub * I[l];
+        if (lhs < L[t]) pick = sel[t];
+      }
+    }
+    W[wv] = I[FW_WAVE - 1];
+    wsel[wv] = pick;
+  }
+  if (nw == 1) return wsel[0];
+
+  float J[16];
+  for (int wv = 0; wv < nw; ++wv) J[wv] = W[wv];
+  row_scan(J, nw);
+  int32_t pick = -1;
+  for (int wv = 0; wv < nw; ++wv) {
+    if (W[wv] > 0.0f) {
+      float ub = u24(draw_bits(seed, walker, step, FW_STREAM_WAVE | (uint32_t)wv, 0u));
+      float lhs = ub * J[wv];
+      if (lhs < W[wv]) pick = wsel[wv];
+    }
+  }
+  return pick;
+}
+
+/* ---- DPRS: natural order, chunked inclusive scan, one Bernoulli per element ------------------ */
+
+/*
+ * include/sampler.cuh:129-200.  Chunks of P*4 elements (one quartet per lane), running sum carried
+ * between chunks; element i is accepted iff bias_i > 0 and u_i * S_i < bias_i; the winner is the
+ * largest accepted index.  u_i is word (a & 3) of Philox block (a - a0) / 4 of stream FW_STREAM_DPRS.
+ * Within a chunk: lane-local 4-element running sums, wave scan of lane totals, row scan of wave
+ * totals, then S_i = carry + (waves before) + (lanes before) + local running sum.
+ */
+static int32_t dprs_sample(const bias_ctx* c, uint32_t off, int32_t deg, int P, uint32_t walker,
+                           uint32_t step) {
+  if (deg <= 0) return -1;
+  const uint64_t seed = c->p->seed;
+  const uint64_t a0 = (uint64_t)off & ~(uint64_t)(FW_QUAD - 1);
+  const uint64_t end = (uint64_t)off + (uint64_t)deg;
+  const uint64_t nq = (end - a0 + FW_QUAD - 1) / FW_QUAD;
+  const int nw = P / FW_WAVE;
+  float carry = 0.0f;
+  int32_t pick = -1;
+  for (uint64_t base = 0; base < nq; base += (uint64_t)P) {
+    float w[FW_MAX_GROUP][FW_QUAD];
+    float lane_tot[FW_MAX_GROUP];
+    for (int t = 0; t < P; ++t) {
+      uint64_t k = base + (uint64_t)t;
+      float s = 0.0f;
+      for (int j = 0; j < FW_QUAD; ++j) {
+        uint64_t a = a0 + FW_QUAD * k + j;
+        float x = (k < nq && a >= off && a < end) ? bias_at(c, a) : 0.0f;
+        w[t][j] = x;
+        s = s + x;
+      }
+      lane_tot[t] = s;
+    }
+    float wave_tot[16];
+    float incl[FW_MAX_GROUP];
+    for (int wv = 0; wv < nw; ++wv) {
+      float I[FW_WAVE];
+      for (int l = 0; l < FW_WAVE; ++l) I[l] = lane_tot[wv * FW_WAVE + l];
+      fw_oracle_wave_scan(I);
+      for (int l = 0; l < FW_WAVE; ++l) incl[wv * FW_WAVE + l] = I[l];
+      wave_tot[wv] = I[FW_WAVE - 1];
+    }
+    float J[16];
+    for (int wv = 0; wv < nw; ++wv) J[wv] = wave_tot[wv];
+    if (nw > 1) row_scan(J, nw);
+    for (int t = 0; t < P; ++t) {
+      uint64_t k = base + (uint64_t)t;
+      if (k >= nq) break;
+      int wv = t / FW_WAVE, l = t % FW_WAVE;
+      /* exclusive prefix of this lane inside the chunk */
+      float before = carry;
+      if (wv > 0) before = before + J[wv - 1];
+      if (l > 0) before = before + incl[t - 1];
+      uint32_t ctr[4] = {walker, step, FW_STREAM_DPRS, (uint32_t)k};
+      uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+      uint32_t r[4];
+      fw_oracle_philox4x32_10(ctr, key, r);
+      float S = before;
+      for (int j = 0; j < FW_QUAD; ++j) {
+        uint64_t a = a0 + FW_QUAD * k + j;
+        float x = w[t][j];
+        S = S + x;
+        if (x > 0.0f) {
+          float lhs = u24(r[j]) * S;
+          if (lhs < x) {
+            int32_t i = (int32_t)(a - off);
+            if (i > pick) pick = i;
+          }
+        }
+      }
+    }
+    carry = carry + J[nw > 1 ? nw - 1 : 0];
+  }
+  return pick;
+}
+
+/* One sampling step, exposed for sampler-level tests.  Granularity by degree as in
+ * include/walker.cuh:1362 (degree <= threshold -> wave, else workgroup). */
+int32_t fw_oracle_sample(const fw_oracle_graph* g, const fw_oracle_params* p, int32_t cur,
+                         int32_t prev, uint32_t walker, uint32_t step) {
+  bias_ctx c;
+  c.g = g; c.p = p; c.prev = prev;
+  c.prev_off = 0; c.prev_deg = 0;
+  if (prev >= 0) { c.prev_off = g->xadj[prev]; c.prev_deg = (int32_t)(g->xadj[prev + 1] - g->xadj[prev]); }
+  c.want_label = (p->app == FW_APP_METAPATH && p->schema_len > 0) ? p->schema[step % (uint32_t)p->schema_len] : 0;
+  uint32_t off = g->xadj[cur];
+  int32_t deg = (int32_t)(g->xadj[cur + 1] - off);
+  int P = (deg > p->hub_threshold) ? p->wg_threads : FW_WAVE;
+  return p->sampler == FW_SAMPLER_DPRS ? dprs_sample(&c, off, deg, P, walker, step)
+                                       : zprs_sample(&c, off, deg, P, walker, step);
+}
+
+/* ---- whole walks (include/walker.cuh:1338-1438) --------------------------------------------- */
+
+static void walk_one(const fw_oracle_graph* g, const fw_oracle_params* p, int32_t start, uint32_t walker,
+                     int32_t* row, uint64_t* steps, uint64_t* edges) {
+  const int md = p->max_depth;
+  for (int i = 0; i < md; ++i) row[i] = -1;
+  if (md <= 0) return;
+  row[0] = start;
+  if (start < 0 || start >= g->V) return;
+  int32_t cur = start, prev = -1;
+  int len = 1;
+  while (len < md) {
+    uint32_t step = (uint32_t)(len - 1);
+    uint32_t off = g->xadj[cur];
+    int32_t deg = (int32_t)(g->xadj[cur + 1] - off);
+    int32_t s = fw_oracle_sample(g, p, cur, prev, walker, step);
+    if (s < 0) break; /* dead end: include/walker.cuh:1373-1374 */
+    int32_t v = g->adjncy[(uint64_t)off + (uint32_t)s];
+    row[len] = v;
+    *steps += 1;
+    *edges += (uint64_t)deg; /* src/main.cu:101-103 */
+    prev = cur;
+    cur = v;
+    ++len;
+    if (p->app == FW_APP_PPR) { /* include/app.cuh:88-94 */
+      float r = u24(draw_bits(p->seed, walker, step, FW_STREAM_STOP, 0u));
+      if (r < p->tp) break;
+    }
+  }
+}
+
+/*
+ * Runs n queries; paths is int32[n][max_depth], -1 padded, column 0 = start vertex
+ * (include/walker.cuh:1342, :1379-1381).  steps / edges as src/main.cu:93-104.
+ * nthreads <= 0: all cores (OpenMP schedule(dynamic) over walkers).
+ */
+int fw_oracle_walk(const fw_oracle_graph* g, const fw_oracle_params* p, const int32_t* starts, int64_t n,
+                   int32_t* paths, uint64_t* steps_out, uint64_t* edges_out, int nthreads) {
+  if (p->wg_threads % FW_WAVE != 0 || p->wg_threads > FW_MAX_GROUP || p->wg_threads < FW_WAVE) return -1;
+  if (p->app == FW_APP_METAPATH && (p->schema_len <= 0 || p->schema_len > FW_MAX_SCHEMA)) return -1;
+  uint64_t steps = 0, edges = 0;
+#ifdef _OPENMP
+  if (nthreads > 0) omp_set_num_threads(nthreads);
+#else
+  (void)nthreads;
+#endif
+#pragma omp parallel for schedule(dynamic, 64) reduction(+ : steps, edges)
+  for (int64_t q = 0; q < n; ++q) {
+    uint64_t s = 0, e = 0;
+    walk_one(g, p, starts[q], p->walker_base + (uint32_t)q, paths + (uint64_t)q * p->max_depth, &s, &e);
+    steps += s;
+    edges += e;
+  }
+  if (steps_out) *steps_out = steps;
+  if (edges_out) *edges_out = edges;
+  return 0;
+}
+
+int fw_oracle_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* ---- sequential ground truth (include/sampler.cuh:26-44), for brute-force equivalence tests -- */
+
+/*
+ * Textbook sequential weighted reservoir sampling over `n` biases in the given order with one
+ * uniform per positive element: accept i iff u_i * S_i < w_i.  Returns the last accepted index.
+ */
+int32_t fw_oracle_sequential_reservoir(const float* w, const float* u, int32_t n) {
+  float S = 0.0f;
+  int32_t pick = -1;
+  for (int32_t i = 0; i < n; ++i) {
+    S = S + w[i];
+    if (w[i] > 0.0f) {
+      float lhs = u[i] * S;
+      if (lhs < w[i]) pick = i;
+    }
+  }
+  return pick;
+}

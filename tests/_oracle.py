@@ -1,0 +1,136 @@
+"""ctypes binding of the CPU oracle (oracle/libfw_oracle.so).  Test infrastructure only."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_LIB = os.path.join(ORACLE_DIR, "libfw_oracle.so")
+
+FW_MAX_SCHEMA = 64
+STREAM_WAVE = 0x40000000
+STREAM_STOP = 0x80000000
+
+
+class OracleParams(C.Structure):
+    _fields_ = [
+        ("app", C.c_int32), ("sampler", C.c_int32), ("max_depth", C.c_int32), ("wg_threads", C.c_int32),
+        ("hub_threshold", C.c_int32), ("schema_len", C.c_int32), ("schema", C.c_int32 * FW_MAX_SCHEMA),
+        ("tp", C.c_float), ("inv_p", C.c_float), ("inv_q", C.c_float), ("walker_base", C.c_uint32),
+        ("seed", C.c_uint64),
+    ]
+
+
+class OracleGraph(C.Structure):
+    _fields_ = [("V", C.c_int32), ("xadj", C.c_void_p), ("adjncy", C.c_void_p), ("weight", C.c_void_p),
+                ("label", C.c_void_p)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(ORACLE_LIB):
+            subprocess.check_call(["make", "-C", ORACLE_DIR])
+        L = C.CDLL(ORACLE_LIB)
+        L.fw_oracle_philox4x32_10.argtypes = [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+        L.fw_oracle_philox4x32_10.restype = None
+        L.fw_oracle_uniform.argtypes = [C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32]
+        L.fw_oracle_uniform.restype = C.c_float
+        L.fw_oracle_wave_scan.argtypes = [C.c_void_p]
+        L.fw_oracle_wave_scan.restype = None
+        L.fw_oracle_sample.argtypes = [C.POINTER(OracleGraph), C.POINTER(OracleParams), C.c_int32, C.c_int32,
+                                       C.c_uint32, C.c_uint32]
+        L.fw_oracle_sample.restype = C.c_int32
+        L.fw_oracle_walk.argtypes = [C.POINTER(OracleGraph), C.POINTER(OracleParams), C.c_void_p, C.c_int64,
+                                     C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.c_int]
+        L.fw_oracle_walk.restype = C.c_int
+        L.fw_oracle_num_threads.restype = C.c_int
+        L.fw_oracle_sequential_reservoir.argtypes = [C.c_void_p, C.c_void_p, C.c_int32]
+        L.fw_oracle_sequential_reservoir.restype = C.c_int32
+        _lib = L
+    return _lib
+
+
+def philox(ctr, key):
+    c = (C.c_uint32 * 4)(*ctr)
+    k = (C.c_uint32 * 2)(*key)
+    o = (C.c_uint32 * 4)()
+    lib().fw_oracle_philox4x32_10(c, k, o)
+    return [int(x) for x in o]
+
+
+def uniform(seed, walker, step, stream, n):
+    return float(lib().fw_oracle_uniform(seed, walker, step, stream, n))
+
+
+def wave_scan(x):
+    x = np.ascontiguousarray(x, dtype=np.float32).copy()
+    assert x.shape == (64,)
+    lib().fw_oracle_wave_scan(x.ctypes.data_as(C.c_void_p))
+    return x
+
+
+class Graph:
+    """Host CSR handed to the oracle; keeps the numpy arrays alive."""
+
+    def __init__(self, xadj, adjncy, weight=None, label=None):
+        self.xadj = np.ascontiguousarray(xadj, dtype=np.uint32)
+        self.adjncy = np.ascontiguousarray(adjncy, dtype=np.int32)
+        self.weight = None if weight is None else np.ascontiguousarray(weight, dtype=np.float32)
+        self.label = None if label is None else np.ascontiguousarray(label, dtype=np.int32)
+        self.V = len(self.xadj) - 1
+        self.E = len(self.adjncy)
+        p = lambda a: None if a is None else a.ctypes.data_as(C.c_void_p)
+        self.c = OracleGraph(self.V, p(self.xadj), p(self.adjncy), p(self.weight), p(self.label))
+
+    def degree(self, v):
+        return int(self.xadj[v + 1]) - int(self.xadj[v])
+
+
+def make_params(app=0, sampler=0, max_depth=81, wg_threads=512, hub_threshold=16384, schema=(0, 1, 2, 3, 4), tp=0.2,
+                p=2.0, q=0.5, walker_base=0, seed=1337):
+    op = OracleParams()
+    op.app, op.sampler, op.max_depth = app, sampler, max_depth
+    op.wg_threads, op.hub_threshold = wg_threads, hub_threshold
+    op.schema_len = len(schema)
+    for i, s in enumerate(schema):
+        op.schema[i] = int(s)
+    op.tp = tp
+    op.inv_p = np.float32(1.0) / np.float32(p)
+    op.inv_q = np.float32(1.0) / np.float32(q)
+    op.walker_base = walker_base
+    op.seed = seed
+    return op
+
+
+def from_walk_params(wp):
+    """OracleParams mirroring a flowwalker WalkParams structure."""
+    return make_params(app=wp.app, sampler=wp.sampler, max_depth=wp.max_depth, wg_threads=wp.wg_threads,
+                       hub_threshold=wp.hub_threshold, schema=[wp.schema[i] for i in range(wp.schema_len)],
+                       tp=wp.tp, p=wp.p, q=wp.q, walker_base=wp.walker_base, seed=wp.seed)
+
+
+def sample(graph, params, cur, prev, walker, step):
+    return int(lib().fw_oracle_sample(C.byref(graph.c), C.byref(params), cur, prev, walker, step))
+
+
+def walk(graph, params, starts, nthreads=0):
+    starts = np.ascontiguousarray(starts, dtype=np.int32)
+    n = len(starts)
+    paths = np.empty((n, params.max_depth), dtype=np.int32)
+    steps, edges = C.c_uint64(), C.c_uint64()
+    rc = lib().fw_oracle_walk(C.byref(graph.c), C.byref(params), starts.ctypes.data_as(C.c_void_p), n,
+                              paths.ctypes.data_as(C.c_void_p), C.byref(steps), C.byref(edges), nthreads)
+    assert rc == 0, "oracle rejected the parameters"
+    return paths, steps.value, edges.value
+
+
+def sequential_reservoir(w, u):
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    u = np.ascontiguousarray(u, dtype=np.float32)
+    return int(lib().fw_oracle_sequential_reservoir(w.ctypes.data_as(C.c_void_p), u.ctypes.data_as(C.c_void_p), len(w)))
