@@ -1,0 +1,188 @@
+#!/usr/bin/env python3
+"""Benchmark of the walk path: one "step" = one pass of the walk kernel over the whole query batch.
+
+Default workload = the headline of BASELINE.json: DeepWalk, length 80, one query per vertex, on the
+symmetrised R-MAT scale-24 graph (edge factor 16, a/b/c/d = .57/.19/.19/.05, weights U[1,100)).
+Inputs (CSR, start vertices, path matrix) are resident in HBM before the timed region starts.
+
+Prints ONE JSON line with the walk-steps/s of the whole job, the HBM roofline of the walk kernel
+(algorithmic bytes / kernel duration measured with HIP events on the launch stream) and the CPU
+oracle timed on the host cores of the same box over a bounded prefix of the same queries.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+# name -> generator / walk settings.  Scales follow BASELINE.json's configs; "headline" is the metric's.
+WORKLOADS = {
+    "deepwalk_rmat24_sym": dict(scale=24, sym=True, app="deepwalk", depth=80, queries="all", labels=0),
+    "deepwalk_rmat22": dict(scale=22, sym=False, app="deepwalk", depth=80, queries="all", labels=0),
+    "ppr_rmat22": dict(scale=22, sym=False, app="ppr", depth=80, queries="all", labels=0),
+    "node2vec_rmat24_sym": dict(scale=24, sym=True, app="node2vec", depth=80, queries="all", labels=0),
+    "metapath_rmat26": dict(scale=26, sym=False, app="metapath", depth=5, queries=10_000_000, labels=5),
+}
+HEADLINE = "deepwalk_rmat24_sym"
+
+# HBM bytes per launch of the walk kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a
+# copy kernel of known size (see profiles/).  None until measured for that workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(app, steps, sampled_edges, queries, probe_terms=0):
+    """Bytes the algorithm has to touch: bias array once per visited neighbour + per-step and per-query words.
+
+    DeepWalk / PPR / MetaPath: 4*D + 16*S + 16*Q; node2vec: 8*D + 24*S + 16*Q (binary-search probes are
+    reported separately and not included).
+    """
+    if app == "node2vec":
+        return 8 * sampled_edges + 24 * steps + 16 * queries
+    return 4 * sampled_edges + 16 * steps + 16 * queries
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--scale", type=int, default=0, help="override the R-MAT scale (smaller boxes / quick checks)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
+    ap.add_argument("--hub-threshold", type=int, default=-1)
+    ap.add_argument("--wg-threads", type=int, default=0)
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; the walk path shards by replicating the CSR and splitting "
+                 "the queries (no collectives), and no multi-GPU figure is produced.  Run with --gpus 1.")
+
+    fw = importlib.import_module("flowwalker-artifact_amd")
+    if fw.device_count() < 1:
+        sys.exit("bench.py: no HIP device visible; the walk engine has no CPU fallback")
+
+    wl = dict(WORKLOADS[args.workload])
+    if args.scale:
+        wl["scale"] = args.scale
+    app_id = {"deepwalk": fw.APP_DEEPWALK, "ppr": fw.APP_PPR, "node2vec": fw.APP_NODE2VEC,
+              "metapath": fw.APP_METAPATH}[wl["app"]]
+
+    t0 = time.time()
+    g = fw.Graph.rmat(wl["scale"], 16, 0.57, 0.19, 0.19, symmetrise=wl["sym"], w_lo=1.0, w_hi=100.0,
+                      n_labels=wl["labels"], make_weights=wl["app"] != "metapath", seed=1)
+    fw.check(fw.lib().fw_dev_sync())
+    gen_s = time.time() - t0
+
+    if wl["queries"] == "all":
+        starts = np.arange(g.V, dtype=np.int32)
+    else:
+        starts = np.random.RandomState(12345).randint(0, g.V, size=int(wl["queries"])).astype(np.int32)
+    n = len(starts)
+    params = fw.default_params(app=app_id, max_depth=wl["depth"] + 1, seed=1)
+    if args.hub_threshold >= 0:
+        params.hub_threshold = args.hub_threshold
+    if args.wg_threads:
+        params.wg_threads = args.wg_threads
+    d_starts = fw.DeviceBuffer.from_numpy(starts)
+    d_paths = fw.DeviceBuffer(n * params.max_depth * 4)
+
+    for _ in range(args.warmup):
+        g.walk_device(params, d_starts, n, d_paths)
+
+    fw.check(fw.lib().fw_dev_sync())
+    t0 = time.perf_counter()
+    kernel_ms = []
+    last = None
+    for _ in range(args.steps):
+        last = g.walk_device(params, d_starts, n, d_paths)  # synchronous: returns after the kernel finished
+        kernel_ms.append(last.kernel_ms)
+    fw.check(fw.lib().fw_dev_sync())
+    wall = time.perf_counter() - t0
+
+    steps_per_pass = last.steps
+    ms_per_step = wall * 1e3 / args.steps
+    value = steps_per_pass * args.steps / wall
+    avg_kernel_ms = float(np.mean(kernel_ms))
+    alg_bytes = algorithmic_bytes(wl["app"], last.steps, last.sampled_edges, n)
+    achieved = alg_bytes / (avg_kernel_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "walk steps/sec (1 GPU) + % of HBM roofline; R-MAT s24 DeepWalk len 80",
+        "value": value,
+        "unit": "steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: R-MAT scale %d ef 16 %s, %s, %d queries, length %d" % (
+                args.workload, wl["scale"], "symmetrised" if wl["sym"] else "directed", wl["app"], n, wl["depth"]),
+            "vertices": g.V, "csr_entries": g.E, "queries": n,
+            "walk_steps_per_pass": int(last.steps), "sampled_edges_per_pass": int(last.sampled_edges),
+            "wg_threads": params.wg_threads, "hub_threshold": params.hub_threshold, "grid": last.grid,
+            "graph_gen_s": round(gen_s, 2),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload if not args.scale else None),
+            "kernel": "fw_walk_zprs",
+            "kernel_ms": avg_kernel_ms,
+            "algorithmic_bytes": int(alg_bytes),
+        },
+    }
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(fw, g, params, starts, args.cpu_seconds)
+
+    g.destroy()
+    print(json.dumps(out))
+
+
+def cpu_baseline(fw, g, params, starts, target_s):
+    """Times the CPU oracle (the checker, used here only as the reported baseline) on a prefix of the queries."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import fw_oracle_binding as orc
+
+    labels = params.app == fw.APP_METAPATH
+    xadj, adj, w, lab = g.download(weights=not labels, labels=labels)
+    og = orc.Graph(xadj, adj, w, lab)
+    op = orc.from_walk_params(params)
+    cores = orc.lib().fw_oracle_num_threads()
+    # pilot to size the sample so that the timed run takes about target_s
+    pilot = min(len(starts), 4096)
+    t = time.perf_counter()
+    _, s0, _ = orc.walk(og, op, starts[:pilot])
+    dt = max(time.perf_counter() - t, 1e-4)
+    m = int(min(len(starts), max(pilot, pilot * target_s / dt)))
+    t = time.perf_counter()
+    _, steps, _ = orc.walk(og, op, starts[:m])
+    dt = time.perf_counter() - t
+    return {
+        "value": steps / dt, "unit": "steps/s", "cores": int(cores), "kind": "port",
+        "sample": "first %d of %d queries of the same workload, %d steps in %.1f s, OpenMP schedule(dynamic)" % (
+            m, len(starts), steps, dt),
+    }
+
+
+if __name__ == "__main__":
+    main()

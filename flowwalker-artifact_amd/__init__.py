@@ -124,18 +124,18 @@ def default_params(**overrides):
     return p
 
 
-def set_params(p, **kw):
+def set_params(params, /, **kw):
     for k, v in kw.items():
         if k == "schema":
             v = list(v)
-            p.schema_len = len(v)
+            params.schema_len = len(v)
             for i, s in enumerate(v[:FW_MAX_SCHEMA]):
-                p.schema[i] = int(s)
+                params.schema[i] = int(s)
         else:
-            if not hasattr(p, k):
+            if not hasattr(params, k):
                 raise AttributeError("unknown walk parameter %r" % k)
-            setattr(p, k, v)
-    return p
+            setattr(params, k, v)
+    return params
 
 
 def _ptr(arr):

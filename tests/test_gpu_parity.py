@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import _graphs
-import _oracle
+import fw_oracle_binding as _oracle
 
 pytestmark = pytest.mark.gpu
 
