@@ -13,7 +13,8 @@ import os
 import numpy as np
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "lib", "libflowwalker_hip.so")
+# FLOWWALKER_LIB points at an alternative build of the same library (A/B measurements)
+LIB_PATH = os.environ.get("FLOWWALKER_LIB") or os.path.join(_PKG, "lib", "libflowwalker_hip.so")
 
 FW_MAX_SCHEMA = 64
 APP_DEEPWALK, APP_PPR, APP_NODE2VEC, APP_METAPATH = 0, 1, 2, 3

@@ -27,6 +27,9 @@ constexpr uint32_t kStreamStop = 0x80000000u;  // PPR stop draw
 constexpr int kHubChunk = 32;                  // hub tasks whose wave partials are parked in LDS at once
 constexpr int kFlagMoved = 1;
 constexpr int kFlagDead = 2;
+#ifndef FW_STREAM_UNROLL
+#define FW_STREAM_UNROLL 4
+#endif
 
 // ---- Philox4x32-10 ---------------------------------------------------------------------------
 
@@ -48,14 +51,6 @@ __device__ __forceinline__ uint4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_
 }
 
 __device__ __forceinline__ float u24(uint32_t bits) { return (float)(bits >> 8) * 0x1p-24f; }
-
-__device__ __forceinline__ uint32_t word_of(const uint4& r, uint32_t i) {
-  uint32_t x = r.x;
-  x = (i == 1u) ? r.y : x;
-  x = (i == 2u) ? r.z : x;
-  x = (i == 3u) ? r.w : x;
-  return x;
-}
 
 // ---- wave64 scans on the DPP network -----------------------------------------------------------
 
@@ -116,92 +111,140 @@ __device__ __forceinline__ bool sorted_contains(const int32_t* __restrict__ arr,
   return false;
 }
 
-// Lane-local reservoir over quartets t, t+P, t+2P, ... of the neighbour list.
+// Per-lane reservoir state while a neighbour list streams by.
+struct LaneState {
+  float S = 0.0f;    // running sum of biases seen by this lane
+  float Sj = 0.0f;   // running sum at the last acceptance
+  float u = 1.0f;    // uniform that decides the next acceptance: first element with S * u > Sj
+  // unread words of the lane's Philox stream, next one first; draw n of the stream is word n & 3 of
+  // block n >> 2, and draw 0 is the lane's combine draw, so block 0 leaves three words for jumps
+  uint32_t q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+  uint32_t avail = 0;  // unread words in the queue
+  uint32_t blk = 0;    // index of the block the queue came from
+  int32_t sel = -1;  // local index of the last accepted element
+  int32_t selv = -1; // its vertex id (only tracked when the adjacency quartet is loaded alongside)
+};
+
+// Feeds one quartet (absolute CSR index base..base+3, raw 32-bit words of the bias array and, when
+// needed, of the adjacency array) to the lane's reservoir.
+template <int kApp, bool kTrackV>
+__device__ __forceinline__ void consume_quartet(LaneState& st, const fw_kargs& a, const StepCtx& c, const int t,
+                                                const uint32_t base, const bool edge, const uint32_t end, uint4 raw,
+                                                int4 adj) {
+  float w0, w1, w2, w3;
+  if (kApp == FW_APP_METAPATH) {  // include/app.cuh:141-146
+    w0 = (int32_t)raw.x == c.want ? 1.0f : 0.0f;
+    w1 = (int32_t)raw.y == c.want ? 1.0f : 0.0f;
+    w2 = (int32_t)raw.z == c.want ? 1.0f : 0.0f;
+    w3 = (int32_t)raw.w == c.want ? 1.0f : 0.0f;
+  } else {
+    w0 = __uint_as_float(raw.x); w1 = __uint_as_float(raw.y);
+    w2 = __uint_as_float(raw.z); w3 = __uint_as_float(raw.w);
+  }
+  if (edge) {  // head / tail quartet: entries outside [off, end) have no bias
+    const bool in0 = base >= c.off && base < end;
+    const bool in1 = base + 1u >= c.off && base + 1u < end;
+    const bool in2 = base + 2u >= c.off && base + 2u < end;
+    const bool in3 = base + 3u >= c.off && base + 3u < end;
+    w0 = in0 ? w0 : 0.0f;
+    w1 = in1 ? w1 : 0.0f;
+    w2 = in2 ? w2 : 0.0f;
+    w3 = in3 ? w3 : 0.0f;
+    if (kApp == FW_APP_NODE2VEC) {  // never search for an entry of a foreign list
+      adj.x = in0 ? adj.x : c.prev; adj.y = in1 ? adj.y : c.prev;
+      adj.z = in2 ? adj.z : c.prev; adj.w = in3 ? adj.w : c.prev;
+    }
+  }
+  if (kApp == FW_APP_NODE2VEC && c.prev != -1) {  // include/app.cuh:108-123
+    const int32_t* __restrict__ plist = a.adjncy + c.prev_off;
+    w0 = (adj.x == c.prev) ? w0 * a.inv_p : (sorted_contains(plist, c.prev_deg, adj.x) ? w0 : w0 * a.inv_q);
+    w1 = (adj.y == c.prev) ? w1 * a.inv_p : (sorted_contains(plist, c.prev_deg, adj.y) ? w1 : w1 * a.inv_q);
+    w2 = (adj.z == c.prev) ? w2 * a.inv_p : (sorted_contains(plist, c.prev_deg, adj.z) ? w2 : w2 * a.inv_q);
+    w3 = (adj.w == c.prev) ? w3 * a.inv_p : (sorted_contains(plist, c.prev_deg, adj.w) ? w3 : w3 * a.inv_q);
+  }
+
+  const float s1 = st.S + w0;
+  const float s2 = s1 + w1;
+  const float s3 = s2 + w2;
+  const float s4 = s3 + w3;
+  // S is non-decreasing, so the next acceptance lies in this quartet iff it triggers at its end.
+  if (s4 * st.u > st.Sj) {
+#define FW_ELEM(sj_, vj_, j_)                                                                        \
+  if ((sj_) * st.u > st.Sj) {                                                                        \
+    st.sel = (int32_t)(base + (j_) - c.off);                                                         \
+    if (kTrackV) st.selv = (vj_);                                                                    \
+    st.Sj = (sj_);                                                                                   \
+    if (st.avail == 0u) {                                                                            \
+      ++st.blk;                                                                                      \
+      const uint4 nb = philox4x32_10(c.walker, c.step, (uint32_t)t, st.blk, a.seed_lo, a.seed_hi);   \
+      st.q0 = nb.x; st.q1 = nb.y; st.q2 = nb.z; st.q3 = nb.w;                                        \
+      st.avail = 4u;                                                                                 \
+    }                                                                                                \
+    st.u = u24(st.q0);                                                                               \
+    st.q0 = st.q1; st.q1 = st.q2; st.q2 = st.q3;                                                     \
+    --st.avail;                                                                                      \
+  }
+    FW_ELEM(s1, adj.x, 0u)
+    FW_ELEM(s2, adj.y, 1u)
+    FW_ELEM(s3, adj.z, 2u)
+    FW_ELEM(s4, adj.w, 3u)
+#undef FW_ELEM
+  }
+  st.S = s4;
+}
+
+// Lane-local reservoir over quartets t, t+P, t+2P, ... of the neighbour list, kU quartets in flight.
 // Outputs the lane total L, the lane's selected local index (or -1), the vertex behind it when
 // kTrackV (the adjacency quartet is then loaded alongside), and the lane's combine draw.
-template <int kApp, int kP, bool kTrackV>
+template <int kApp, int kP, bool kTrackV, int kU>
 __device__ __forceinline__ void lane_pass(const fw_kargs& a, const StepCtx& c, const int t, float& L, int32_t& sel,
                                           int32_t& selv, uint32_t& bern) {
   const uint32_t a0 = c.off & ~3u;
   const uint32_t end = c.off + (uint32_t)c.deg;
   const uint32_t nq = (end - a0 + 3u) >> 2;
+  const uint32_t* __restrict__ bias =
+      reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
+  const bool need_adj = kTrackV || (kApp == FW_APP_NODE2VEC && c.prev != -1);
 
-  float S = 0.0f, Sj = 0.0f, u = 1.0f;
-  uint32_t nd = 0;
-  uint4 r = make_uint4(0, 0, 0, 0);
-  sel = -1;
-  selv = -1;
+  LaneState st;
   bern = 0;
   if ((uint32_t)t < nq) {
-    r = philox4x32_10(c.walker, c.step, (uint32_t)t, 0u, a.seed_lo, a.seed_hi);
-    bern = r.x;
+    const uint4 b0 = philox4x32_10(c.walker, c.step, (uint32_t)t, 0u, a.seed_lo, a.seed_hi);
+    bern = b0.x;
+    st.q0 = b0.y; st.q1 = b0.z; st.q2 = b0.w;
+    st.avail = 3u;
   }
 
-  for (uint32_t k = (uint32_t)t; k < nq; k += (uint32_t)kP) {
-    const uint32_t base = a0 + 4u * k;
-    float w0, w1, w2, w3;
-    int32_t v0 = -1, v1 = -1, v2 = -1, v3 = -1;
-    if (kApp == FW_APP_METAPATH) {
-      const int4 lab = *reinterpret_cast<const int4*>(a.label + base);
-      w0 = lab.x == c.want ? 1.0f : 0.0f;
-      w1 = lab.y == c.want ? 1.0f : 0.0f;
-      w2 = lab.z == c.want ? 1.0f : 0.0f;
-      w3 = lab.w == c.want ? 1.0f : 0.0f;
-    } else {
-      const float4 w = *reinterpret_cast<const float4*>(a.weight + base);
-      w0 = w.x; w1 = w.y; w2 = w.z; w3 = w.w;
-    }
-    const bool need_adj = kTrackV || (kApp == FW_APP_NODE2VEC && c.prev != -1);
-    if (need_adj) {
-      const int4 adj = *reinterpret_cast<const int4*>(a.adjncy + base);
-      v0 = adj.x; v1 = adj.y; v2 = adj.z; v3 = adj.w;
-    }
-    if (k == 0u || k == nq - 1u) {  // head / tail quartet: entries outside [off, end) have no bias
-      const bool in0 = base >= c.off && base < end;
-      const bool in1 = base + 1u >= c.off && base + 1u < end;
-      const bool in2 = base + 2u >= c.off && base + 2u < end;
-      const bool in3 = base + 3u >= c.off && base + 3u < end;
-      w0 = in0 ? w0 : 0.0f;
-      w1 = in1 ? w1 : 0.0f;
-      w2 = in2 ? w2 : 0.0f;
-      w3 = in3 ? w3 : 0.0f;
-      if (kApp == FW_APP_NODE2VEC) {  // never search for an entry of a foreign list
-        v0 = in0 ? v0 : c.prev; v1 = in1 ? v1 : c.prev; v2 = in2 ? v2 : c.prev; v3 = in3 ? v3 : c.prev;
+  uint32_t k = (uint32_t)t;
+  if (kU > 1) {
+    // all kU quartets of the group exist for this lane: issue the loads together, then consume in order
+    for (; k + (uint32_t)((kU - 1) * kP) < nq; k += (uint32_t)(kU * kP)) {
+      uint4 raw[kU];
+      int4 adj[kU];
+#pragma unroll
+      for (int j = 0; j < kU; ++j) {
+        const uint32_t base = a0 + 4u * (k + (uint32_t)(j * kP));
+        raw[j] = *reinterpret_cast<const uint4*>(bias + base);
+        adj[j] = make_int4(-1, -1, -1, -1);
+        if (need_adj) adj[j] = *reinterpret_cast<const int4*>(a.adjncy + base);
+      }
+#pragma unroll
+      for (int j = 0; j < kU; ++j) {
+        const uint32_t kk = k + (uint32_t)(j * kP);
+        consume_quartet<kApp, kTrackV>(st, a, c, t, a0 + 4u * kk, kk == 0u || kk == nq - 1u, end, raw[j], adj[j]);
       }
     }
-    if (kApp == FW_APP_NODE2VEC && c.prev != -1) {  // include/app.cuh:108-123
-      const int32_t* __restrict__ plist = a.adjncy + c.prev_off;
-      w0 = (v0 == c.prev) ? w0 * a.inv_p : (sorted_contains(plist, c.prev_deg, v0) ? w0 : w0 * a.inv_q);
-      w1 = (v1 == c.prev) ? w1 * a.inv_p : (sorted_contains(plist, c.prev_deg, v1) ? w1 : w1 * a.inv_q);
-      w2 = (v2 == c.prev) ? w2 * a.inv_p : (sorted_contains(plist, c.prev_deg, v2) ? w2 : w2 * a.inv_q);
-      w3 = (v3 == c.prev) ? w3 * a.inv_p : (sorted_contains(plist, c.prev_deg, v3) ? w3 : w3 * a.inv_q);
-    }
-
-    const float s1 = S + w0;
-    const float s2 = s1 + w1;
-    const float s3 = s2 + w2;
-    const float s4 = s3 + w3;
-    // S is non-decreasing, so the next acceptance lies in this quartet iff it triggers at its end.
-    if (s4 * u > Sj) {
-#define FW_ELEM(sj_, vj_, j_)                                                            \
-  if ((sj_) * u > Sj) {                                                                  \
-    sel = (int32_t)(base + (j_) - c.off);                                                \
-    if (kTrackV) selv = (vj_);                                                           \
-    Sj = (sj_);                                                                          \
-    const uint32_t n = 1u + nd;                                                          \
-    if ((n & 3u) == 0u) r = philox4x32_10(c.walker, c.step, (uint32_t)t, n >> 2, a.seed_lo, a.seed_hi); \
-    u = u24(word_of(r, n & 3u));                                                         \
-    ++nd;                                                                                \
   }
-      FW_ELEM(s1, v0, 0u)
-      FW_ELEM(s2, v1, 1u)
-      FW_ELEM(s3, v2, 2u)
-      FW_ELEM(s4, v3, 3u)
-#undef FW_ELEM
-    }
-    S = s4;
+  for (; k < nq; k += (uint32_t)kP) {
+    const uint32_t base = a0 + 4u * k;
+    const uint4 raw = *reinterpret_cast<const uint4*>(bias + base);
+    int4 adj = make_int4(-1, -1, -1, -1);
+    if (need_adj) adj = *reinterpret_cast<const int4*>(a.adjncy + base);
+    consume_quartet<kApp, kTrackV>(st, a, c, t, base, k == 0u || k == nq - 1u, end, raw, adj);
   }
-  L = S;
+  L = st.S;
+  sel = st.sel;
+  selv = st.selv;
 }
 
 // Combines the 64 lane reservoirs of one wave: lane l is accepted iff L > 0 and bern * prefix < L;
@@ -282,6 +325,8 @@ __device__ __forceinline__ void commit(const fw_kargs& a, TaskTable<kWGT>& tt, i
 template <int kApp, int kWGT>
 __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
   constexpr int kNW = kWGT / 64;
+  // quartets in flight per lane while streaming; node2vec is bound by its adjacency probes instead
+  constexpr int kUnroll = (kApp == FW_APP_NODE2VEC) ? 1 : FW_STREAM_UNROLL;
   __shared__ TaskTable<kWGT> tt;
 
   const int tid = (int)threadIdx.x;
@@ -317,7 +362,7 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
           float L, W;
           int32_t sel, selv;
           uint32_t bern;
-          lane_pass<kApp, kWGT, false>(a, c, tid, L, sel, selv, bern);
+          lane_pass<kApp, kWGT, false, kUnroll>(a, c, tid, L, sel, selv, bern);
           const int win = wave_combine(L, bern, W);
           const int32_t wsel = (win >= 0) ? __builtin_amdgcn_readlane(sel, win) : -1;
           if (lane == 0) {
@@ -367,11 +412,11 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
         int win;
         int32_t v = -1;
         if (nq <= 64u) {  // one quartet per lane: fetch the adjacency with the weights, no dependent load
-          lane_pass<kApp, 64, true>(a, c, lane, L, sel, selv, bern);
+          lane_pass<kApp, 64, true, 1>(a, c, lane, L, sel, selv, bern);
           win = wave_combine(L, bern, W);
           if (win >= 0) v = __builtin_amdgcn_readlane(selv, win);
         } else {
-          lane_pass<kApp, 64, false>(a, c, lane, L, sel, selv, bern);
+          lane_pass<kApp, 64, false, kUnroll>(a, c, lane, L, sel, selv, bern);
           win = wave_combine(L, bern, W);
           if (win >= 0) {
             const int32_t pick = __builtin_amdgcn_readlane(sel, win);
