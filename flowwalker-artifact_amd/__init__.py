@@ -24,7 +24,7 @@ FW_OK = 0
 # every symbol include/flowwalker.h declares
 EXPORTED = [
     "fw_last_error", "fw_device_count", "fw_device_mem_info", "fw_walk_params_default", "fw_autobatch_size",
-    "fw_dev_alloc", "fw_dev_free", "fw_dev_upload", "fw_dev_download", "fw_dev_fill_i32", "fw_dev_sync",
+    "fw_dev_alloc", "fw_dev_free", "fw_dev_upload", "fw_dev_download", "fw_dev_fill_i32", "fw_dev_copy", "fw_dev_sync",
     "fw_graph_create", "fw_graph_adopt_device", "fw_graph_destroy", "fw_graph_info", "fw_graph_is_sorted",
     "fw_graph_download", "fw_walk_device", "fw_walk_batch", "fw_host_alloc_pinned", "fw_host_free_pinned",
     "fw_gen_rmat",
@@ -83,6 +83,7 @@ def lib():
         L.fw_dev_upload.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         L.fw_dev_download.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         L.fw_dev_fill_i32.argtypes = [C.c_void_p, C.c_int32, C.c_size_t]
+        L.fw_dev_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         L.fw_graph_create.argtypes = [C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.POINTER(C.c_void_p)]
         L.fw_graph_adopt_device.argtypes = [C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

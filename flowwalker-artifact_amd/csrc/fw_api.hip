@@ -130,6 +130,25 @@ extern "C" int fw_dev_fill_i32(int32_t* d_dst, int32_t value, size_t count) {
   FW_HIP(hipDeviceSynchronize());
   return FW_OK;
 }
+__global__ void fw_copy_u32x4_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t count) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) dst[i] = src[i];
+}
+extern "C" int fw_dev_copy(void* d_dst, const void* d_src, size_t bytes) {
+  if (bytes == 0) return FW_OK;
+  if ((bytes & 15u) || (((uintptr_t)d_dst | (uintptr_t)d_src) & 15u)) {
+    fw_set_error("fw_dev_copy: pointers and size must be multiples of 16 bytes");
+    return FW_ERR_INVALID;
+  }
+  const size_t count = bytes / 16;
+  size_t blocks = (count + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL(fw_copy_u32x4_kernel, dim3((unsigned)blocks), dim3(256), 0, 0, static_cast<uint4*>(d_dst),
+                     static_cast<const uint4*>(d_src), count);
+  FW_HIP(hipGetLastError());
+  FW_HIP(hipDeviceSynchronize());
+  return FW_OK;
+}
 extern "C" int fw_dev_sync(void) {
   FW_HIP(hipDeviceSynchronize());
   return FW_OK;

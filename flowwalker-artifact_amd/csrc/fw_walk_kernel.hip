@@ -1,35 +1,42 @@
 // Sampler-centric random-walk kernel for gfx950 (MI355X): persistent workgroups, an LDS task table,
-// a global atomic query dispenser, a one-pass zero-preprocessing parallel reservoir sampler (ZPRS)
-// at wavefront (64 lanes) and workgroup granularity, Philox4x32-10 counter-based draws, and the
+// a global atomic query dispenser, a one-pass zero-preprocessing parallel reservoir sampler at
+// wavefront (64 lanes) and workgroup granularity, Philox4x32-10 counter-based draws, and the
 // DeepWalk / PPR / node2vec / MetaPath bias functors.
 //
 // Reference behaviour this replaces: walker_wb_dynamic_zprs / _dprs (include/walker.cuh:1307-1580),
-// sampler_warp / sampler_block (include/sampler.cuh:46-127), Task (include/gpu_task.cuh:24-78),
-// the functors of include/app.cuh:58-152 and check_connect (include/gpu_graph.cuh:97-118).
+// sampler_warp / sampler_block and their one-loop forms (include/sampler.cuh:46-200), Task
+// (include/gpu_task.cuh:24-78), the functors of include/app.cuh:58-152 and check_connect
+// (include/gpu_graph.cuh:97-118).
+//
+// Sampler.  A neighbour list is cut into groups of 64 lanes x 4 quartets x 4 elements = 1024 biases.
+// A wave streams the groups it owns: four aligned 16-byte loads per lane, 16 adds, one DPP scan of the
+// lane totals.  The group totals feed a sequential weighted reservoir whose acceptance test
+// "S * u > Sj" uses one uniform per ACCEPTED group (the probability of no acceptance between two
+// groups telescopes to a ratio of running sums), so the common iteration has no random draw and no
+// divergent branch.  Inside an accepted group the element is found by inverse transform on the scan
+// prefix.  All draws of a step are wave-uniform, so Philox runs on the scalar unit.
 //
 // Round structure of one workgroup (WGT threads, WGT task slots in LDS, SoA):
-//   B  every hub slot (degree > hub_threshold) is streamed by the whole workgroup: lane-local
-//      reservoirs, per-wave combine, partial (selection, total) pairs parked in LDS; one barrier per
-//      chunk of hubs, then one wave per hub combines the wave partials and commits the step.
+//   B  every hub slot (degree > hub_threshold) is streamed by the whole workgroup, wave w taking
+//      groups w, w + NW, ...; per-wave (selection, total) pairs are parked in LDS; one barrier per
+//      chunk of hubs, then one wave per hub picks the winning wave and commits the step.
 //   A  waves claim the remaining slots one by one from an LDS counter and sample them alone.
 //   C  one thread per slot: reload the CSR range of the new vertex, stop test, refill from the
 //      global dispenser (one atomic per wave per refill round), classify into next round's lists.
 //
 // Results depend only on (seed, walker id, graph, parameters): every random draw is addressed by
-// (walker, step, lane stream, draw index), never by which wave or workgroup happens to run the slot.
+// (walker, step, stream, draw index), never by which wave or workgroup happens to run the slot.
 
 #include "fw_internal.h"
 
 namespace {
 
-constexpr uint32_t kStreamWave = 0x40000000u;  // | wave index: workgroup-level combine draws
+constexpr uint32_t kStreamWave = 0x40000000u;  // workgroup-level combine draw
 constexpr uint32_t kStreamStop = 0x80000000u;  // PPR stop draw
 constexpr int kHubChunk = 32;                  // hub tasks whose wave partials are parked in LDS at once
+constexpr int kGroupQuartets = 4;              // quartets per lane per group (part of the sampler's definition)
 constexpr int kFlagMoved = 1;
 constexpr int kFlagDead = 2;
-#ifndef FW_STREAM_UNROLL
-#define FW_STREAM_UNROLL 4
-#endif
 
 // ---- Philox4x32-10 ---------------------------------------------------------------------------
 
@@ -86,6 +93,10 @@ __device__ __forceinline__ float row_scan(float x) {
 
 __device__ __forceinline__ int lane_id() { return (int)__lane_id(); }
 
+__device__ __forceinline__ float readlane_f(float x, int l) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), l));
+}
+
 // ---- per-step context (wave-uniform) -----------------------------------------------------------
 
 struct StepCtx {
@@ -111,152 +122,174 @@ __device__ __forceinline__ bool sorted_contains(const int32_t* __restrict__ arr,
   return false;
 }
 
-// Per-lane reservoir state while a neighbour list streams by.
-struct LaneState {
-  float S = 0.0f;    // running sum of biases seen by this lane
-  float Sj = 0.0f;   // running sum at the last acceptance
-  float u = 1.0f;    // uniform that decides the next acceptance: first element with S * u > Sj
-  // unread words of the lane's Philox stream, next one first; draw n of the stream is word n & 3 of
-  // block n >> 2, and draw 0 is the lane's combine draw, so block 0 leaves three words for jumps
-  uint32_t q0 = 0, q1 = 0, q2 = 0, q3 = 0;
-  uint32_t avail = 0;  // unread words in the queue
-  uint32_t blk = 0;    // index of the block the queue came from
-  int32_t sel = -1;  // local index of the last accepted element
-  int32_t selv = -1; // its vertex id (only tracked when the adjacency quartet is loaded alongside)
-};
-
-// Feeds one quartet (absolute CSR index base..base+3, raw 32-bit words of the bias array and, when
-// needed, of the adjacency array) to the lane's reservoir.
-template <int kApp, bool kTrackV>
-__device__ __forceinline__ void consume_quartet(LaneState& st, const fw_kargs& a, const StepCtx& c, const int t,
-                                                const uint32_t base, const bool edge, const uint32_t end, uint4 raw,
-                                                int4 adj) {
-  float w0, w1, w2, w3;
-  if (kApp == FW_APP_METAPATH) {  // include/app.cuh:141-146
-    w0 = (int32_t)raw.x == c.want ? 1.0f : 0.0f;
-    w1 = (int32_t)raw.y == c.want ? 1.0f : 0.0f;
-    w2 = (int32_t)raw.z == c.want ? 1.0f : 0.0f;
-    w3 = (int32_t)raw.w == c.want ? 1.0f : 0.0f;
-  } else {
-    w0 = __uint_as_float(raw.x); w1 = __uint_as_float(raw.y);
-    w2 = __uint_as_float(raw.z); w3 = __uint_as_float(raw.w);
-  }
-  if (edge) {  // head / tail quartet: entries outside [off, end) have no bias
-    const bool in0 = base >= c.off && base < end;
-    const bool in1 = base + 1u >= c.off && base + 1u < end;
-    const bool in2 = base + 2u >= c.off && base + 2u < end;
-    const bool in3 = base + 3u >= c.off && base + 3u < end;
-    w0 = in0 ? w0 : 0.0f;
-    w1 = in1 ? w1 : 0.0f;
-    w2 = in2 ? w2 : 0.0f;
-    w3 = in3 ? w3 : 0.0f;
-    if (kApp == FW_APP_NODE2VEC) {  // never search for an entry of a foreign list
-      adj.x = in0 ? adj.x : c.prev; adj.y = in1 ? adj.y : c.prev;
-      adj.z = in2 ? adj.z : c.prev; adj.w = in3 ? adj.w : c.prev;
-    }
-  }
-  if (kApp == FW_APP_NODE2VEC && c.prev != -1) {  // include/app.cuh:108-123
-    const int32_t* __restrict__ plist = a.adjncy + c.prev_off;
-    w0 = (adj.x == c.prev) ? w0 * a.inv_p : (sorted_contains(plist, c.prev_deg, adj.x) ? w0 : w0 * a.inv_q);
-    w1 = (adj.y == c.prev) ? w1 * a.inv_p : (sorted_contains(plist, c.prev_deg, adj.y) ? w1 : w1 * a.inv_q);
-    w2 = (adj.z == c.prev) ? w2 * a.inv_p : (sorted_contains(plist, c.prev_deg, adj.z) ? w2 : w2 * a.inv_q);
-    w3 = (adj.w == c.prev) ? w3 * a.inv_p : (sorted_contains(plist, c.prev_deg, adj.w) ? w3 : w3 * a.inv_q);
-  }
-
-  const float s1 = st.S + w0;
-  const float s2 = s1 + w1;
-  const float s3 = s2 + w2;
-  const float s4 = s3 + w3;
-  // S is non-decreasing, so the next acceptance lies in this quartet iff it triggers at its end.
-  if (s4 * st.u > st.Sj) {
-#define FW_ELEM(sj_, vj_, j_)                                                                        \
-  if ((sj_) * st.u > st.Sj) {                                                                        \
-    st.sel = (int32_t)(base + (j_) - c.off);                                                         \
-    if (kTrackV) st.selv = (vj_);                                                                    \
-    st.Sj = (sj_);                                                                                   \
-    if (st.avail == 0u) {                                                                            \
-      ++st.blk;                                                                                      \
-      const uint4 nb = philox4x32_10(c.walker, c.step, (uint32_t)t, st.blk, a.seed_lo, a.seed_hi);   \
-      st.q0 = nb.x; st.q1 = nb.y; st.q2 = nb.z; st.q3 = nb.w;                                        \
-      st.avail = 4u;                                                                                 \
-    }                                                                                                \
-    st.u = u24(st.q0);                                                                               \
-    st.q0 = st.q1; st.q1 = st.q2; st.q2 = st.q3;                                                     \
-    --st.avail;                                                                                      \
-  }
-    FW_ELEM(s1, adj.x, 0u)
-    FW_ELEM(s2, adj.y, 1u)
-    FW_ELEM(s3, adj.z, 2u)
-    FW_ELEM(s4, adj.w, 3u)
-#undef FW_ELEM
-  }
-  st.S = s4;
+// node2vec bias of one neighbour (include/app.cuh:108-123).  Entries outside the list arrive with
+// post == prev and weight 0, so they are never searched for.
+__device__ __forceinline__ float n2v_bias(const fw_kargs& a, const StepCtx& c, float w, int32_t post) {
+  if (post == c.prev) return w * a.inv_p;
+  return sorted_contains(a.adjncy + c.prev_off, c.prev_deg, post) ? w : w * a.inv_q;
 }
 
-// Lane-local reservoir over quartets t, t+P, t+2P, ... of the neighbour list, kU quartets in flight.
-// Outputs the lane total L, the lane's selected local index (or -1), the vertex behind it when
-// kTrackV (the adjacency quartet is then loaded alongside), and the lane's combine draw.
-template <int kApp, int kP, bool kTrackV, int kU>
-__device__ __forceinline__ void lane_pass(const fw_kargs& a, const StepCtx& c, const int t, float& L, int32_t& sel,
-                                          int32_t& selv, uint32_t& bern) {
+// Wave-uniform queue of Philox words: draw n of a stream is word n & 3 of block n >> 2.
+struct DrawQueue {
+  uint32_t q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+  uint32_t avail = 0;
+  uint32_t blk = 0;
+};
+
+__device__ __forceinline__ float next_uniform(DrawQueue& d, const fw_kargs& a, const StepCtx& c, uint32_t stream) {
+  if (d.avail == 0u) {
+    const uint4 b = philox4x32_10(c.walker, c.step, stream, d.blk, a.seed_lo, a.seed_hi);
+    d.q0 = b.x; d.q1 = b.y; d.q2 = b.z; d.q3 = b.w;
+    d.avail = 4u;
+    ++d.blk;
+  }
+  const float u = u24(d.q0);
+  d.q0 = d.q1; d.q1 = d.q2; d.q2 = d.q3;
+  --d.avail;
+  return u;
+}
+
+// One wave streams the groups w, w + nw, ... of a neighbour list and keeps a reservoir over them.
+// kJ = quartets per lane per group that can exist (kGroupQuartets, or 1 when the caller knows that the
+// list has at most 64 quartets).  kTrackV: also load the adjacency quartet and return the selected
+// vertex.  Outputs: running total S of the wave's groups, selected local index (or -1), its vertex.
+template <int kApp, int kJ, bool kTrackV>
+__device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c, const int lane, const uint32_t w,
+                                            const uint32_t nw, float& S_out, int32_t& sel_out, int32_t& selv_out) {
+  constexpr uint32_t kG = 64u * kGroupQuartets;  // quartets per group
+  constexpr int kEl = 4 * kJ;
   const uint32_t a0 = c.off & ~3u;
   const uint32_t end = c.off + (uint32_t)c.deg;
   const uint32_t nq = (end - a0 + 3u) >> 2;
+  const uint32_t ngroups = (nq + kG - 1u) / kG;
   const uint32_t* __restrict__ bias =
       reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
-  const bool need_adj = kTrackV || (kApp == FW_APP_NODE2VEC && c.prev != -1);
+  const bool n2v = kApp == FW_APP_NODE2VEC && c.prev != -1;
+  const bool need_adj = kTrackV || n2v;
 
-  LaneState st;
-  bern = 0;
-  if ((uint32_t)t < nq) {
-    const uint4 b0 = philox4x32_10(c.walker, c.step, (uint32_t)t, 0u, a.seed_lo, a.seed_hi);
-    bern = b0.x;
-    st.q0 = b0.y; st.q1 = b0.z; st.q2 = b0.w;
-    st.avail = 3u;
-  }
+  float S = 0.0f, Sj = 0.0f, u = 1.0f;
+  int32_t sel = -1, selv = -1;
+  DrawQueue dq;
 
-  uint32_t k = (uint32_t)t;
-  if (kU > 1) {
-    // all kU quartets of the group exist for this lane: issue the loads together, then consume in order
-    for (; k + (uint32_t)((kU - 1) * kP) < nq; k += (uint32_t)(kU * kP)) {
-      uint4 raw[kU];
-      int4 adj[kU];
+  for (uint32_t g = w; g < ngroups; g += nw) {
+    const uint32_t kb = g * kG + (uint32_t)lane;  // this lane's quartet for j = 0
+    uint4 raw[kJ];
+    int4 adj[kJ];
+    float x[kEl];
+    const bool interior = g > 0u && (g + 1u) * kG < nq;  // no head / tail quartet, every quartet exists
+    if (interior) {
 #pragma unroll
-      for (int j = 0; j < kU; ++j) {
-        const uint32_t base = a0 + 4u * (k + (uint32_t)(j * kP));
+      for (int j = 0; j < kJ; ++j) {
+        const uint32_t base = a0 + 4u * (kb + 64u * (uint32_t)j);
         raw[j] = *reinterpret_cast<const uint4*>(bias + base);
         adj[j] = make_int4(-1, -1, -1, -1);
         if (need_adj) adj[j] = *reinterpret_cast<const int4*>(a.adjncy + base);
       }
+    } else {
 #pragma unroll
-      for (int j = 0; j < kU; ++j) {
-        const uint32_t kk = k + (uint32_t)(j * kP);
-        consume_quartet<kApp, kTrackV>(st, a, c, t, a0 + 4u * kk, kk == 0u || kk == nq - 1u, end, raw[j], adj[j]);
+      for (int j = 0; j < kJ; ++j) {
+        const uint32_t k = kb + 64u * (uint32_t)j;
+        const uint32_t base = a0 + 4u * k;
+        raw[j] = make_uint4(0, 0, 0, 0);
+        adj[j] = make_int4(c.prev, c.prev, c.prev, c.prev);
+        if (k < nq) {
+          raw[j] = *reinterpret_cast<const uint4*>(bias + base);
+          if (need_adj) adj[j] = *reinterpret_cast<const int4*>(a.adjncy + base);
+        }
       }
     }
-  }
-  for (; k < nq; k += (uint32_t)kP) {
-    const uint32_t base = a0 + 4u * k;
-    const uint4 raw = *reinterpret_cast<const uint4*>(bias + base);
-    int4 adj = make_int4(-1, -1, -1, -1);
-    if (need_adj) adj = *reinterpret_cast<const int4*>(a.adjncy + base);
-    consume_quartet<kApp, kTrackV>(st, a, c, t, base, k == 0u || k == nq - 1u, end, raw, adj);
-  }
-  L = st.S;
-  sel = st.sel;
-  selv = st.selv;
-}
+#pragma unroll
+    for (int j = 0; j < kJ; ++j) {
+      if (kApp == FW_APP_METAPATH) {  // include/app.cuh:141-146
+        x[4 * j + 0] = (int32_t)raw[j].x == c.want ? 1.0f : 0.0f;
+        x[4 * j + 1] = (int32_t)raw[j].y == c.want ? 1.0f : 0.0f;
+        x[4 * j + 2] = (int32_t)raw[j].z == c.want ? 1.0f : 0.0f;
+        x[4 * j + 3] = (int32_t)raw[j].w == c.want ? 1.0f : 0.0f;
+      } else {
+        x[4 * j + 0] = __uint_as_float(raw[j].x);
+        x[4 * j + 1] = __uint_as_float(raw[j].y);
+        x[4 * j + 2] = __uint_as_float(raw[j].z);
+        x[4 * j + 3] = __uint_as_float(raw[j].w);
+      }
+    }
+    if (!interior) {  // entries outside [off, end) (head / tail quartet, quartets past the list) have no bias
+#pragma unroll
+      for (int j = 0; j < kJ; ++j) {
+        const uint32_t k = kb + 64u * (uint32_t)j;
+        const uint32_t base = a0 + 4u * k;
+        const bool ex = k < nq;
+        const bool in0 = ex && base >= c.off && base < end;
+        const bool in1 = ex && base + 1u >= c.off && base + 1u < end;
+        const bool in2 = ex && base + 2u >= c.off && base + 2u < end;
+        const bool in3 = ex && base + 3u >= c.off && base + 3u < end;
+        x[4 * j + 0] = in0 ? x[4 * j + 0] : 0.0f;
+        x[4 * j + 1] = in1 ? x[4 * j + 1] : 0.0f;
+        x[4 * j + 2] = in2 ? x[4 * j + 2] : 0.0f;
+        x[4 * j + 3] = in3 ? x[4 * j + 3] : 0.0f;
+        if (kApp == FW_APP_NODE2VEC) {  // never search for an entry of a foreign list
+          adj[j].x = in0 ? adj[j].x : c.prev; adj[j].y = in1 ? adj[j].y : c.prev;
+          adj[j].z = in2 ? adj[j].z : c.prev; adj[j].w = in3 ? adj[j].w : c.prev;
+        }
+      }
+    }
+    if (n2v) {
+#pragma unroll
+      for (int j = 0; j < kJ; ++j) {
+        x[4 * j + 0] = n2v_bias(a, c, x[4 * j + 0], adj[j].x);
+        x[4 * j + 1] = n2v_bias(a, c, x[4 * j + 1], adj[j].y);
+        x[4 * j + 2] = n2v_bias(a, c, x[4 * j + 2], adj[j].z);
+        x[4 * j + 3] = n2v_bias(a, c, x[4 * j + 3], adj[j].w);
+      }
+    }
 
-// Combines the 64 lane reservoirs of one wave: lane l is accepted iff L > 0 and bern * prefix < L;
-// the last accepted lane wins (include/sampler.cuh:82-84 takes the max over lane-tagged keys).
-// Returns the winning lane or -1; W = wave total.
-__device__ __forceinline__ int wave_combine(float L, uint32_t bern, float& W) {
-  const float I = wave_scan(L);
-  const bool acc = (L > 0.0f) && (u24(bern) * I < L);
-  const uint64_t m = __ballot(acc);
-  W = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(I), 63));
-  if (m == 0ull) return -1;
-  return 63 - __builtin_clzll(m);
+    float q = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kEl; ++i) q = q + x[i];
+    const float I = wave_scan(q);
+    const float T = readlane_f(I, 63);
+    const float Snew = S + T;
+    if (Snew * u > Sj) {  // wave-uniform: the reservoir accepts this group
+      const float target = next_uniform(dq, a, c, w) * T;
+      const bool pos = q > 0.0f;
+      const uint64_t m = __ballot(pos && I > target);
+      int l;
+      if (m != 0ull) {
+        l = __builtin_ctzll(m);
+      } else {  // rounding in the scan tree left no crossing: last lane with a positive total
+        l = 63 - __builtin_clzll(__ballot(pos));
+      }
+      // every lane resolves its own elements; the answer of lane l is the one that is read
+      float e = I - q;
+      int pick = -1, last = -1;
+#pragma unroll
+      for (int i = 0; i < kEl; ++i) {
+        e = e + x[i];
+        const bool p = x[i] > 0.0f;
+        pick = (p && e > target && pick < 0) ? i : pick;
+        last = p ? i : last;
+      }
+      pick = pick < 0 ? last : pick;
+      const uint32_t abs_idx = a0 + 4u * kb + 256u * (uint32_t)(pick >> 2) + (uint32_t)(pick & 3);
+      sel = __builtin_amdgcn_readlane((int32_t)(abs_idx - c.off), l);
+      if (kTrackV) {
+        int32_t v = adj[0].x;
+#pragma unroll
+        for (int j = 0; j < kJ; ++j) {
+          v = (pick == 4 * j + 0) ? adj[j].x : v;
+          v = (pick == 4 * j + 1) ? adj[j].y : v;
+          v = (pick == 4 * j + 2) ? adj[j].z : v;
+          v = (pick == 4 * j + 3) ? adj[j].w : v;
+        }
+        selv = __builtin_amdgcn_readlane(v, l);
+      }
+      Sj = Snew;
+      u = next_uniform(dq, a, c, w);
+    }
+    S = Snew;
+  }
+  S_out = S;
+  sel_out = sel;
+  selv_out = selv;
 }
 
 // ---- LDS task table ----------------------------------------------------------------------------
@@ -285,16 +318,17 @@ struct TaskTable {
   int32_t hub_sel[kHubChunk][16];
 };
 
+// The slot index is wave-uniform; readfirstlane tells the compiler so (scalar registers, scalar Philox).
 template <int kWGT>
 __device__ __forceinline__ StepCtx load_ctx(const fw_kargs& a, const TaskTable<kWGT>& tt, int slot) {
   StepCtx c;
-  c.off = tt.off[slot];
-  c.deg = tt.deg[slot];
-  c.prev = tt.prev[slot];
-  c.prev_off = tt.prev_off[slot];
-  c.prev_deg = tt.prev_deg[slot];
-  c.walker = a.walker_base + (uint32_t)tt.walker[slot];
-  c.step = (uint32_t)(tt.len[slot] - 1);
+  c.off = (uint32_t)__builtin_amdgcn_readfirstlane((int)tt.off[slot]);
+  c.deg = __builtin_amdgcn_readfirstlane(tt.deg[slot]);
+  c.prev = __builtin_amdgcn_readfirstlane(tt.prev[slot]);
+  c.prev_off = (uint32_t)__builtin_amdgcn_readfirstlane((int)tt.prev_off[slot]);
+  c.prev_deg = __builtin_amdgcn_readfirstlane(tt.prev_deg[slot]);
+  c.walker = a.walker_base + (uint32_t)__builtin_amdgcn_readfirstlane(tt.walker[slot]);
+  c.step = (uint32_t)(__builtin_amdgcn_readfirstlane(tt.len[slot]) - 1);
   c.want = 0;
   return c;
 }
@@ -325,8 +359,6 @@ __device__ __forceinline__ void commit(const fw_kargs& a, TaskTable<kWGT>& tt, i
 template <int kApp, int kWGT>
 __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
   constexpr int kNW = kWGT / 64;
-  // quartets in flight per lane while streaming; node2vec is bound by its adjacency probes instead
-  constexpr int kUnroll = (kApp == FW_APP_NODE2VEC) ? 1 : FW_STREAM_UNROLL;
   __shared__ TaskTable<kWGT> tt;
 
   const int tid = (int)threadIdx.x;
@@ -359,15 +391,12 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
           const int slot = tt.hub_list[parity][hb + h];
           StepCtx c = load_ctx(a, tt, slot);
           if (kApp == FW_APP_METAPATH) c.want = a.schema[c.step % (uint32_t)a.schema_len];
-          float L, W;
+          float W;
           int32_t sel, selv;
-          uint32_t bern;
-          lane_pass<kApp, kWGT, false, kUnroll>(a, c, tid, L, sel, selv, bern);
-          const int win = wave_combine(L, bern, W);
-          const int32_t wsel = (win >= 0) ? __builtin_amdgcn_readlane(sel, win) : -1;
+          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, (uint32_t)wave, (uint32_t)kNW, W, sel, selv);
           if (lane == 0) {
             tt.hub_w[h][wave] = W;
-            tt.hub_sel[h][wave] = wsel;
+            tt.hub_sel[h][wave] = sel;
           }
         }
         __syncthreads();
@@ -376,17 +405,24 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
           const StepCtx c = load_ctx(a, tt, slot);
           float W = 0.0f;
           int32_t s = -1;
-          uint32_t bits = 0;
           if (lane < kNW) {
             W = tt.hub_w[h][lane];
             s = tt.hub_sel[h][lane];
-            bits = philox4x32_10(c.walker, c.step, kStreamWave | (uint32_t)lane, 0u, a.seed_lo, a.seed_hi).x;
           }
+          // inverse transform over the wave totals (lanes >= kNW hold 0 and never qualify)
           const float J = row_scan(W);
-          const bool acc = (lane < kNW) && (W > 0.0f) && (u24(bits) * J < W);
-          const uint64_t m = __ballot(acc);
+          const float total = readlane_f(J, kNW - 1);
+          const uint32_t bits = philox4x32_10(c.walker, c.step, kStreamWave, 0u, a.seed_lo, a.seed_hi).x;
+          const float target = u24(bits) * total;
+          const bool pos = W > 0.0f;
+          uint64_t m = __ballot(pos && J > target);
           int32_t pick = -1;
-          if (m != 0ull) pick = __builtin_amdgcn_readlane(s, 63 - __builtin_clzll(m));
+          if (m != 0ull) {
+            pick = __builtin_amdgcn_readlane(s, __builtin_ctzll(m));
+          } else {
+            m = __ballot(pos);
+            if (m != 0ull) pick = __builtin_amdgcn_readlane(s, 63 - __builtin_clzll(m));
+          }
           if (lane == 0) {
             int32_t v = -1;
             if (pick >= 0) v = a.adjncy[c.off + (uint32_t)pick];
@@ -405,25 +441,18 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
         const int slot = tt.small_list[parity][idx];
         StepCtx c = load_ctx(a, tt, slot);
         if (kApp == FW_APP_METAPATH) c.want = a.schema[c.step % (uint32_t)a.schema_len];
-        float L, W;
+        float W;
         int32_t sel, selv;
-        uint32_t bern;
         const uint32_t nq = ((c.off + (uint32_t)c.deg) - (c.off & ~3u) + 3u) >> 2;
-        int win;
         int32_t v = -1;
-        if (nq <= 64u) {  // one quartet per lane: fetch the adjacency with the weights, no dependent load
-          lane_pass<kApp, 64, true, 1>(a, c, lane, L, sel, selv, bern);
-          win = wave_combine(L, bern, W);
-          if (win >= 0) v = __builtin_amdgcn_readlane(selv, win);
+        if (nq <= 64u) {  // one quartet per lane: fetch the adjacency with the biases, no dependent load
+          wave_stream<kApp, 1, true>(a, c, lane, 0u, 1u, W, sel, selv);
+          v = selv;
         } else {
-          lane_pass<kApp, 64, false, kUnroll>(a, c, lane, L, sel, selv, bern);
-          win = wave_combine(L, bern, W);
-          if (win >= 0) {
-            const int32_t pick = __builtin_amdgcn_readlane(sel, win);
-            v = a.adjncy[c.off + (uint32_t)pick];
-          }
+          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, 0u, 1u, W, sel, selv);
+          if (sel >= 0) v = a.adjncy[c.off + (uint32_t)sel];
         }
-        if (lane == 0) commit(a, tt, slot, c, v, win >= 0, n_steps, n_edges);
+        if (lane == 0) commit(a, tt, slot, c, v, sel >= 0, n_steps, n_edges);
       }
       __syncthreads();
       if (tid == 0) {  // this round's lists are drained; they become the lists produced two rounds later
@@ -554,8 +583,10 @@ int launch_app(const fw_kargs& a, int wg_threads, int grid, hipStream_t stream, 
 
 int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, hipStream_t stream,
                    int* grid_used) {
-  if (sampler != FW_SAMPLER_ZPRS) {
-    fw_set_error("sampler %d is not available in this build", sampler);
+  // FW_SAMPLER_DPRS is an alias: the one sampler already evaluates every bias exactly once, which is
+  // what the reference's DPRS kernel (include/walker.cuh:1444) exists for.
+  if (sampler != FW_SAMPLER_ZPRS && sampler != FW_SAMPLER_DPRS) {
+    fw_set_error("unknown sampler %d", sampler);
     return FW_ERR_INVALID;
   }
   switch (app) {

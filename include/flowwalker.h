@@ -103,6 +103,9 @@ int fw_dev_free(void* d_ptr);
 int fw_dev_upload(void* d_dst, const void* h_src, size_t bytes);
 int fw_dev_download(void* h_dst, const void* d_src, size_t bytes);
 int fw_dev_fill_i32(int32_t* d_dst, int32_t value, size_t count);
+/* Plain device-to-device copy kernel (16-byte granularity); also the known-size kernel that HBM traffic
+ * counters are calibrated against. */
+int fw_dev_copy(void* d_dst, const void* d_src, size_t bytes);
 int fw_dev_sync(void);
 
 /* ---- graph ------------------------------------------------------------------------------------ */

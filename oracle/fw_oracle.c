@@ -14,12 +14,9 @@
  * What follows the reference, and where:
  *   - walk control flow (start write, step commit, dead end, stop, -1 padded rows):
  *       include/walker.cuh:1338-1350, :1357-1438; include/gpu_task.cuh:52-77
- *   - sampler: weighted reservoir sampling whose winner is "the last accepted element in
- *       lane-major order" over lane-strided elements, lane totals combined with a prefix scan and
- *       a max over accepted lanes: include/sampler.cuh:46-85 (warp), :87-127 (block);
- *       sequential ground truth include/sampler.cuh:26-44
- *   - DPRS (natural order, chunked inclusive scan, one Bernoulli per element):
- *       include/sampler.cuh:129-155, :157-200
+ *   - sampler: parallel weighted reservoir sampling over lane-strided elements with a prefix scan
+ *       over lane totals: include/sampler.cuh:46-85 (warp), :87-127 (block), chunk carry of
+ *       :129-155, :157-200; sequential ground truth include/sampler.cuh:26-44
  *   - bias functors and stop rules: include/app.cuh:58-71 (DeepWalk), :73-95 (PPR),
  *       :97-127 (node2vec), :129-152 (MetaPath); adjacency test include/gpu_graph.cuh:97-118
  *   - workload counters (steps, sum of source degrees): src/main.cu:82-113
@@ -28,21 +25,25 @@
  *   - RNG: Philox4x32-10 (Salmon et al., SC'11), keyed by the 64-bit seed, counter =
  *       (walker id, step, stream, block).  Replaces the stateful XORWOW of include/myrand.cuh.
  *       Pinned by the Random123 known-answer vectors (tests/golden/philox4x32_10_kat.json).
- *   - ZPRS is one pass: every lane runs a sequential reservoir over its own elements starting
- *       from 0 (not from the exclusive lane prefix), and lanes are then combined by one Bernoulli
- *       per lane against the inclusive lane prefix.  The law of the winner is unchanged
- *       (w_i / sum w); the second pass over the weights of include/sampler.cuh:70-80 disappears.
- *   - acceptance inside a lane uses the telescoping identity
+ *   - the sampler is one pass and evaluates every bias once.  The neighbour list is cut into groups
+ *       of FW_GROUP_QUARTETS * 64 quartets (1024 elements); each wave runs a sequential weighted
+ *       reservoir over the groups it owns, where "element" = a whole group with its total as weight
+ *       (the prefix / carry structure of include/sampler.cuh:139-152), and inside an accepted group
+ *       the element is picked by inverse transform on the same wave-scan prefix.  The law of the
+ *       winner is unchanged: P(i) = (T_g / sum T) * (w_i / T_g) = w_i / sum w.
+ *   - reservoir acceptance uses the telescoping identity
  *       P(no accept in (j,k]) = prod S_{i-1}/S_i = S_j/S_k,
- *       so one uniform u decides the NEXT accepted element (first k with S_k*u > S_j) instead of one
- *       uniform per element.  Same law as include/sampler.cuh:76, O(log n) draws per lane.
+ *       so one uniform u decides the NEXT accepted group (first k with S_k*u > S_j) instead of one
+ *       uniform per element (include/sampler.cuh:76).  O(log n) draws per step, all wave-uniform.
  *   - no division anywhere: tests are u*S < w-shaped products, never FMA-contracted.
  *   - uniforms are (x >> 8) * 2^-24 in [0,1), exact in f32.
  *   - elements are grouped in 4-element quartets aligned to the absolute CSR index (16-byte
- *       aligned vector loads on the GPU); quartet k of a list belongs to lane k mod P.
+ *       aligned vector loads on the GPU).
  *   - PPR stop draw is made once per completed step of a live walk, from its own stream
  *       (the reference also draws for empty slots, include/walker.cuh:1422-1431).
  *   - node2vec multiplies by host-computed f32 reciprocals 1/p and 1/q instead of dividing.
+ *   - --dprs selects nothing different: the one sampler already has DPRS's property (one bias
+ *       evaluation per neighbour, include/sampler.cuh:129-200), so FW_SAMPLER_DPRS is an alias.
  *
  * Build: make -C oracle   (gcc -O2 -ffp-contract=off -fopenmp)
  */
@@ -56,15 +57,15 @@
 
 #define FW_WAVE 64
 #define FW_QUAD 4
+#define FW_GROUP_QUARTETS 4 /* quartets per lane per group: a group spans 64 * 4 * 4 = 1024 elements */
 #define FW_MAX_SCHEMA 64
 #define FW_MAX_GROUP 1024
 
 enum { FW_APP_DEEPWALK = 0, FW_APP_PPR = 1, FW_APP_NODE2VEC = 2, FW_APP_METAPATH = 3 };
 enum { FW_SAMPLER_ZPRS = 0, FW_SAMPLER_DPRS = 1 };
 
-#define FW_STREAM_WAVE 0x40000000u /* | wave index : workgroup-level combine draws */
+#define FW_STREAM_WAVE 0x40000000u /* workgroup-level combine draw */
 #define FW_STREAM_STOP 0x80000000u /* PPR stop draw */
-#define FW_STREAM_DPRS 0xC0000000u /* DPRS: block index carries the element quartet */
 
 typedef struct {
   int32_t app;           /* FW_APP_* */
@@ -194,156 +195,102 @@ static float bias_at(const bias_ctx* c, uint64_t a) {
   }
 }
 
-/* ---- ZPRS: one-pass zero-preprocessing parallel reservoir sampler ---------------------------- */
+/* ---- one-pass zero-preprocessing parallel reservoir sampler ------------------------------------- */
+
+/* first i in [0,n) with v[i] > 0 and prefix[i] > target; if there is none, the last i with v[i] > 0
+ * (rounding in the prefix tree may leave no crossing); -1 when no v[i] is positive. */
+static int pick_by_prefix(const float* v, const float* prefix, int n, float target) {
+  int last = -1;
+  for (int i = 0; i < n; ++i) {
+    if (v[i] > 0.0f) {
+      if (prefix[i] > target) return i;
+      last = i;
+    }
+  }
+  return last;
+}
 
 /*
  * Samples one local index in [0,deg) with probability bias_i / sum(bias), or -1 when no bias is
- * positive.  P lanes (64 = wave, wg_threads = workgroup).  Follows the lane-strided / prefix /
- * max structure of include/sampler.cuh:46-127 with the one-pass and jump changes listed on top.
+ * positive.  nw waves of 64 lanes (1 = wave granularity, wg_threads / 64 = workgroup).
+ *
+ * Quartet k of the list (aligned to the absolute CSR index) belongs to group k / (64 * U), U =
+ * FW_GROUP_QUARTETS; inside group g, lane l owns quartets g*64*U + j*64 + l, j = 0..U-1.  Wave w owns
+ * groups w, w + nw, ...  For each owned group: lane totals q (sequential f32 adds in (j, element)
+ * order), wave scan I of q, group total T = I[63], running sum S += T; the group is accepted iff
+ * S * u > Sj.  On acceptance: target = draw * T; lane = pick_by_prefix(q, I); inside the lane the
+ * running sum starts at I[lane] - q[lane] and the element is pick_by_prefix again; then Sj = S and
+ * u = next draw.  Draws of wave w at (walker, step) are consecutive words of Philox stream w.
+ * Waves are combined by one more inverse transform on the row scan of the wave totals.
  */
-static int32_t zprs_sample(const bias_ctx* c, uint32_t off, int32_t deg, int P, uint32_t walker,
-                           uint32_t step) {
+static int32_t group_sample(const bias_ctx* c, uint32_t off, int32_t deg, int nw, uint32_t walker,
+                            uint32_t step) {
   if (deg <= 0) return -1;
+  enum { U = FW_GROUP_QUARTETS, EL = FW_GROUP_QUARTETS * FW_QUAD, G = FW_WAVE * FW_GROUP_QUARTETS };
   const uint64_t seed = c->p->seed;
   const uint64_t a0 = (uint64_t)off & ~(uint64_t)(FW_QUAD - 1);
   const uint64_t end = (uint64_t)off + (uint64_t)deg;
   const uint64_t nq = (end - a0 + FW_QUAD - 1) / FW_QUAD;
+  const uint64_t ngroups = (nq + G - 1) / G;
 
-  float L[FW_MAX_GROUP];
-  int32_t sel[FW_MAX_GROUP];
-
-  for (int t = 0; t < P; ++t) {
-    float S = 0.0f, Sj = 0.0f, u = 1.0f;
-    int32_t s = -1;
-    uint32_t ndraw = 0;
-    for (uint64_t k = (uint64_t)t; k < nq; k += (uint64_t)P) {
-      for (int j = 0; j < FW_QUAD; ++j) {
-        uint64_t a = a0 + FW_QUAD * k + j;
-        if (a < off || a >= end) continue;
-        float w = bias_at(c, a);
-        S = S + w;
-        float lhs = S * u;
-        if (lhs > Sj) {
-          s = (int32_t)(a - off);
-          Sj = S;
-          u = u24(draw_bits(seed, walker, step, (uint32_t)t, 1u + ndraw));
-          ++ndraw;
-        }
-      }
-    }
-    L[t] = S;
-    sel[t] = s;
-  }
-
-  const int nw = P / FW_WAVE;
   float W[16];
   int32_t wsel[16];
   for (int wv = 0; wv < nw; ++wv) {
-    float I[FW_WAVE];
-    for (int l = 0; l < FW_WAVE; ++l) I[l] = L[wv * FW_WAVE + l];
-    fw_oracle_wave_scan(I);
-    int32_t pick = -1;
-    for (int l = 0; l < FW_WAVE; ++l) {
-      int t = wv * FW_WAVE + l;
-      if (L[t] > 0.0f) {
-        float ub = u24(draw_bits(seed, walker, step, (uint32_t)t, 0u));
-        float lhs = ub * I[l];
-        if (lhs < L[t]) pick = sel[t];
+    float S = 0.0f, Sj = 0.0f, u = 1.0f;
+    int32_t sel = -1;
+    uint32_t nd = 0;
+    for (uint64_t g = (uint64_t)wv; g < ngroups; g += (uint64_t)nw) {
+      float x[FW_WAVE][EL];
+      float q[FW_WAVE], I[FW_WAVE];
+      for (int l = 0; l < FW_WAVE; ++l) {
+        float s = 0.0f;
+        for (int j = 0; j < U; ++j) {
+          const uint64_t k = g * G + (uint64_t)j * FW_WAVE + (uint64_t)l;
+          for (int e = 0; e < FW_QUAD; ++e) {
+            const uint64_t a = a0 + FW_QUAD * k + (uint64_t)e;
+            const float b = (k < nq && a >= off && a < end) ? bias_at(c, a) : 0.0f;
+            x[l][j * FW_QUAD + e] = b;
+            s = s + b;
+          }
+        }
+        q[l] = s;
+        I[l] = s;
       }
+      fw_oracle_wave_scan(I);
+      const float T = I[FW_WAVE - 1];
+      const float Snew = S + T;
+      const float lhs = Snew * u;
+      if (lhs > Sj) {
+        const float u2 = u24(draw_bits(seed, walker, step, (uint32_t)wv, nd++));
+        const float target = u2 * T;
+        const int lane = pick_by_prefix(q, I, FW_WAVE, target);
+        /* lane >= 0: acceptance implies T > 0, hence some q > 0 */
+        float pre[EL];
+        float e = I[lane] - q[lane];
+        for (int i = 0; i < EL; ++i) {
+          e = e + x[lane][i];
+          pre[i] = e;
+        }
+        const int pick = pick_by_prefix(x[lane], pre, EL, target);
+        const uint64_t k = g * G + (uint64_t)(pick / FW_QUAD) * FW_WAVE + (uint64_t)lane;
+        sel = (int32_t)(a0 + FW_QUAD * k + (uint64_t)(pick % FW_QUAD) - off);
+        Sj = Snew;
+        u = u24(draw_bits(seed, walker, step, (uint32_t)wv, nd++));
+      }
+      S = Snew;
     }
-    W[wv] = I[FW_WAVE - 1];
-    wsel[wv] = pick;
+    W[wv] = S;
+    wsel[wv] = sel;
   }
   if (nw == 1) return wsel[0];
 
   float J[16];
   for (int wv = 0; wv < nw; ++wv) J[wv] = W[wv];
   row_scan(J, nw);
-  int32_t pick = -1;
-  for (int wv = 0; wv < nw; ++wv) {
-    if (W[wv] > 0.0f) {
-      float ub = u24(draw_bits(seed, walker, step, FW_STREAM_WAVE | (uint32_t)wv, 0u));
-      float lhs = ub * J[wv];
-      if (lhs < W[wv]) pick = wsel[wv];
-    }
-  }
-  return pick;
-}
-
-/* ---- DPRS: natural order, chunked inclusive scan, one Bernoulli per element ------------------ */
-
-/*
- * include/sampler.cuh:129-200.  Chunks of P*4 elements (one quartet per lane), running sum carried
- * between chunks; element i is accepted iff bias_i > 0 and u_i * S_i < bias_i; the winner is the
- * largest accepted index.  u_i is word (a & 3) of Philox block (a - a0) / 4 of stream FW_STREAM_DPRS.
- * Within a chunk: lane-local 4-element running sums, wave scan of lane totals, row scan of wave
- * totals, then S_i = carry + (waves before) + (lanes before) + local running sum.
- */
-static int32_t dprs_sample(const bias_ctx* c, uint32_t off, int32_t deg, int P, uint32_t walker,
-                           uint32_t step) {
-  if (deg <= 0) return -1;
-  const uint64_t seed = c->p->seed;
-  const uint64_t a0 = (uint64_t)off & ~(uint64_t)(FW_QUAD - 1);
-  const uint64_t end = (uint64_t)off + (uint64_t)deg;
-  const uint64_t nq = (end - a0 + FW_QUAD - 1) / FW_QUAD;
-  const int nw = P / FW_WAVE;
-  float carry = 0.0f;
-  int32_t pick = -1;
-  for (uint64_t base = 0; base < nq; base += (uint64_t)P) {
-    float w[FW_MAX_GROUP][FW_QUAD];
-    float lane_tot[FW_MAX_GROUP];
-    for (int t = 0; t < P; ++t) {
-      uint64_t k = base + (uint64_t)t;
-      float s = 0.0f;
-      for (int j = 0; j < FW_QUAD; ++j) {
-        uint64_t a = a0 + FW_QUAD * k + j;
-        float x = (k < nq && a >= off && a < end) ? bias_at(c, a) : 0.0f;
-        w[t][j] = x;
-        s = s + x;
-      }
-      lane_tot[t] = s;
-    }
-    float wave_tot[16];
-    float incl[FW_MAX_GROUP];
-    for (int wv = 0; wv < nw; ++wv) {
-      float I[FW_WAVE];
-      for (int l = 0; l < FW_WAVE; ++l) I[l] = lane_tot[wv * FW_WAVE + l];
-      fw_oracle_wave_scan(I);
-      for (int l = 0; l < FW_WAVE; ++l) incl[wv * FW_WAVE + l] = I[l];
-      wave_tot[wv] = I[FW_WAVE - 1];
-    }
-    float J[16];
-    for (int wv = 0; wv < nw; ++wv) J[wv] = wave_tot[wv];
-    if (nw > 1) row_scan(J, nw);
-    for (int t = 0; t < P; ++t) {
-      uint64_t k = base + (uint64_t)t;
-      if (k >= nq) break;
-      int wv = t / FW_WAVE, l = t % FW_WAVE;
-      /* exclusive prefix of this lane inside the chunk */
-      float before = carry;
-      if (wv > 0) before = before + J[wv - 1];
-      if (l > 0) before = before + incl[t - 1];
-      uint32_t ctr[4] = {walker, step, FW_STREAM_DPRS, (uint32_t)k};
-      uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
-      uint32_t r[4];
-      fw_oracle_philox4x32_10(ctr, key, r);
-      float S = before;
-      for (int j = 0; j < FW_QUAD; ++j) {
-        uint64_t a = a0 + FW_QUAD * k + j;
-        float x = w[t][j];
-        S = S + x;
-        if (x > 0.0f) {
-          float lhs = u24(r[j]) * S;
-          if (lhs < x) {
-            int32_t i = (int32_t)(a - off);
-            if (i > pick) pick = i;
-          }
-        }
-      }
-    }
-    carry = carry + J[nw > 1 ? nw - 1 : 0];
-  }
-  return pick;
+  const float u3 = u24(draw_bits(seed, walker, step, FW_STREAM_WAVE, 0u));
+  const float target = u3 * J[nw - 1];
+  const int wv = pick_by_prefix(W, J, nw, target);
+  return wv < 0 ? -1 : wsel[wv];
 }
 
 /* One sampling step, exposed for sampler-level tests.  Granularity by degree as in
@@ -357,9 +304,8 @@ int32_t fw_oracle_sample(const fw_oracle_graph* g, const fw_oracle_params* p, in
   c.want_label = (p->app == FW_APP_METAPATH && p->schema_len > 0) ? p->schema[step % (uint32_t)p->schema_len] : 0;
   uint32_t off = g->xadj[cur];
   int32_t deg = (int32_t)(g->xadj[cur + 1] - off);
-  int P = (deg > p->hub_threshold) ? p->wg_threads : FW_WAVE;
-  return p->sampler == FW_SAMPLER_DPRS ? dprs_sample(&c, off, deg, P, walker, step)
-                                       : zprs_sample(&c, off, deg, P, walker, step);
+  const int nw = (deg > p->hub_threshold) ? p->wg_threads / FW_WAVE : 1;
+  return group_sample(&c, off, deg, nw, walker, step);
 }
 
 /* ---- whole walks (include/walker.cuh:1338-1438) --------------------------------------------- */
