@@ -27,7 +27,7 @@ EXPORTED = [
     "fw_dev_alloc", "fw_dev_free", "fw_dev_upload", "fw_dev_download", "fw_dev_fill_i32", "fw_dev_copy", "fw_dev_sync",
     "fw_graph_create", "fw_graph_adopt_device", "fw_graph_destroy", "fw_graph_info", "fw_graph_is_sorted",
     "fw_graph_download", "fw_walk_device", "fw_walk_batch", "fw_host_alloc_pinned", "fw_host_free_pinned",
-    "fw_gen_rmat",
+    "fw_gen_rmat", "fw_csr_read_header", "fw_csr_load", "fw_csr_write", "fw_graph_load",
 ]
 
 
@@ -100,6 +100,10 @@ def lib():
         L.fw_host_alloc_pinned.argtypes = [C.c_size_t, C.POINTER(C.c_void_p)]
         L.fw_host_free_pinned.argtypes = [C.c_void_p]
         L.fw_gen_rmat.argtypes = [C.POINTER(RmatParams), C.POINTER(C.c_void_p)]
+        L.fw_csr_read_header.argtypes = [C.c_char_p, C.POINTER(C.c_int32), C.POINTER(C.c_uint64)]
+        L.fw_csr_load.argtypes = [C.c_char_p, C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.fw_csr_write.argtypes = [C.c_char_p, C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.fw_graph_load.argtypes = [C.c_char_p, C.c_int, C.c_int, C.POINTER(C.c_void_p)]
         _lib = L
     return _lib
 
@@ -142,6 +146,27 @@ def set_params(params, /, **kw):
 
 def _ptr(arr):
     return None if arr is None else arr.ctypes.data_as(C.c_void_p)
+
+
+def csr_read(prefix, weights=True, labels=False):
+    """Reads <prefix>_xadj/_edge/_weight/_label.bin (host side only).  Returns (xadj, adjncy, weight, label)."""
+    V, E = C.c_int32(), C.c_uint64()
+    check(lib().fw_csr_read_header(prefix.encode(), C.byref(V), C.byref(E)))
+    xadj = np.empty(V.value + 1, dtype=np.uint32)
+    adjncy = np.empty(E.value, dtype=np.int32)
+    weight = np.empty(E.value, dtype=np.float32) if weights else None
+    label = np.empty(E.value, dtype=np.int32) if labels else None
+    check(lib().fw_csr_load(prefix.encode(), V.value, E.value, _ptr(xadj), _ptr(adjncy), _ptr(weight), _ptr(label)))
+    return xadj, adjncy, weight, label
+
+
+def csr_write(prefix, xadj, adjncy, weight=None, label=None):
+    xadj = np.ascontiguousarray(xadj, dtype=np.uint32)
+    adjncy = np.ascontiguousarray(adjncy, dtype=np.int32)
+    weight = None if weight is None else np.ascontiguousarray(weight, dtype=np.float32)
+    label = None if label is None else np.ascontiguousarray(label, dtype=np.int32)
+    check(lib().fw_csr_write(prefix.encode(), len(xadj) - 1, len(adjncy), _ptr(xadj), _ptr(adjncy), _ptr(weight),
+                             _ptr(label)))
 
 
 class DeviceBuffer:
@@ -196,6 +221,12 @@ class Graph:
         h = C.c_void_p()
         check(lib().fw_graph_create(len(xadj) - 1, len(adjncy), _ptr(xadj), _ptr(adjncy), _ptr(weight), _ptr(label),
                                     C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def load(cls, prefix, weights=True, labels=False):
+        h = C.c_void_p()
+        check(lib().fw_graph_load(prefix.encode(), int(weights), int(labels), C.byref(h)))
         return cls(h)
 
     @classmethod

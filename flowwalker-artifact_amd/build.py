@@ -28,8 +28,8 @@ HIP_FLAGS = [
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
 ]
 
-KERNEL_SOURCES = ["fw_walk_kernel.hip", "fw_api.hip", "fw_gen.hip"]
-HOST_TOOLS = {"flowwalker": ["flowwalker_main.cpp", "csr_io.cpp"], "fw_gen": ["fw_gen_main.cpp", "csr_io.cpp"]}
+KERNEL_SOURCES = ["fw_walk_kernel.hip", "fw_api.hip", "fw_gen.hip", "fw_csr_io.hip"]
+HOST_TOOLS = {"flowwalker": ["flowwalker_main.cpp"], "fw_gen": ["fw_gen_main.cpp"]}
 
 
 def _run(cmd):
@@ -51,7 +51,7 @@ def build_library():
         src, obj = pair
         _run([HIPCC] + HIP_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
 
-    with ThreadPoolExecutor(max_workers=3) as ex:
+    with ThreadPoolExecutor(max_workers=4) as ex:
         list(ex.map(compile_one, zip(KERNEL_SOURCES, objs)))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
     return LIB

@@ -138,6 +138,24 @@ int fw_graph_is_sorted(const fw_graph* g, int* sorted);
 /* Copies the device CSR back (any output pointer may be NULL). */
 int fw_graph_download(const fw_graph* g, uint32_t* h_xadj, int32_t* h_adjncy, float* h_weight, int32_t* h_label);
 
+/* ---- on-disk CSR: <prefix>_xadj.bin / _edge.bin / _weight.bin / _label.bin ---------------------- */
+
+/*
+ * Replaces graph::load_graph (include/graph.cuh:93-190); the layout is the one
+ * data/EdgeListToCSR.cpp:216-251 writes: _xadj.bin = int32 V, uint32 E, uint32 xadj[V+1]; _edge.bin =
+ * int32 adjncy[E]; _weight.bin = float32[E]; _label.bin = int32[E].  The reference's asserts
+ * (:113, :119, :135-136, :155, :176) become FW_ERR_IO with a message.
+ */
+int fw_csr_read_header(const char* prefix, int32_t* V, uint64_t* E);
+/* Reads into caller-owned arrays sized from the header; h_weight / h_label may be NULL (not read). */
+int fw_csr_load(const char* prefix, int32_t V, uint64_t E, uint32_t* h_xadj, int32_t* h_adjncy, float* h_weight,
+                int32_t* h_label);
+/* Writes the four files (weight / label only when given). */
+int fw_csr_write(const char* prefix, int32_t V, uint64_t E, const uint32_t* h_xadj, const int32_t* h_adjncy,
+                 const float* h_weight, const int32_t* h_label);
+/* load + fw_graph_create: graph::graph(...) followed by gpu_graph::gpu_graph(graph*) (src/main.cu:312-325). */
+int fw_graph_load(const char* prefix, int want_weight, int want_label, fw_graph** out);
+
 /* ---- walks ------------------------------------------------------------------------------------ */
 
 /*

@@ -1,0 +1,83 @@
+"""The flowwalker command-line front end end to end on the GPU: same flags as the reference, walk paths equal
+to the oracle's, printed report in the reference's format."""
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import _graphs
+import fw_oracle_binding as orc
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CLI = os.path.join(ROOT, "flowwalker-artifact_amd", "bin", "flowwalker")
+
+
+def _run(*args):
+    r = subprocess.run([CLI] + list(args), stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    return r.stdout
+
+
+@pytest.fixture(scope="module")
+def graph_files(gpu, tmp_path_factory):
+    d = tmp_path_factory.mktemp("g")
+    xadj, adj, w, lab = _graphs.hub_graph(V=7115, hub_degrees=(3000,), base_degree=7, seed=1, w_hi=5.0)
+    prefix = str(d / "hub")
+    gpu.csr_write(prefix, xadj, adj, w, lab)
+    return prefix, (xadj, adj, w, lab)
+
+
+def test_deepwalk_n100_print(gpu, graph_files, tmp_path):
+    prefix, csr = graph_files
+    out = str(tmp_path / "paths.bin")
+    text = _run("--input", prefix, "--deepwalk", "--n=100", "--seq", "--seed=5", "--printresult", "--printworkload",
+                "--savepaths", out)
+    paths = np.fromfile(out, dtype=np.int32).reshape(100, 81)
+    ref, steps, edges = orc.walk(orc.Graph(*csr), orc.make_params(max_depth=81, seed=5), np.arange(100, dtype=np.int32))
+    assert (paths == ref).all()
+    assert "Vertex count:7115 Expected edge count: %d" % len(csr[1]) in text
+    assert "Read Graph!" in text and re.search(r"Max degree: \d+, idx: 0", text)
+    assert "grid:" in text and "sampling time:" in text
+    assert text.count("Walker ") == 100                                          # src/main.cu:165
+    row0 = re.search(r"Walker 0:\n([^\n]*)\nTotal length=(\d+)", text)
+    assert [int(t) for t in row0.group(1).split()] == ref[0][ref[0] >= 0].tolist()
+    assert int(row0.group(2)) == int((ref[0] >= 0).sum())
+    assert "Total sampled vertex: %d" % steps in text                            # src/main.cu:109-111
+    assert "Total sampled edge: %d," % edges in text
+
+
+def test_all_batch_modes_agree(gpu, graph_files, tmp_path):
+    prefix, csr = graph_files
+    V = len(csr[0]) - 1
+    ref, _, _ = orc.walk(orc.Graph(*csr), orc.make_params(app=2, max_depth=21, seed=1337), np.arange(V, dtype=np.int32))
+    for i, extra in enumerate((["--all"], ["--all", "--syn"], ["--n=%d" % V, "--seq", "--batch", "--batchsize=1000"],
+                               ["--n=%d" % V, "--seq", "--dprs"])):
+        out = str(tmp_path / ("p%d.bin" % i))
+        text = _run("--input", prefix, "--node2vec", "--d=20", "--p=2.0", "--q=0.5", "--savepaths", out, *extra)
+        assert (np.fromfile(out, dtype=np.int32).reshape(V, 21) == ref).all(), extra
+        if "--all" in extra:
+            assert "batch size=%d" % V in text                                   # src/main.cu:270
+
+
+def test_metapath_and_ppr(gpu, graph_files, tmp_path):
+    prefix, csr = graph_files
+    xadj, adj, w, lab = csr
+    out = str(tmp_path / "m.bin")
+    text = _run("--input", prefix, "--metapath", "--schema=2,0,1", "--n=50", "--seq", "--printresult", "--savepaths", out)
+    assert "schema len=3" in text
+    ref, _, _ = orc.walk(orc.Graph(xadj, adj, None, lab), orc.make_params(app=3, max_depth=4, schema=[2, 0, 1], seed=1337),
+                         np.arange(50, dtype=np.int32))
+    assert (np.fromfile(out, dtype=np.int32).reshape(50, 4) == ref).all()
+    assert text.count("Walker ") == 50 and re.search(r"\[2\]\t\d+\t", text)       # labels printed before each hop
+    # --ppr starts every query from the max-degree vertex (src/main.cu:277-281); --pprstart=seq from 0..n-1
+    out = str(tmp_path / "p.bin")
+    _run("--input", prefix, "--ppr", "--n=300", "--tp=0.3", "--savepaths", out)
+    got = np.fromfile(out, dtype=np.int32).reshape(300, 81)
+    assert (got[:, 0] == 0).all()
+    ref, _, _ = orc.walk(orc.Graph(*csr), orc.make_params(app=1, max_depth=81, tp=0.3, seed=1337), np.zeros(300, dtype=np.int32))
+    assert (got == ref).all()
+    _run("--input", prefix, "--ppr", "--n=300", "--seq", "--pprstart=seq", "--savepaths", out)
+    assert (np.fromfile(out, dtype=np.int32).reshape(300, 81)[:, 0] == np.arange(300)).all()
