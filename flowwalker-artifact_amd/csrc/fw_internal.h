@@ -38,6 +38,7 @@ struct fw_kargs {
   int32_t n;
   int32_t max_depth;
   int32_t hub_threshold;
+  int32_t slot_limit;           // task slots a workgroup may fill (small batches are spread over the grid)
   uint32_t seed_lo, seed_hi;
   uint32_t walker_base;
   float tp, inv_p, inv_q;

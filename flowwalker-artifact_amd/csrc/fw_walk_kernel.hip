@@ -468,7 +468,7 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
       const int np = first ? 0 : parity;  // lists to fill for the next round
       first = false;
       int32_t len = tt.len[tid];
-      bool need = true;  // slot wants a new query
+      bool need = tid < a.slot_limit;  // slot wants a new query
       int32_t deg = 0;
       if (len >= 0) {
         if (tt.flag[tid] == kFlagMoved) {
@@ -524,7 +524,7 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
           }
         }
       }
-      if (need) {
+      if (need || len < 0) {  // nothing to run in this slot (finished / never filled / beyond slot_limit)
         tt.len[tid] = -1;
       } else {
         tt.len[tid] = len;
@@ -547,7 +547,7 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
 }
 
 template <int kApp, int kWGT>
-int launch_one(const fw_kargs& a, int grid, hipStream_t stream, int* grid_used) {
+int launch_one(fw_kargs a, int grid, hipStream_t stream, int* grid_used) {
   if (grid <= 0) {
     int dev = 0;
     hipDeviceProp_t prop;
@@ -558,9 +558,11 @@ int launch_one(const fw_kargs& a, int grid, hipStream_t stream, int* grid_used) 
     if (per_cu < 1) per_cu = 1;
     grid = prop.multiProcessorCount * per_cu;
   }
-  // no more workgroups than there are slots to fill
-  const long long max_useful = ((long long)a.n + kWGT - 1) / kWGT;
-  if ((long long)grid > max_useful) grid = (int)(max_useful > 0 ? max_useful : 1);
+  // a small batch is spread over the grid (down to one query per workgroup) instead of filling the
+  // task table of a few workgroups: fewer slots per workgroup, same persistent grid
+  if (grid > a.n) grid = a.n;
+  const long long per_wg = ((long long)a.n + grid - 1) / grid;
+  a.slot_limit = (int32_t)(per_wg < kWGT ? per_wg : kWGT);
   hipLaunchKernelGGL((fw_walk_zprs<kApp, kWGT>), dim3(grid), dim3(kWGT), 0, stream, a);
   FW_HIP(hipGetLastError());
   if (grid_used) *grid_used = grid;
