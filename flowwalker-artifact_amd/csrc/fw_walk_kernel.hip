@@ -110,23 +110,134 @@ struct StepCtx {
   uint32_t step;
 };
 
-// include/gpu_graph.cuh:97-112
-__device__ __forceinline__ bool sorted_contains(const int32_t* __restrict__ arr, int32_t size, int32_t target) {
-  int32_t lo = 0, hi = size;
-  while (lo < hi) {
-    const int32_t mid = (int32_t)(((uint32_t)lo + (uint32_t)hi) >> 1);
-    const int32_t v = arr[mid];
-    if (v == target) return true;
-    if (v < target) lo = mid + 1; else hi = mid;
-  }
-  return false;
+// ---- node2vec adjacency test (include/gpu_graph.cuh:97-118) -----------------------------------------
+// The reference binary-searches the whole list of prev for every neighbour of cur.  Both lists are
+// ascending, so here (1) one wave-cooperative 64-ary search per group bounds the part of N(prev) that can
+// hold the group's vertices, and (2) every lane gallops forward from the position of its previous
+// neighbour.  The answers (is post in N(prev)?) are the same.
+
+// max over the wave of a per-lane int (INT_MIN where a lane has nothing), result in every lane
+__device__ __forceinline__ int32_t wave_max_i32(int32_t v) {
+  constexpr int kMin = (int)0x80000000;
+  v = max(v, __builtin_amdgcn_update_dpp(kMin, v, 0x111, 0xF, 0xF, false));
+  v = max(v, __builtin_amdgcn_update_dpp(kMin, v, 0x112, 0xF, 0xF, false));
+  v = max(v, __builtin_amdgcn_update_dpp(kMin, v, 0x114, 0xF, 0xF, false));
+  v = max(v, __builtin_amdgcn_update_dpp(kMin, v, 0x118, 0xF, 0xF, false));
+  v = max(v, __builtin_amdgcn_update_dpp(kMin, v, 0x142, 0xA, 0xF, false));
+  v = max(v, __builtin_amdgcn_update_dpp(kMin, v, 0x143, 0xC, 0xF, false));
+  return __builtin_amdgcn_readlane(v, 63);
 }
 
-// node2vec bias of one neighbour (include/app.cuh:108-123).  Entries outside the list arrive with
-// post == prev and weight 0, so they are never searched for.
-__device__ __forceinline__ float n2v_bias(const fw_kargs& a, const StepCtx& c, float w, int32_t post) {
-  if (post == c.prev) return w * a.inv_p;
-  return sorted_contains(a.adjncy + c.prev_off, c.prev_deg, post) ? w : w * a.inv_q;
+// number of entries of arr[lo, hi) that are <= x, plus lo; all 64 lanes probe one split point per round
+__device__ __forceinline__ uint32_t coop_upper_bound(const int32_t* __restrict__ arr, uint32_t lo, uint32_t hi,
+                                                     int32_t x, int lane) {
+  while (hi - lo > 64u) {
+    const uint32_t chunk = (hi - lo + 63u) >> 6;
+    uint32_t idx = lo + ((uint32_t)lane + 1u) * chunk - 1u;  // last entry of this lane's chunk
+    idx = idx < hi ? idx : hi - 1u;
+    const uint32_t cnt = (uint32_t)__builtin_popcountll(__ballot(arr[idx] <= x));
+    if (cnt == 64u) return hi;
+    const uint32_t nlo = lo + cnt * chunk;           // chunks before `cnt` are all <= x
+    const uint32_t nhi = lo + (cnt + 1u) * chunk - 1u;  // the last entry of chunk `cnt` is > x
+    lo = nlo;
+    hi = nhi < hi ? nhi : hi - 1u;
+  }
+  const uint32_t i = lo + (uint32_t)lane;
+  const bool le = i < hi && arr[i] <= x;
+  return lo + (uint32_t)__builtin_popcountll(__ballot(le));
+}
+
+// first index in [lo, hi) with arr[index] >= x (hi if none), galloping from lo
+__device__ __forceinline__ uint32_t gallop_lower_bound(const int32_t* __restrict__ arr, uint32_t lo, uint32_t hi,
+                                                       int32_t x) {
+  uint32_t a = lo, b = lo, step = 1u;
+  while (b < hi && arr[b] < x) {
+    a = b + 1u;
+    b = a + step - 1u;
+    step <<= 1;
+  }
+  uint32_t r = b < hi ? b : hi;
+  while (a < r) {
+    const uint32_t mid = (a + r) >> 1;
+    if (arr[mid] < x) a = mid + 1u; else r = mid;
+  }
+  return a;
+}
+
+// first index in [lo, hi) with arr[index] >= x (hi if none); all 64 lanes probe one split point per round
+__device__ __forceinline__ uint32_t coop_lower_bound(const int32_t* __restrict__ arr, uint32_t lo, uint32_t hi,
+                                                     int32_t x, int lane) {
+  while (hi - lo > 64u) {
+    const uint32_t chunk = (hi - lo + 63u) >> 6;
+    uint32_t idx = lo + ((uint32_t)lane + 1u) * chunk - 1u;
+    idx = idx < hi ? idx : hi - 1u;
+    const uint32_t cnt = (uint32_t)__builtin_popcountll(__ballot(arr[idx] < x));
+    if (cnt == 64u) return hi;
+    const uint32_t nlo = lo + cnt * chunk;
+    const uint32_t nhi = lo + (cnt + 1u) * chunk - 1u;
+    lo = nlo;
+    hi = nhi < hi ? nhi : hi - 1u;
+  }
+  const uint32_t i = lo + (uint32_t)lane;
+  const bool lt = i < hi && arr[i] < x;
+  return lo + (uint32_t)__builtin_popcountll(__ballot(lt));
+}
+
+// Per-wave LDS scratch of the reversed adjacency test (entries of N(prev) looked up in N(cur)).
+constexpr int kN2vChunk = 256;  // entries of N(prev) resolved per refill: 4 per lane
+struct N2vScratch {
+  int32_t match[kN2vChunk];  // local indices in N(cur) of common neighbours, ascending
+  uint32_t mask[64];         // per lane: bit i set = the lane's i-th bias of the current group is a common neighbour
+};
+
+// Wave-uniform cursor of the reversed test.
+struct N2vCursor {
+  uint32_t pc = 0;      // entries of N(prev) before this index are resolved
+  uint32_t cov = 0;     // local indices of N(cur) below this are resolved (all their matches are recorded)
+  uint32_t mcount = 0;  // matches in the buffer
+  uint32_t mpos = 0;    // matches already applied
+};
+
+// Resolves the next kN2vChunk entries of N(prev): each lane looks its 4 consecutive entries up in N(cur)
+// (galloping from the resolved prefix) and the hits are written to scr.match in ascending order.
+__device__ __forceinline__ void n2v_refill(const int32_t* __restrict__ clist, uint32_t dc,
+                                           const int32_t* __restrict__ plist, uint32_t dp, N2vScratch& scr,
+                                           N2vCursor& k, int lane) {
+  const uint32_t cnt = (dp - k.pc) < (uint32_t)kN2vChunk ? (dp - k.pc) : (uint32_t)kN2vChunk;
+  const uint32_t base = k.pc + 4u * (uint32_t)lane;
+  uint32_t pos = k.cov;
+  uint32_t hit_pos[4];
+  bool hit[4];
+  uint32_t resolved = k.cov;  // after this lane's last entry: indices below are resolved
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    hit[e] = false;
+    hit_pos[e] = 0u;
+    if (base + (uint32_t)e < k.pc + cnt) {
+      const int32_t y = plist[base + (uint32_t)e];
+      pos = gallop_lower_bound(clist, pos, dc, y);
+      hit[e] = pos < dc && clist[pos] == y;
+      hit_pos[e] = pos;
+      resolved = pos + (hit[e] ? 1u : 0u);
+    }
+  }
+  const uint64_t m0 = __ballot(hit[0]), m1 = __ballot(hit[1]), m2 = __ballot(hit[2]), m3 = __ballot(hit[3]);
+  const uint64_t below = (1ull << lane) - 1ull;
+  uint32_t at = (uint32_t)(__builtin_popcountll(m0 & below) + __builtin_popcountll(m1 & below) +
+                           __builtin_popcountll(m2 & below) + __builtin_popcountll(m3 & below));
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (hit[e]) scr.match[at++] = (int32_t)hit_pos[e];
+  }
+  k.mcount = (uint32_t)(__builtin_popcountll(m0) + __builtin_popcountll(m1) + __builtin_popcountll(m2) +
+                        __builtin_popcountll(m3));
+  k.mpos = 0u;
+  k.pc += cnt;
+  const uint32_t last_lane = (cnt - 1u) >> 2;
+  const uint32_t cov = (uint32_t)__builtin_amdgcn_readlane((int)resolved, (int)last_lane);
+  k.cov = k.pc >= dp ? dc : cov;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
 }
 
 // Wave-uniform queue of Philox words: draw n of a stream is word n & 3 of block n >> 2.
@@ -155,7 +266,8 @@ __device__ __forceinline__ float next_uniform(DrawQueue& d, const fw_kargs& a, c
 // vertex.  Outputs: running total S of the wave's groups, selected local index (or -1), its vertex.
 template <int kApp, int kJ, bool kTrackV>
 __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c, const int lane, const uint32_t w,
-                                            const uint32_t nw, float& S_out, int32_t& sel_out, int32_t& selv_out) {
+                                            const uint32_t nw, N2vScratch* scr, float& S_out, int32_t& sel_out,
+                                            int32_t& selv_out) {
   constexpr uint32_t kG = 64u * kGroupQuartets;  // quartets per group
   constexpr int kEl = 4 * kJ;
   const uint32_t a0 = c.off & ~3u;
@@ -165,11 +277,21 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
   const uint32_t* __restrict__ bias =
       reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
   const bool n2v = kApp == FW_APP_NODE2VEC && c.prev != -1;
-  const bool need_adj = kTrackV || n2v;
+  // reversed adjacency test: look the entries of the shorter list N(prev) up in N(cur) (wave granularity only)
+  const bool reversed = n2v && nw == 1u && c.prev_deg <= c.deg;
+  const bool need_adj = kTrackV || (n2v && !reversed);
+  N2vCursor cur;
+  int32_t ret_idx = -1;  // local index of prev in N(cur): the return edge (include/app.cuh:113-114)
+  if (kApp == FW_APP_NODE2VEC && reversed) {
+    const int32_t* __restrict__ clist = a.adjncy + c.off;
+    const uint32_t r = coop_lower_bound(clist, 0u, (uint32_t)c.deg, c.prev, lane);
+    if (r < (uint32_t)c.deg && clist[r] == c.prev) ret_idx = (int32_t)r;
+  }
 
   float S = 0.0f, Sj = 0.0f, u = 1.0f;
   int32_t sel = -1, selv = -1;
   DrawQueue dq;
+  uint32_t seg_lo = 0u;  // node2vec: entries of N(prev) below this index are smaller than anything still to come
 
   for (uint32_t g = w; g < ngroups; g += nw) {
     const uint32_t kb = g * kG + (uint32_t)lane;  // this lane's quartet for j = 0
@@ -232,14 +354,79 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
         }
       }
     }
-    if (n2v) {
+    if (kApp == FW_APP_NODE2VEC && reversed) {
+      // include/app.cuh:108-123 with the roles of the two lists swapped: every bias becomes w/q except the
+      // common neighbours recorded in scr->match (w) and the return edge (w/p)
+      const int32_t* __restrict__ clist = a.adjncy + c.off;
+      const int32_t* __restrict__ plist = a.adjncy + c.prev_off;
+      const int32_t gs = (int32_t)(a0 + 4u * g * kG - c.off);  // local index of the group's first slot
+      const int32_t ge = gs + (int32_t)(4u * kG);
+      const uint32_t need = (uint32_t)ge < (uint32_t)c.deg ? (uint32_t)ge : (uint32_t)c.deg;
+      scr->mask[lane] = 0u;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      for (;;) {
+        while (cur.mpos < cur.mcount) {  // 64 buffered matches at a time
+          const uint32_t i = cur.mpos + (uint32_t)lane;
+          const int32_t p = i < cur.mcount ? scr->match[i] : 0x7FFFFFFF;
+          const bool in = p < ge;
+          if (in) {
+            const uint32_t rel = (uint32_t)(p - gs);
+            const uint32_t qd = rel >> 2;
+            atomicOr(&scr->mask[qd & 63u], 1u << (((qd >> 6) << 2) | (rel & 3u)));
+          }
+          const uint32_t nin = (uint32_t)__builtin_popcountll(__ballot(in));
+          cur.mpos += nin;
+          if (nin < 64u) break;
+        }
+        if (cur.cov >= need) break;  // every index of this group is resolved
+        n2v_refill(clist, (uint32_t)c.deg, plist, (uint32_t)c.prev_deg, *scr, cur, lane);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      const uint32_t common = scr->mask[lane];
+      int ret_slot = -1;  // which of this lane's biases is the return edge
+      if (ret_idx >= gs && ret_idx < ge) {
+        const uint32_t rel = (uint32_t)(ret_idx - gs);
+        const uint32_t qd = rel >> 2;
+        if ((int)(qd & 63u) == lane) ret_slot = (int)(((qd >> 6) << 2) | (rel & 3u));
+      }
+#pragma unroll
+      for (int i = 0; i < kEl; ++i) {
+        const float wq = x[i] * a.inv_q;
+        const float wp = x[i] * a.inv_p;
+        x[i] = (i == ret_slot) ? wp : (((common >> i) & 1u) ? x[i] : wq);
+      }
+    } else if (n2v) {  // include/app.cuh:108-123: w/p back to prev, w for common neighbours, w/q otherwise
+      const int32_t* __restrict__ plist = a.adjncy + c.prev_off;
+      // entries outside the list were replaced by prev above, so they never count as the group's maximum
+      int32_t vmax = (int)0x80000000;
 #pragma unroll
       for (int j = 0; j < kJ; ++j) {
-        x[4 * j + 0] = n2v_bias(a, c, x[4 * j + 0], adj[j].x);
-        x[4 * j + 1] = n2v_bias(a, c, x[4 * j + 1], adj[j].y);
-        x[4 * j + 2] = n2v_bias(a, c, x[4 * j + 2], adj[j].z);
-        x[4 * j + 3] = n2v_bias(a, c, x[4 * j + 3], adj[j].w);
+        vmax = (adj[j].x != c.prev && adj[j].x > vmax) ? adj[j].x : vmax;
+        vmax = (adj[j].y != c.prev && adj[j].y > vmax) ? adj[j].y : vmax;
+        vmax = (adj[j].z != c.prev && adj[j].z > vmax) ? adj[j].z : vmax;
+        vmax = (adj[j].w != c.prev && adj[j].w > vmax) ? adj[j].w : vmax;
       }
+      vmax = wave_max_i32(vmax);
+      // N(prev)[seg_lo, seg_hi) can hold this group's vertices; later groups only hold larger ones
+      const uint32_t seg_hi = coop_upper_bound(plist, seg_lo, (uint32_t)c.prev_deg, vmax, lane);
+      uint32_t pos = seg_lo;
+#pragma unroll
+      for (int j = 0; j < kJ; ++j) {
+        const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (post[e] == c.prev) {
+            x[4 * j + e] = x[4 * j + e] * a.inv_p;
+          } else {
+            pos = gallop_lower_bound(plist, pos, seg_hi, post[e]);
+            const bool common = pos < seg_hi && plist[pos] == post[e];
+            x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
+          }
+        }
+      }
+      seg_lo = seg_hi;
     }
 
     float q = 0.0f;
@@ -294,7 +481,7 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
 
 // ---- LDS task table ----------------------------------------------------------------------------
 
-template <int kWGT>
+template <int kWGT, int kApp>
 struct TaskTable {
   // include/gpu_task.cuh:24-33, as structure of arrays; len < 0 marks an empty slot.
   int32_t walker[kWGT];
@@ -316,11 +503,13 @@ struct TaskTable {
   // wave partials of the hub chunk in flight
   float hub_w[kHubChunk][16];
   int32_t hub_sel[kHubChunk][16];
+  // node2vec only: one scratch block per wave for the reversed adjacency test
+  N2vScratch n2v[kApp == FW_APP_NODE2VEC ? kWGT / 64 : 1];
 };
 
 // The slot index is wave-uniform; readfirstlane tells the compiler so (scalar registers, scalar Philox).
-template <int kWGT>
-__device__ __forceinline__ StepCtx load_ctx(const fw_kargs& a, const TaskTable<kWGT>& tt, int slot) {
+template <int kWGT, int kApp>
+__device__ __forceinline__ StepCtx load_ctx(const fw_kargs& a, const TaskTable<kWGT, kApp>& tt, int slot) {
   StepCtx c;
   c.off = (uint32_t)__builtin_amdgcn_readfirstlane((int)tt.off[slot]);
   c.deg = __builtin_amdgcn_readfirstlane(tt.deg[slot]);
@@ -335,8 +524,8 @@ __device__ __forceinline__ StepCtx load_ctx(const fw_kargs& a, const TaskTable<k
 
 // Step commit by one lane: include/walker.cuh:1372-1385 and Task::update (include/gpu_task.cuh:70-77).
 // The CSR range of the new vertex is reloaded in phase C by the slot's own thread.
-template <int kWGT>
-__device__ __forceinline__ void commit(const fw_kargs& a, TaskTable<kWGT>& tt, int slot, const StepCtx& c, int32_t v,
+template <int kWGT, int kApp>
+__device__ __forceinline__ void commit(const fw_kargs& a, TaskTable<kWGT, kApp>& tt, int slot, const StepCtx& c, int32_t v,
                                        bool ok, unsigned long long& n_steps, unsigned long long& n_edges) {
   if (!ok) {
     tt.flag[slot] = kFlagDead;
@@ -359,11 +548,12 @@ __device__ __forceinline__ void commit(const fw_kargs& a, TaskTable<kWGT>& tt, i
 template <int kApp, int kWGT>
 __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
   constexpr int kNW = kWGT / 64;
-  __shared__ TaskTable<kWGT> tt;
+  __shared__ TaskTable<kWGT, kApp> tt;
 
   const int tid = (int)threadIdx.x;
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  N2vScratch* const scr = &tt.n2v[kApp == FW_APP_NODE2VEC ? wave : 0];
   unsigned long long n_steps = 0ull, n_edges = 0ull;
 
   tt.len[tid] = -1;
@@ -393,7 +583,7 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
           if (kApp == FW_APP_METAPATH) c.want = a.schema[c.step % (uint32_t)a.schema_len];
           float W;
           int32_t sel, selv;
-          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, (uint32_t)wave, (uint32_t)kNW, W, sel, selv);
+          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, (uint32_t)wave, (uint32_t)kNW, scr, W, sel, selv);
           if (lane == 0) {
             tt.hub_w[h][wave] = W;
             tt.hub_sel[h][wave] = sel;
@@ -446,10 +636,10 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
         const uint32_t nq = ((c.off + (uint32_t)c.deg) - (c.off & ~3u) + 3u) >> 2;
         int32_t v = -1;
         if (nq <= 64u) {  // one quartet per lane: fetch the adjacency with the biases, no dependent load
-          wave_stream<kApp, 1, true>(a, c, lane, 0u, 1u, W, sel, selv);
+          wave_stream<kApp, 1, true>(a, c, lane, 0u, 1u, scr, W, sel, selv);
           v = selv;
         } else {
-          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, 0u, 1u, W, sel, selv);
+          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, 0u, 1u, scr, W, sel, selv);
           if (sel >= 0) v = a.adjncy[c.off + (uint32_t)sel];
         }
         if (lane == 0) commit(a, tt, slot, c, v, sel >= 0, n_steps, n_edges);
