@@ -36,7 +36,7 @@ class WalkParams(C.Structure):
         ("app", C.c_int32), ("sampler", C.c_int32), ("max_depth", C.c_int32), ("wg_threads", C.c_int32),
         ("hub_threshold", C.c_int32), ("schema_len", C.c_int32), ("schema", C.c_int32 * FW_MAX_SCHEMA),
         ("tp", C.c_float), ("p", C.c_float), ("q", C.c_float), ("walker_base", C.c_uint32),
-        ("seed", C.c_uint64), ("grid", C.c_int32), ("reserved", C.c_int32),
+        ("seed", C.c_uint64), ("grid", C.c_int32), ("park_threshold", C.c_int32),
     ]
 
 

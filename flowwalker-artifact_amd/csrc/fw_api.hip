@@ -68,7 +68,7 @@ extern "C" void fw_walk_params_default(fw_walk_params* p) {
   p->sampler = FW_SAMPLER_ZPRS;
   p->max_depth = 81;
   p->wg_threads = 512;
-  p->hub_threshold = 16384;
+  p->hub_threshold = 4096;
   p->schema_len = 5;
   for (int i = 0; i < 5; ++i) p->schema[i] = i;
   p->tp = 0.2f;
@@ -216,6 +216,10 @@ extern "C" int fw_graph_destroy(fw_graph* g) {
     for (void* p : ptrs) {
       if (p && hipFree(p) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
     }
+  }
+  void* index_ptrs[2] = {g->hub_index, g->hub_vertex};
+  for (void* p : index_ptrs) {
+    if (p && hipFree(p) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
   }
   delete g;
   return rc;
@@ -410,6 +414,221 @@ static void fill_kargs(fw_kargs* a, const fw_graph* g, const fw_walk_params* p) 
   a->inv_q = 1.0f / p->q;
   a->schema_len = p->schema_len;
   for (int i = 0; i < FW_MAX_SCHEMA; ++i) a->schema[i] = (i < p->schema_len) ? p->schema[i] : 0;
+  a->park_threshold = INT_MAX;
+  a->n_labels_per_hub = 1;
+}
+
+// ---- hub parking: walkers that reach a very-high-degree vertex wait there and are served in batches -------
+//
+// Execution strategy only: every walker still gets the vertex that the sampling definition gives it for
+// (seed, walker id, step), so results are identical with and without parking.  The walk kernel parks a walker
+// when it arrives on a vertex whose degree exceeds park_threshold; the parked records are grouped by hub
+// (counting sort on the device), the hub batch kernel serves up to 64 walkers of a hub with one pass over its
+// list, and the survivors resume in the next walk launch.  Loop until nobody is parked.
+
+__global__ void fw_hub_count_kernel(const uint32_t* __restrict__ xadj, int32_t V, int32_t threshold, unsigned* count) {
+  const int stride = gridDim.x * blockDim.x;
+  unsigned local = 0;
+  for (int v = blockIdx.x * blockDim.x + threadIdx.x; v < V; v += stride)
+    local += (int32_t)(xadj[v + 1] - xadj[v]) > threshold ? 1u : 0u;
+  if (local) atomicAdd(count, local);
+}
+
+__global__ void fw_hub_index_kernel(const uint32_t* __restrict__ xadj, int32_t V, int32_t threshold, unsigned* next,
+                                    int32_t* hub_index, int32_t* hub_vertex) {
+  const int stride = gridDim.x * blockDim.x;
+  for (int v = blockIdx.x * blockDim.x + threadIdx.x; v < V; v += stride) {
+    int32_t idx = -1;
+    if ((int32_t)(xadj[v + 1] - xadj[v]) > threshold) {
+      idx = (int32_t)atomicAdd(next, 1u);
+      hub_vertex[idx] = v;
+    }
+    hub_index[v] = idx;
+  }
+}
+
+// (Re)builds g->hub_index / hub_vertex for `threshold`; cached in the graph.
+static int ensure_hub_index(fw_graph* g, int32_t threshold) {
+  if (g->hub_index_threshold == threshold && g->hub_index) return FW_OK;
+  if (g->hub_index) { (void)hipFree(g->hub_index); g->hub_index = nullptr; }
+  if (g->hub_vertex) { (void)hipFree(g->hub_vertex); g->hub_vertex = nullptr; }
+  g->hub_index_threshold = -1;
+  g->n_hubs = 0;
+  unsigned* d_cnt = nullptr;
+  FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_cnt), 2 * sizeof(unsigned)));
+  FW_HIP(hipMemset(d_cnt, 0, 2 * sizeof(unsigned)));
+  hipLaunchKernelGGL(fw_hub_count_kernel, dim3(1024), dim3(256), 0, 0, g->xadj, g->V, threshold, d_cnt);
+  unsigned n_hubs = 0;
+  int rc = fw_check_hip(hipMemcpy(&n_hubs, d_cnt, sizeof(unsigned), hipMemcpyDeviceToHost), "hipMemcpy(hub count)", __FILE__, __LINE__);
+  if (rc == FW_OK) rc = fw_check_hip(hipMalloc(reinterpret_cast<void**>(&g->hub_index), (size_t)g->V * sizeof(int32_t)), "hipMalloc(hub_index)", __FILE__, __LINE__);
+  if (rc == FW_OK) rc = fw_check_hip(hipMalloc(reinterpret_cast<void**>(&g->hub_vertex), (size_t)(n_hubs ? n_hubs : 1) * sizeof(int32_t)), "hipMalloc(hub_vertex)", __FILE__, __LINE__);
+  if (rc == FW_OK) {
+    hipLaunchKernelGGL(fw_hub_index_kernel, dim3(1024), dim3(256), 0, 0, g->xadj, g->V, threshold, d_cnt + 1,
+                       g->hub_index, g->hub_vertex);
+    rc = fw_check_hip(hipDeviceSynchronize(), "hub index", __FILE__, __LINE__);
+  }
+  (void)hipFree(d_cnt);
+  if (rc != FW_OK) return rc;
+  g->n_hubs = (int32_t)n_hubs;
+  g->hub_index_threshold = threshold;
+  return FW_OK;
+}
+
+// One workgroup: exclusive scan of the bucket counts, and one task per 64 parked walkers of a bucket.
+// ctrs[2] = number of tasks (out).
+__global__ __launch_bounds__(1024) void fw_bucket_scan_kernel(const uint32_t* __restrict__ bucket_count,
+                                                              uint32_t* bucket_offset, int n_buckets, uint2* tasks,
+                                                              uint32_t* ctrs) {
+  __shared__ uint32_t partial[1024];
+  const int tid = (int)threadIdx.x;
+  const int per = (n_buckets + 1023) / 1024;
+  const int lo = tid * per;
+  const int hi = lo + per < n_buckets ? lo + per : n_buckets;
+  uint32_t sum = 0;
+  for (int b = lo; b < hi; ++b) sum += bucket_count[b];
+  partial[tid] = sum;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {  // Hillis-Steele inclusive scan over the 1024 partial sums
+    const uint32_t add = tid >= off ? partial[tid - off] : 0u;
+    __syncthreads();
+    partial[tid] += add;
+    __syncthreads();
+  }
+  uint32_t run = partial[tid] - sum;  // exclusive prefix of this thread's chunk
+  for (int b = lo; b < hi; ++b) {
+    const uint32_t c = bucket_count[b];
+    bucket_offset[b] = run;
+    run += c;
+    if (c != 0u) {
+      const uint32_t nb = (c + 63u) >> 6;
+      const uint32_t t0 = atomicAdd(&ctrs[2], nb);
+      for (uint32_t k = 0; k < nb; ++k) tasks[t0 + k] = make_uint2((uint32_t)b, k * 64u);
+    }
+  }
+}
+
+__global__ void fw_scatter_parked_kernel(const fw_walker_rec* __restrict__ parked, uint32_t m,
+                                         const int32_t* __restrict__ hub_index, int labels, int metapath,
+                                         const uint32_t* __restrict__ bucket_offset, uint32_t* bucket_fill,
+                                         uint32_t* sorted_idx) {
+  const uint32_t stride = gridDim.x * blockDim.x;
+  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < m; i += stride) {
+    const fw_walker_rec r = parked[i];
+    const uint32_t slot = metapath ? (uint32_t)(r.len - 1) % (uint32_t)labels : 0u;
+    const uint32_t b = (uint32_t)hub_index[r.cur] * (uint32_t)labels + slot;
+    sorted_idx[bucket_offset[b] + atomicAdd(&bucket_fill[b], 1u)] = i;
+  }
+}
+
+// Device buffers of one park / batch / resume loop (one per stream in flight).
+struct ParkBuffers {
+  size_t cap = 0;       // walkers
+  int n_buckets = 0;
+  fw_walker_rec* parked = nullptr;
+  fw_walker_rec* resume = nullptr;
+  uint32_t* sorted_idx = nullptr;
+  uint32_t* bucket_count = nullptr;   // [3 * n_buckets]: count, offset, fill
+  uint2* tasks = nullptr;
+  uint32_t* ctrs = nullptr;           // [0] parked, [1] resumed, [2] tasks, [3] task dispenser
+  uint32_t* h_ctrs = nullptr;         // pinned mirror of ctrs[0..1]
+
+  int alloc(size_t walkers, int buckets) {
+    cap = walkers;
+    n_buckets = buckets;
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&parked), cap * sizeof(fw_walker_rec)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&resume), cap * sizeof(fw_walker_rec)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&sorted_idx), cap * sizeof(uint32_t)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&bucket_count), (size_t)3 * buckets * sizeof(uint32_t)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&tasks), (cap / 64 + (size_t)buckets + 1) * sizeof(uint2)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), 4 * sizeof(uint32_t)));
+    FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), 4 * sizeof(uint32_t), hipHostMallocDefault));
+    return FW_OK;
+  }
+  void release() {
+    void* dev[6] = {parked, resume, sorted_idx, bucket_count, tasks, ctrs};
+    for (void* p : dev) if (p) (void)hipFree(p);
+    if (h_ctrs) (void)hipHostFree(h_ctrs);
+    parked = resume = nullptr; sorted_idx = bucket_count = ctrs = h_ctrs = nullptr; tasks = nullptr;
+  }
+};
+
+// Decides whether a call parks walkers, and at which degree.  Returns INT_MAX for "no".
+static int32_t resolve_park_threshold(const fw_walk_params* p, int32_t n) {
+  if (p->app == FW_APP_NODE2VEC) return INT_MAX;  // its biases depend on the walker: nothing to share
+  if (p->park_threshold < 0) return INT_MAX;
+  if (p->park_threshold == 0) {
+    // default: only batches large enough for walkers to meet on hubs
+    if (n < 65536) return INT_MAX;
+    return p->hub_threshold > 4096 ? p->hub_threshold : 4096;
+  }
+  // parked hubs are sampled at workgroup granularity, so they must be above the wave / workgroup threshold
+  return p->park_threshold > p->hub_threshold ? p->park_threshold : p->hub_threshold;
+}
+
+// Runs all walks of one batch on `stream`: a single walk launch, or the park / batch / resume loop.
+// `a` is complete except for the parking fields; a.dispenser / a.counters point at zeroed memory.
+static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_kargs a, int32_t park_threshold,
+                             ParkBuffers* pb, hipStream_t stream, int* grid_used, int* launches) {
+  *launches = 0;
+  if (park_threshold == INT_MAX || g->n_hubs == 0 || pb == nullptr) {
+    *launches = 1;
+    return fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, grid_used);
+  }
+  const int labels = p->app == FW_APP_METAPATH ? p->schema_len : 1;
+  const int32_t n_total = a.n;
+  a.park_threshold = park_threshold;
+  a.n_labels_per_hub = labels;
+  a.hub_index = g->hub_index;
+  a.parked = pb->parked;
+  a.parked_count = &pb->ctrs[0];
+  a.bucket_count = pb->bucket_count;
+  uint32_t* bucket_offset = pb->bucket_count + pb->n_buckets;
+  uint32_t* bucket_fill = pb->bucket_count + 2 * pb->n_buckets;
+  fw_hub_args h;
+  h.parked = pb->parked;
+  h.sorted_idx = pb->sorted_idx;
+  h.bucket_count = pb->bucket_count;
+  h.bucket_offset = bucket_offset;
+  h.tasks = pb->tasks;
+  h.ntasks = &pb->ctrs[2];
+  h.task_next = &pb->ctrs[3];
+  h.hub_vertex = g->hub_vertex;
+  h.resume = pb->resume;
+  h.resume_count = &pb->ctrs[1];
+
+  a.resume = nullptr;
+  for (int iter = 0;; ++iter) {
+    FW_HIP(hipMemsetAsync(a.dispenser, 0, sizeof(uint32_t), stream));
+    FW_HIP(hipMemsetAsync(pb->ctrs, 0, 4 * sizeof(uint32_t), stream));
+    FW_HIP(hipMemsetAsync(pb->bucket_count, 0, (size_t)3 * pb->n_buckets * sizeof(uint32_t), stream));
+    int rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, iter == 0 ? grid_used : nullptr);
+    if (rc != FW_OK) return rc;
+    ++*launches;
+    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    FW_HIP(hipStreamSynchronize(stream));
+    const uint32_t m = pb->h_ctrs[0];
+    if (m == 0u) break;
+    if ((size_t)m > pb->cap) { fw_set_error("internal: %u walkers parked, capacity %zu", m, pb->cap); return FW_ERR_INVALID; }
+    hipLaunchKernelGGL(fw_bucket_scan_kernel, dim3(1), dim3(1024), 0, stream, pb->bucket_count, bucket_offset,
+                       pb->n_buckets, pb->tasks, pb->ctrs);
+    FW_HIP(hipGetLastError());
+    unsigned blocks = (m + 255u) / 256u;
+    if (blocks > 4096u) blocks = 4096u;
+    hipLaunchKernelGGL(fw_scatter_parked_kernel, dim3(blocks), dim3(256), 0, stream, pb->parked, m, g->hub_index,
+                       labels, p->app == FW_APP_METAPATH ? 1 : 0, bucket_offset, bucket_fill, pb->sorted_idx);
+    FW_HIP(hipGetLastError());
+    rc = fw_launch_hub_batch(a, h, p->app, p->wg_threads, stream);
+    if (rc != FW_OK) return rc;
+    ++*launches;
+    FW_HIP(hipMemcpyAsync(pb->h_ctrs + 1, pb->ctrs + 1, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    FW_HIP(hipStreamSynchronize(stream));
+    const uint32_t r = pb->h_ctrs[1];
+    if (r == 0u) break;
+    if ((size_t)r > pb->cap || r > (uint32_t)n_total) { fw_set_error("internal: %u walkers resumed, capacity %zu", r, pb->cap); return FW_ERR_INVALID; }
+    a.resume = pb->resume;
+    a.n = (int32_t)r;
+  }
+  return FW_OK;
 }
 
 struct Scratch {  // dispenser word + two 64-bit counters, 32 bytes per launch slot
@@ -431,6 +650,14 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
   hipStream_t stream = reinterpret_cast<hipStream_t>(stream_v);
   const double t0 = now_ms();
 
+  const int32_t park_threshold = resolve_park_threshold(p, n);
+  ParkBuffers pb;
+  bool use_pb = false;
+  if (park_threshold != INT_MAX) {
+    rc = ensure_hub_index(const_cast<fw_graph*>(g), park_threshold);
+    if (rc != FW_OK) return rc;
+    use_pb = g->n_hubs > 0;
+  }
   Scratch* d_scr = nullptr;
   FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_scr), sizeof(Scratch)));
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -438,12 +665,17 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
     if (ev0) (void)hipEventDestroy(ev0);
     if (ev1) (void)hipEventDestroy(ev1);
     if (d_scr) (void)hipFree(d_scr);
+    pb.release();
   };
 #define FW_TRY(call)                                                 \
   do {                                                               \
     int rc_ = fw_check_hip((call), #call, __FILE__, __LINE__);       \
     if (rc_ != FW_OK) { cleanup(); return rc_; }                     \
   } while (0)
+  if (use_pb) {
+    rc = pb.alloc((size_t)n, g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1));
+    if (rc != FW_OK) { cleanup(); return rc; }
+  }
   FW_TRY(hipEventCreate(&ev0));
   FW_TRY(hipEventCreate(&ev1));
   FW_TRY(hipMemsetAsync(d_scr, 0, sizeof(Scratch), stream));
@@ -457,9 +689,9 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
   a.n = n;
   a.dispenser = &d_scr->dispenser;
   a.counters = d_scr->counters;
-  int grid_used = 0;
+  int grid_used = 0, launches = 0;
   FW_TRY(hipEventRecord(ev0, stream));
-  rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, &grid_used);
+  rc = run_walk_launches(g, p, a, park_threshold, use_pb ? &pb : nullptr, stream, &grid_used, &launches);
   if (rc != FW_OK) { cleanup(); return rc; }
   FW_TRY(hipEventRecord(ev1, stream));
   FW_TRY(hipStreamSynchronize(stream));
@@ -473,7 +705,7 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
     stats->total_ms = now_ms() - t0;
     stats->steps = h.counters[0];
     stats->sampled_edges = h.counters[1];
-    stats->launches = 1;
+    stats->launches = launches;
     stats->grid = grid_used;
   }
   return FW_OK;
@@ -495,6 +727,14 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
   const size_t bs = batch_size;
   const size_t md = (size_t)p->max_depth;
 
+  const int32_t park_threshold = resolve_park_threshold(p, (int32_t)bs);
+  bool use_pb = false;
+  if (park_threshold != INT_MAX) {
+    rc = ensure_hub_index(const_cast<fw_graph*>(g), park_threshold);
+    if (rc != FW_OK) return rc;
+    use_pb = g->n_hubs > 0;
+  }
+  ParkBuffers pbs[2];
   int32_t* d_starts = nullptr;
   int32_t* d_paths = nullptr;
   Scratch* d_scr = nullptr;
@@ -506,7 +746,15 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     if (d_starts) (void)hipFree(d_starts);
     if (d_paths) (void)hipFree(d_paths);
     if (d_scr) (void)hipFree(d_scr);
+    pbs[0].release();
+    pbs[1].release();
   };
+  if (use_pb) {
+    for (int i = 0; i < nbuf; ++i) {
+      rc = pbs[i].alloc(bs, g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1));
+      if (rc != FW_OK) { cleanup(); return rc; }
+    }
+  }
   FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_starts), bs * nbuf * sizeof(int32_t)));
   FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_paths), bs * nbuf * md * sizeof(int32_t)));
   const int nbatch = (int)(((size_t)n + bs - 1) / bs);
@@ -535,7 +783,8 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     a.dispenser = &d_scr[b].dispenser;
     a.counters = d_scr[b].counters;
     FW_TRY(hipEventRecord(events[2 * b], streams[s]));
-    rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, streams[s], &grid_used);
+    int launches = 0;
+    rc = run_walk_launches(g, p, a, park_threshold, use_pb ? &pbs[s] : nullptr, streams[s], &grid_used, &launches);
     if (rc != FW_OK) { cleanup(); return rc; }
     FW_TRY(hipEventRecord(events[2 * b + 1], streams[s]));
     FW_TRY(hipMemcpyAsync(h_paths + first * md, dp, (size_t)cnt * md * sizeof(int32_t), hipMemcpyDeviceToHost, streams[s]));

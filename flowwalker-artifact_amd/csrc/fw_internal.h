@@ -20,9 +20,22 @@ struct fw_graph {
   int32_t max_degree = -1;  // lazily computed
   int32_t max_degree_vertex = -1;
   int sorted = -1;          // lazily computed
+  // lazily built index of the vertices whose degree exceeds hub_index_threshold (hub parking)
+  int32_t hub_index_threshold = -1;
+  int32_t n_hubs = 0;
+  int32_t* hub_index = nullptr;   // int32[V]: position in hub_vertex, or -1
+  int32_t* hub_vertex = nullptr;  // int32[n_hubs]
 };
 
 constexpr int FW_EDGE_PAD = 4;
+
+// A walker in transit between kernels (parked on a hub, or resuming after its hub step): 16 bytes.
+struct fw_walker_rec {
+  int32_t q;     // query index inside the launch (walker id = walker_base + q)
+  int32_t cur;   // current vertex
+  int32_t prev;  // previous vertex or -1
+  int32_t len;   // path entries written so far
+};
 
 // Arguments of one walk-kernel launch.
 struct fw_kargs {
@@ -44,6 +57,28 @@ struct fw_kargs {
   float tp, inv_p, inv_q;
   int32_t schema_len;
   int32_t schema[FW_MAX_SCHEMA];
+  // hub parking (park_threshold = INT32_MAX switches it off)
+  int32_t park_threshold;            // a walker that arrives on a vertex of larger degree is parked
+  int32_t n_labels_per_hub;          // buckets per hub: 1, or schema_len for metapath (walkers wanting one label share a scan)
+  const int32_t* hub_index;          // int32[V]
+  fw_walker_rec* parked;             // out: parked walkers
+  uint32_t* parked_count;
+  uint32_t* bucket_count;            // [n_hubs * n_labels_per_hub]
+  const fw_walker_rec* resume;       // in: walkers to continue instead of fresh queries (NULL: use starts)
+};
+
+// Arguments of the hub batch kernel: one workgroup serves up to 64 parked walkers of one hub with one scan.
+struct fw_hub_args {
+  const fw_walker_rec* parked;
+  const uint32_t* sorted_idx;        // parked record indices grouped by bucket
+  const uint32_t* bucket_count;
+  const uint32_t* bucket_offset;
+  const uint2* tasks;                // (bucket, first walker of the batch inside the bucket)
+  const uint32_t* ntasks;
+  uint32_t* task_next;               // task dispenser
+  const int32_t* hub_vertex;
+  fw_walker_rec* resume;             // out: walkers that continue
+  uint32_t* resume_count;
 };
 
 void fw_set_error(const char* fmt, ...);
@@ -58,3 +93,6 @@ int fw_check_hip(hipError_t e, const char* what, const char* file, int line);
 // Returns the grid used through *grid_used.
 int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, hipStream_t stream,
                    int* grid_used);
+
+// Launches the hub batch kernel (persistent grid, tasks taken from h.task_next).
+int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, hipStream_t stream);

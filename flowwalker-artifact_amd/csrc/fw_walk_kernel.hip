@@ -658,7 +658,8 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
       const int np = first ? 0 : parity;  // lists to fill for the next round
       first = false;
       int32_t len = tt.len[tid];
-      bool need = tid < a.slot_limit;  // slot wants a new query
+      bool need = tid < a.slot_limit;  // slot wants a new walker
+      bool park = false;               // the slot's walker has reached a hub that is served by the batch kernel
       int32_t deg = 0;
       if (len >= 0) {
         if (tt.flag[tid] == kFlagMoved) {
@@ -675,11 +676,36 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
             stop = u24(bits) < a.tp;
           }
           need = stop;
+          park = !stop && deg > a.park_threshold;
         }
         // kFlagDead: dead end (no neighbour with positive bias), include/walker.cuh:1373-1374
       }
       bool exhausted = tt.exhausted != 0;
       for (;;) {
+        // park first: the record leaves the slot, which then asks for the next walker
+        const uint64_t pm = __ballot(park);
+        if (pm != 0ull) {
+          uint32_t pbase = 0;
+          const int pleader = __builtin_ctzll(pm);
+          if (lane == pleader) pbase = atomicAdd(a.parked_count, (uint32_t)__builtin_popcountll(pm));
+          pbase = (uint32_t)__builtin_amdgcn_readlane((int)pbase, pleader);
+          if (park) {
+            const uint32_t at = pbase + (uint32_t)__builtin_popcountll(pm & ((1ull << lane) - 1ull));
+            const int32_t v = tt.cur[tid];
+            fw_walker_rec rec;
+            rec.q = tt.walker[tid];
+            rec.cur = v;
+            rec.prev = tt.prev[tid];
+            rec.len = len;
+            a.parked[at] = rec;
+            const uint32_t label_slot =
+                kApp == FW_APP_METAPATH ? (uint32_t)(len - 1) % (uint32_t)a.n_labels_per_hub : 0u;
+            atomicAdd(&a.bucket_count[(uint32_t)a.hub_index[v] * (uint32_t)a.n_labels_per_hub + label_slot], 1u);
+            park = false;
+            need = true;
+            len = -1;
+          }
+        }
         const bool want = need && !exhausted;
         const uint64_t m = __ballot(want);
         if (m == 0ull) break;
@@ -690,22 +716,29 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
         if (want) {
           const uint32_t q = base + (uint32_t)__builtin_popcountll(m & ((1ull << lane) - 1ull));
           if (q < (uint32_t)a.n) {
-            const int32_t sp = a.starts[q];
-            a.paths[(uint64_t)q * (uint64_t)a.max_depth] = sp;  // include/walker.cuh:1342
-            if ((uint32_t)sp < (uint32_t)a.V && a.max_depth > 1) {
+            int32_t wq, sp, pv, ln;
+            if (a.resume != nullptr) {  // a walker coming back from its hub step
+              const fw_walker_rec rec = a.resume[q];
+              wq = rec.q; sp = rec.cur; pv = rec.prev; ln = rec.len;
+            } else {                    // a fresh query (include/walker.cuh:1340-1343)
+              wq = (int32_t)q; sp = a.starts[q]; pv = -1; ln = 1;
+              a.paths[(uint64_t)q * (uint64_t)a.max_depth] = sp;
+            }
+            if ((uint32_t)sp < (uint32_t)a.V && ln < a.max_depth) {
               const uint32_t o = a.xadj[sp];
               const uint32_t e = a.xadj[sp + 1];
               deg = (int32_t)(e - o);
               if (deg > 0) {
-                tt.walker[tid] = (int32_t)q;
+                tt.walker[tid] = wq;
                 tt.cur[tid] = sp;
-                tt.prev[tid] = -1;
+                tt.prev[tid] = pv;
                 tt.off[tid] = o;
                 tt.deg[tid] = deg;
                 tt.prev_off[tid] = 0;
                 tt.prev_deg[tid] = 0;
-                len = 1;
+                len = ln;
                 need = false;
+                park = deg > a.park_threshold;
               }
             }
           } else {
@@ -714,7 +747,7 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
           }
         }
       }
-      if (need || len < 0) {  // nothing to run in this slot (finished / never filled / beyond slot_limit)
+      if (need || len < 0) {  // nothing to run in this slot (finished / parked / never filled / beyond slot_limit)
         tt.len[tid] = -1;
       } else {
         tt.len[tid] = len;
@@ -733,6 +766,276 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
   if (n_steps != 0ull) {
     atomicAdd(&a.counters[0], n_steps);
     atomicAdd(&a.counters[1], n_edges);
+  }
+}
+
+// ---- hub batch kernel -----------------------------------------------------------------------------
+//
+// Many walkers stand on the same high-degree vertex at the same time (visits are proportional to degree), and
+// for DeepWalk / PPR / MetaPath the biases of a list do not depend on the walker.  One workgroup therefore
+// serves up to 64 parked walkers of one hub with ONE pass over its list: lane i of every wave carries walker
+// i's reservoir (Sj, u, selection, its own Philox stream), while the group loads, the 16 adds, the DPP scan and
+// the running total S are shared by all 64.  The sampling definition is the workgroup sampler's, unchanged:
+// wave w owns groups w, w + NW, ..., the wave totals are combined by inverse transform, every draw is
+// addressed by (walker, step, stream, index).  Each walker gets exactly the vertex it would have got alone.
+
+// per-lane Philox word queue (same addressing as DrawQueue, different walker in every lane)
+struct LaneDraw {
+  uint32_t q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+  uint32_t avail = 0;
+  uint32_t blk = 0;
+};
+
+__device__ __forceinline__ float next_uniform_lane(LaneDraw& d, const fw_kargs& a, uint32_t walker, uint32_t step,
+                                                   uint32_t stream) {
+  if (d.avail == 0u) {
+    const uint4 b = philox4x32_10(walker, step, stream, d.blk, a.seed_lo, a.seed_hi);
+    d.q0 = b.x; d.q1 = b.y; d.q2 = b.z; d.q3 = b.w;
+    d.avail = 4u;
+    ++d.blk;
+  }
+  const float u = u24(d.q0);
+  d.q0 = d.q1; d.q1 = d.q2; d.q2 = d.q3;
+  --d.avail;
+  return u;
+}
+
+__device__ __forceinline__ float bperm_f(int byte_addr, float x) {
+  return __int_as_float(__builtin_amdgcn_ds_bpermute(byte_addr, __float_as_int(x)));
+}
+
+template <int kApp, int kWGT>
+__global__ __launch_bounds__(kWGT) void fw_hub_batch(const fw_kargs a, const fw_hub_args h) {
+  constexpr int kNW = kWGT / 64;
+  constexpr uint32_t kG = 64u * kGroupQuartets;
+  constexpr int kEl = 4 * kGroupQuartets;
+  __shared__ int32_t s_sel[kNW][64];
+  __shared__ float s_w[16];
+  __shared__ uint32_t s_task;
+
+  const int tid = (int)threadIdx.x;
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t ntasks = *h.ntasks;
+  const uint32_t labels = (uint32_t)a.n_labels_per_hub;
+  const uint32_t* __restrict__ bias =
+      reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
+  unsigned long long n_steps = 0ull, n_edges = 0ull;
+
+  for (;;) {
+    if (tid == 0) s_task = atomicAdd(h.task_next, 1u);
+    __syncthreads();
+    const uint32_t t = s_task;
+    __syncthreads();  // everyone has read s_task before it is overwritten; also fences s_sel / s_w reuse
+    if (t >= ntasks) break;
+
+    const uint2 task = h.tasks[t];
+    const uint32_t bucket = task.x;
+    const uint32_t in_bucket = h.bucket_count[bucket] - task.y;
+    const int count = (int)(in_bucket < 64u ? in_bucket : 64u);
+    const uint32_t rec_base = h.bucket_offset[bucket] + task.y;
+    const int32_t v = h.hub_vertex[bucket / labels];
+    const int32_t want = kApp == FW_APP_METAPATH ? a.schema[bucket % labels] : 0;
+    const uint32_t off = a.xadj[v];
+    const uint32_t deg = a.xadj[v + 1] - off;
+    const uint32_t a0 = off & ~3u;
+    const uint32_t end = off + deg;
+    const uint32_t nq = (end - a0 + 3u) >> 2;
+    const uint32_t ngroups = (nq + kG - 1u) / kG;
+
+    // lane i carries walker i of the batch
+    const bool have = lane < count;
+    fw_walker_rec rec;
+    rec.q = 0; rec.cur = v; rec.prev = -1; rec.len = 1;
+    if (have) rec = h.parked[h.sorted_idx[rec_base + (uint32_t)lane]];
+    const uint32_t walker = a.walker_base + (uint32_t)rec.q;
+    const uint32_t step = (uint32_t)(rec.len - 1);
+
+    float S = 0.0f;                      // shared: running total of this wave's groups
+    float Sj = 0.0f, u = 1.0f;           // per walker
+    int32_t sel = -1;
+    LaneDraw dq;
+
+    for (uint32_t g = (uint32_t)wave; g < ngroups; g += (uint32_t)kNW) {
+      const uint32_t kb = g * kG + (uint32_t)lane;
+      const bool interior = g > 0u && (g + 1u) * kG < nq;
+      uint4 raw[kGroupQuartets];
+      float x[kEl];
+      if (interior) {
+#pragma unroll
+        for (int j = 0; j < kGroupQuartets; ++j)
+          raw[j] = *reinterpret_cast<const uint4*>(bias + a0 + 4u * (kb + 64u * (uint32_t)j));
+      } else {
+#pragma unroll
+        for (int j = 0; j < kGroupQuartets; ++j) {
+          const uint32_t k = kb + 64u * (uint32_t)j;
+          raw[j] = make_uint4(0, 0, 0, 0);
+          if (k < nq) raw[j] = *reinterpret_cast<const uint4*>(bias + a0 + 4u * k);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kGroupQuartets; ++j) {
+        if (kApp == FW_APP_METAPATH) {
+          x[4 * j + 0] = (int32_t)raw[j].x == want ? 1.0f : 0.0f;
+          x[4 * j + 1] = (int32_t)raw[j].y == want ? 1.0f : 0.0f;
+          x[4 * j + 2] = (int32_t)raw[j].z == want ? 1.0f : 0.0f;
+          x[4 * j + 3] = (int32_t)raw[j].w == want ? 1.0f : 0.0f;
+        } else {
+          x[4 * j + 0] = __uint_as_float(raw[j].x);
+          x[4 * j + 1] = __uint_as_float(raw[j].y);
+          x[4 * j + 2] = __uint_as_float(raw[j].z);
+          x[4 * j + 3] = __uint_as_float(raw[j].w);
+        }
+      }
+      if (!interior) {
+#pragma unroll
+        for (int j = 0; j < kGroupQuartets; ++j) {
+          const uint32_t k = kb + 64u * (uint32_t)j;
+          const uint32_t base = a0 + 4u * k;
+          const bool ex = k < nq;
+          x[4 * j + 0] = (ex && base >= off && base < end) ? x[4 * j + 0] : 0.0f;
+          x[4 * j + 1] = (ex && base + 1u >= off && base + 1u < end) ? x[4 * j + 1] : 0.0f;
+          x[4 * j + 2] = (ex && base + 2u >= off && base + 2u < end) ? x[4 * j + 2] : 0.0f;
+          x[4 * j + 3] = (ex && base + 3u >= off && base + 3u < end) ? x[4 * j + 3] : 0.0f;
+        }
+      }
+      float q = 0.0f;
+#pragma unroll
+      for (int i = 0; i < kEl; ++i) q = q + x[i];
+      const float I = wave_scan(q);
+      const float T = readlane_f(I, 63);
+      const float Snew = S + T;
+
+      const bool acc = have && (Snew * u > Sj);  // per walker: this group enters its reservoir
+      const uint64_t macc = __ballot(acc);
+      if (macc != 0ull) {
+        float target = 0.0f;
+        if (acc) target = next_uniform_lane(dq, a, walker, step, (uint32_t)wave) * T;
+        // which lane's biases hold the target of walker k: first lane with a positive total whose prefix
+        // exceeds it, else the last lane with a positive total
+        const bool pos = q > 0.0f;
+        const uint64_t mpos = __ballot(pos);
+        int src = 0;
+        for (uint64_t mm = macc; mm != 0ull; mm &= mm - 1ull) {
+          const int k = __builtin_ctzll(mm);
+          const float tk = readlane_f(target, k);
+          const uint64_t mk = __ballot(pos && I > tk);
+          const int lk = mk != 0ull ? __builtin_ctzll(mk) : 63 - __builtin_clzll(mpos);
+          src = (lane == k) ? lk : src;
+        }
+        // every walker resolves its own target on the 16 biases of its source lane (fetched across lanes)
+        const int addr = src << 2;
+        float e = bperm_f(addr, I - q);
+        int pick = -1, last = -1;
+#pragma unroll
+        for (int i = 0; i < kEl; ++i) {
+          const float xi = bperm_f(addr, x[i]);
+          e = e + xi;
+          const bool p = xi > 0.0f;
+          pick = (p && e > target && pick < 0) ? i : pick;
+          last = p ? i : last;
+        }
+        pick = pick < 0 ? last : pick;
+        if (acc) {
+          const uint32_t abs_idx = a0 + 4u * (g * kG + (uint32_t)src) + 256u * (uint32_t)(pick >> 2) + (uint32_t)(pick & 3);
+          sel = (int32_t)(abs_idx - off);
+          Sj = Snew;
+          u = next_uniform_lane(dq, a, walker, step, (uint32_t)wave);
+        }
+      }
+      S = Snew;
+    }
+
+    s_sel[wave][lane] = sel;
+    if (lane == 0) s_w[wave] = S;
+    __syncthreads();
+
+    if (wave == 0) {
+      // inverse transform over the wave totals, per walker (include/sampler.cuh:118-126 is the max-reduce analogue)
+      const float Wl = lane < kNW ? s_w[lane] : 0.0f;
+      const float J = row_scan(Wl);
+      const float total = readlane_f(J, kNW - 1);
+      int32_t pick = -1;
+      if (have) {
+        const float target = u24(philox4x32_10(walker, step, kStreamWave, 0u, a.seed_lo, a.seed_hi).x) * total;
+        int wsel = -1, wlast = -1;
+#pragma unroll
+        for (int w = 0; w < kNW; ++w) {
+          const float Ww = readlane_f(Wl, w);
+          const float Jw = readlane_f(J, w);
+          if (Ww > 0.0f) {
+            wsel = (wsel < 0 && Jw > target) ? w : wsel;
+            wlast = w;
+          }
+        }
+        wsel = wsel < 0 ? wlast : wsel;
+        if (wsel >= 0) pick = s_sel[wsel][lane];
+      }
+      const bool moved = have && pick >= 0;
+      bool go_on = false;
+      int32_t nv = -1;
+      if (moved) {  // step commit: include/walker.cuh:1410-1417
+        nv = a.adjncy[off + (uint32_t)pick];
+        a.paths[(uint64_t)(uint32_t)rec.q * (uint64_t)a.max_depth + (uint64_t)rec.len] = nv;
+        go_on = rec.len + 1 < a.max_depth;
+        if (kApp == FW_APP_PPR && go_on) {
+          const uint32_t bits = philox4x32_10(walker, step, kStreamStop, 0u, a.seed_lo, a.seed_hi).x;
+          go_on = !(u24(bits) < a.tp);
+        }
+      }
+      const uint64_t mmoved = __ballot(moved);
+      if (lane == 0) {
+        const unsigned long long c = (unsigned long long)__builtin_popcountll(mmoved);
+        n_steps += c;
+        n_edges += c * (unsigned long long)deg;
+      }
+      const uint64_t mgo = __ballot(go_on);
+      if (mgo != 0ull) {  // survivors resume in the next walk launch
+        uint32_t rbase = 0;
+        const int leader = __builtin_ctzll(mgo);
+        if (lane == leader) rbase = atomicAdd(h.resume_count, (uint32_t)__builtin_popcountll(mgo));
+        rbase = (uint32_t)__builtin_amdgcn_readlane((int)rbase, leader);
+        if (go_on) {
+          fw_walker_rec out;
+          out.q = rec.q;
+          out.cur = nv;
+          out.prev = v;
+          out.len = rec.len + 1;
+          h.resume[rbase + (uint32_t)__builtin_popcountll(mgo & ((1ull << lane) - 1ull))] = out;
+        }
+      }
+    }
+  }
+  if (n_steps != 0ull) {
+    atomicAdd(&a.counters[0], n_steps);
+    atomicAdd(&a.counters[1], n_edges);
+  }
+}
+
+template <int kApp, int kWGT>
+int launch_hub_one(const fw_kargs& a, const fw_hub_args& h, hipStream_t stream) {
+  int dev = 0;
+  hipDeviceProp_t prop;
+  FW_HIP(hipGetDevice(&dev));
+  FW_HIP(hipGetDeviceProperties(&prop, dev));
+  int per_cu = 0;
+  FW_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fw_hub_batch<kApp, kWGT>, kWGT, 0));
+  if (per_cu < 1) per_cu = 1;
+  const int grid = prop.multiProcessorCount * per_cu;
+  hipLaunchKernelGGL((fw_hub_batch<kApp, kWGT>), dim3(grid), dim3(kWGT), 0, stream, a, h);
+  FW_HIP(hipGetLastError());
+  return FW_OK;
+}
+
+template <int kApp>
+int launch_hub_app(const fw_kargs& a, const fw_hub_args& h, int wg_threads, hipStream_t stream) {
+  switch (wg_threads) {
+    case 256: return launch_hub_one<kApp, 256>(a, h, stream);
+    case 512: return launch_hub_one<kApp, 512>(a, h, stream);
+    case 1024: return launch_hub_one<kApp, 1024>(a, h, stream);
+    default:
+      fw_set_error("wg_threads must be 256, 512 or 1024 (got %d)", wg_threads);
+      return FW_ERR_INVALID;
   }
 }
 
@@ -772,6 +1075,17 @@ int launch_app(const fw_kargs& a, int wg_threads, int grid, hipStream_t stream, 
 }
 
 }  // namespace
+
+int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, hipStream_t stream) {
+  switch (app) {
+    case FW_APP_DEEPWALK: return launch_hub_app<FW_APP_DEEPWALK>(a, h, wg_threads, stream);
+    case FW_APP_PPR: return launch_hub_app<FW_APP_PPR>(a, h, wg_threads, stream);
+    case FW_APP_METAPATH: return launch_hub_app<FW_APP_METAPATH>(a, h, wg_threads, stream);
+    default:
+      fw_set_error("the hub batch kernel serves DeepWalk, PPR and MetaPath (node2vec biases depend on the walker)");
+      return FW_ERR_INVALID;
+  }
+}
 
 int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, hipStream_t stream,
                    int* grid_used) {

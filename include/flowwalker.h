@@ -60,7 +60,10 @@ typedef struct {
   uint32_t walker_base;  /* global walker id of query 0: keys the RNG, so batches do not repeat streams */
   uint64_t seed;         /* RNG seed (the reference hard-codes 1337: include/walker.cuh:1324) */
   int32_t grid;          /* workgroups to launch; 0 = library default (src/walk.cu:84-92 analogue) */
-  int32_t reserved;
+  int32_t park_threshold; /* hub parking, an execution strategy that never changes results: walkers that arrive on a
+                            vertex of larger degree wait there and are served 64 at a time by one shared scan of its
+                            list.  0 = library default (on for batches >= 65536 queries), < 0 = off, > 0 = degree
+                            (raised to hub_threshold if smaller).  Not used by node2vec. */
 } fw_walk_params;
 
 /* What src/main.cu:82-113 (calculate_workload) and the timing code of src/walk.cu report. */
@@ -69,7 +72,7 @@ typedef struct {
   double total_ms;        /* wall time of the call, transfers included (src/walk.cu:388,459,465) */
   uint64_t steps;         /* "Total sampled vertex" */
   uint64_t sampled_edges; /* "Total sampled edge": sum over steps of deg(source) */
-  int32_t launches;       /* kernel launches (= batches) */
+  int32_t launches;       /* fw_walk_batch: batches; fw_walk_device: walk + hub-batch kernel launches */
   int32_t grid;           /* workgroups per launch actually used */
 } fw_walk_stats;
 

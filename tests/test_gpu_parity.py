@@ -74,6 +74,42 @@ def test_metapath(gpu, hub):
     _check(gpu, hub, starts, app=gpu.APP_METAPATH, max_depth=9, schema=[3, 1], hub_threshold=64, seed=8)
 
 
+@pytest.mark.parametrize("wg", [256, 512, 1024])
+@pytest.mark.parametrize("app", ["deepwalk", "ppr", "metapath"])
+def test_hub_parking_does_not_change_results(gpu, hub, app, wg):
+    """Hub parking (walkers waiting on a hub are served 64 at a time by one shared scan) is an execution
+    strategy: with it forced on, every path must still equal the oracle's, which knows nothing about it."""
+    starts = np.random.RandomState(4).randint(0, 12000, size=6000).astype(np.int32)
+    starts[:700] = 0       # many walkers meet on the 9000-degree hub at once (several batches of 64)
+    starts[700:800] = 1    # and on the 2500-degree one
+    kw = dict(deepwalk=dict(app=gpu.APP_DEEPWALK, max_depth=41),
+              ppr=dict(app=gpu.APP_PPR, max_depth=81, tp=0.15),
+              metapath=dict(app=gpu.APP_METAPATH, max_depth=11, schema=[1, 3, 0]))[app]
+    for hub_thr, park in ((1000, 1000), (64, 2000), (500, 8000)):
+        _, st = _check(gpu, hub, starts, wg_threads=wg, hub_threshold=hub_thr, park_threshold=park, seed=77, **kw)
+        assert st.launches >= 3                      # walk, hub batch, walk ...
+
+
+def test_hub_parking_through_the_batch_driver(gpu, hub):
+    xadj, adj, w, lab = hub
+    starts = np.random.RandomState(5).randint(0, 12000, size=9000).astype(np.int32)
+    starts[::7] = 0
+    og = _oracle.Graph(xadj, adj, w, lab)
+    g = gpu.Graph.from_csr(xadj, adj, w, lab)
+    try:
+        p = gpu.default_params(max_depth=31, hub_threshold=1000, park_threshold=1500, seed=3)
+        ref, steps, edges = _oracle.walk(og, _oracle.from_walk_params(p), starts)
+        for bs, sync in ((9000, False), (2048, False), (2500, True)):
+            paths, st = g.walk_batch(p, starts, batch_size=bs, sync=sync)
+            assert (paths == ref).all()
+            assert (st.steps, st.sampled_edges) == (steps, edges)
+        p_off = gpu.default_params(max_depth=31, hub_threshold=1000, park_threshold=-1, seed=3)
+        paths, st = g.walk(p_off, starts)
+        assert (paths == ref).all() and st.launches == 1
+    finally:
+        g.destroy()
+
+
 def test_result_independent_of_launch_shape(gpu, hub):
     """Row q depends only on (seed, walker id, graph, parameters): grid size, workgroup scheduling and
     batching must not change a byte (the reference is not reproducible here: include/walker.cuh:1324,1339)."""
