@@ -337,13 +337,13 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
     if (!interior) {  // entries outside [off, end) (head / tail quartet, quartets past the list) have no bias
 #pragma unroll
       for (int j = 0; j < kJ; ++j) {
-        const uint32_t k = kb + 64u * (uint32_t)j;
-        const uint32_t base = a0 + 4u * k;
-        const bool ex = k < nq;
-        const bool in0 = ex && base >= c.off && base < end;
-        const bool in1 = ex && base + 1u >= c.off && base + 1u < end;
-        const bool in2 = ex && base + 2u >= c.off && base + 2u < end;
-        const bool in3 = ex && base + 3u >= c.off && base + 3u < end;
+        // local index of the quartet's first slot; it wraps below 0 for the head quartet, and quartets past
+        // the list start at or beyond deg, so one unsigned compare per slot decides membership
+        const uint32_t li = a0 + 4u * (kb + 64u * (uint32_t)j) - c.off;
+        const bool in0 = li < (uint32_t)c.deg;
+        const bool in1 = li + 1u < (uint32_t)c.deg;
+        const bool in2 = li + 2u < (uint32_t)c.deg;
+        const bool in3 = li + 3u < (uint32_t)c.deg;
         x[4 * j + 0] = in0 ? x[4 * j + 0] : 0.0f;
         x[4 * j + 1] = in1 ? x[4 * j + 1] : 0.0f;
         x[4 * j + 2] = in2 ? x[4 * j + 2] : 0.0f;
@@ -505,6 +505,9 @@ struct TaskTable {
   int32_t hub_sel[kHubChunk][16];
   // node2vec only: one scratch block per wave for the reversed adjacency test
   N2vScratch n2v[kApp == FW_APP_NODE2VEC ? kWGT / 64 : 1];
+  // metapath only: the schema, so that the per-step label is an LDS read (a dynamic index into the
+  // by-value kernel arguments would force a private copy of the whole array)
+  int32_t schema[kApp == FW_APP_METAPATH ? FW_MAX_SCHEMA : 1];
 };
 
 // The slot index is wave-uniform; readfirstlane tells the compiler so (scalar registers, scalar Philox).
@@ -558,6 +561,10 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
 
   tt.len[tid] = -1;
   tt.flag[tid] = 0;
+  if (kApp == FW_APP_METAPATH && tid == 0) {
+#pragma unroll
+    for (int i = 0; i < FW_MAX_SCHEMA; ++i) tt.schema[i] = a.schema[i];
+  }
   if (tid == 0) {
     tt.small_count[0] = tt.small_count[1] = 0;
     tt.hub_count[0] = tt.hub_count[1] = 0;
@@ -580,7 +587,7 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
         for (int h = 0; h < cnt; ++h) {
           const int slot = tt.hub_list[parity][hb + h];
           StepCtx c = load_ctx(a, tt, slot);
-          if (kApp == FW_APP_METAPATH) c.want = a.schema[c.step % (uint32_t)a.schema_len];
+          if (kApp == FW_APP_METAPATH) c.want = tt.schema[c.step % (uint32_t)a.schema_len];
           float W;
           int32_t sel, selv;
           wave_stream<kApp, kGroupQuartets, false>(a, c, lane, (uint32_t)wave, (uint32_t)kNW, scr, W, sel, selv);
@@ -630,7 +637,7 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
         if (idx >= ns) break;
         const int slot = tt.small_list[parity][idx];
         StepCtx c = load_ctx(a, tt, slot);
-        if (kApp == FW_APP_METAPATH) c.want = a.schema[c.step % (uint32_t)a.schema_len];
+        if (kApp == FW_APP_METAPATH) c.want = tt.schema[c.step % (uint32_t)a.schema_len];
         float W;
         int32_t sel, selv;
         const uint32_t nq = ((c.off + (uint32_t)c.deg) - (c.off & ~3u) + 3u) >> 2;
@@ -812,10 +819,15 @@ __global__ __launch_bounds__(kWGT) void fw_hub_batch(const fw_kargs a, const fw_
   __shared__ int32_t s_sel[kNW][64];
   __shared__ float s_w[16];
   __shared__ uint32_t s_task;
+  __shared__ int32_t s_schema[kApp == FW_APP_METAPATH ? FW_MAX_SCHEMA : 1];
 
   const int tid = (int)threadIdx.x;
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (kApp == FW_APP_METAPATH && threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < FW_MAX_SCHEMA; ++i) s_schema[i] = a.schema[i];
+  }
   const uint32_t ntasks = *h.ntasks;
   const uint32_t labels = (uint32_t)a.n_labels_per_hub;
   const uint32_t* __restrict__ bias =
@@ -835,7 +847,7 @@ __global__ __launch_bounds__(kWGT) void fw_hub_batch(const fw_kargs a, const fw_
     const int count = (int)(in_bucket < 64u ? in_bucket : 64u);
     const uint32_t rec_base = h.bucket_offset[bucket] + task.y;
     const int32_t v = h.hub_vertex[bucket / labels];
-    const int32_t want = kApp == FW_APP_METAPATH ? a.schema[bucket % labels] : 0;
+    const int32_t want = kApp == FW_APP_METAPATH ? s_schema[bucket % labels] : 0;
     const uint32_t off = a.xadj[v];
     const uint32_t deg = a.xadj[v + 1] - off;
     const uint32_t a0 = off & ~3u;
@@ -890,13 +902,11 @@ __global__ __launch_bounds__(kWGT) void fw_hub_batch(const fw_kargs a, const fw_
       if (!interior) {
 #pragma unroll
         for (int j = 0; j < kGroupQuartets; ++j) {
-          const uint32_t k = kb + 64u * (uint32_t)j;
-          const uint32_t base = a0 + 4u * k;
-          const bool ex = k < nq;
-          x[4 * j + 0] = (ex && base >= off && base < end) ? x[4 * j + 0] : 0.0f;
-          x[4 * j + 1] = (ex && base + 1u >= off && base + 1u < end) ? x[4 * j + 1] : 0.0f;
-          x[4 * j + 2] = (ex && base + 2u >= off && base + 2u < end) ? x[4 * j + 2] : 0.0f;
-          x[4 * j + 3] = (ex && base + 3u >= off && base + 3u < end) ? x[4 * j + 3] : 0.0f;
+          const uint32_t li = a0 + 4u * (kb + 64u * (uint32_t)j) - off;  // wraps below 0 for the head quartet
+          x[4 * j + 0] = li < deg ? x[4 * j + 0] : 0.0f;
+          x[4 * j + 1] = li + 1u < deg ? x[4 * j + 1] : 0.0f;
+          x[4 * j + 2] = li + 2u < deg ? x[4 * j + 2] : 0.0f;
+          x[4 * j + 3] = li + 3u < deg ? x[4 * j + 3] : 0.0f;
         }
       }
       float q = 0.0f;
