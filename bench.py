@@ -5,9 +5,12 @@ Default workload = the headline of BASELINE.json: DeepWalk, length 80, one query
 symmetrised R-MAT scale-24 graph (edge factor 16, a/b/c/d = .57/.19/.19/.05, weights U[1,100)).
 Inputs (CSR, start vertices, path matrix) are resident in HBM before the timed region starts.
 
-Prints ONE JSON line with the walk-steps/s of the whole job, the HBM roofline of the walk kernel
-(algorithmic bytes / kernel duration measured with HIP events on the launch stream) and the CPU
-oracle timed on the host cores of the same box over a bounded prefix of the same queries.
+Prints ONE JSON line with the walk-steps/s of the whole job, the HBM roofline of the walk path
+(algorithmic bytes of one pass / device time of that pass, measured with HIP events on the launch
+stream) and the CPU oracle timed on the host cores of the same box over a bounded prefix of the same
+queries.  With hub parking (the default for large batches) one pass is a short pipeline of launches --
+fw_walk_zprs, then per round fw_hub_batch + fw_walk_zprs -- and the HIP events bracket the whole
+pipeline, host-side round trips included.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 """
@@ -35,9 +38,10 @@ WORKLOADS = {
 }
 HEADLINE = "deepwalk_rmat24_sym"
 
-# HBM bytes per launch of the walk kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a
-# copy kernel of known size (see profiles/).  None until measured for that workload.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM-side bytes of one pass (all fw_walk_zprs + fw_hub_batch launches) from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs, each scaled by what the same counter reads for the 1 GiB copy kernel (profiles/).
+# None for workloads that have not been measured.
+MEASURED_TRAFFIC_BYTES = {"deepwalk_rmat24_sym": 2.225e12}
 
 
 def algorithmic_bytes(app, steps, sampled_edges, queries, probe_terms=0):
@@ -62,6 +66,10 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
     ap.add_argument("--hub-threshold", type=int, default=-1)
     ap.add_argument("--wg-threads", type=int, default=0)
+    ap.add_argument("--park-threshold", type=int, default=0, help="0 = library default, -1 = hub parking off")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run the plain copy kernel on 1 GiB (what rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE are "
+                         "scaled against)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -94,8 +102,16 @@ def main():
         params.hub_threshold = args.hub_threshold
     if args.wg_threads:
         params.wg_threads = args.wg_threads
+    params.park_threshold = args.park_threshold
     d_starts = fw.DeviceBuffer.from_numpy(starts)
     d_paths = fw.DeviceBuffer(n * params.max_depth * 4)
+
+    if args.calibration_copy:
+        src, dst = fw.DeviceBuffer(1 << 30), fw.DeviceBuffer(1 << 30)
+        fw.check(fw.lib().fw_dev_fill_i32(src.ptr, 7, (1 << 30) // 4))
+        fw.check(fw.lib().fw_dev_copy(dst.ptr, src.ptr, 1 << 30))  # fw_copy_u32x4_kernel: reads 1 GiB, writes 1 GiB
+        src.free()
+        dst.free()
 
     for _ in range(args.warmup):
         g.walk_device(params, d_starts, n, d_paths)
@@ -135,7 +151,8 @@ def main():
                 args.workload, wl["scale"], "symmetrised" if wl["sym"] else "directed", wl["app"], n, wl["depth"]),
             "vertices": g.V, "csr_entries": g.E, "queries": n,
             "walk_steps_per_pass": int(last.steps), "sampled_edges_per_pass": int(last.sampled_edges),
-            "wg_threads": params.wg_threads, "hub_threshold": params.hub_threshold, "grid": last.grid,
+            "wg_threads": params.wg_threads, "hub_threshold": params.hub_threshold,
+            "park_threshold": params.park_threshold, "launches_per_pass": last.launches, "grid": last.grid,
             "graph_gen_s": round(gen_s, 2),
         },
         "roofline": {
@@ -145,11 +162,23 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload if not args.scale else None),
-            "kernel": "fw_walk_zprs",
+            "kernel": "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_batch pipeline",
             "kernel_ms": avg_kernel_ms,
             "algorithmic_bytes": int(alg_bytes),
         },
     }
+    if last.launches > 1:
+        # per-kernel view of the last pass: each kernel's own HIP-event time and the algorithmic bytes of the steps
+        # it took (what every walker would have to read on its own; fw_hub_batch reads a hub list once per batch
+        # of up to 64 walkers, so its figure measures reuse, not DRAM speed)
+        walk_b = algorithmic_bytes(wl["app"], last.steps - last.hub_steps, last.sampled_edges - last.hub_sampled_edges, n)
+        hub_b = algorithmic_bytes(wl["app"], last.hub_steps, last.hub_sampled_edges, 0)
+        out["roofline"]["kernels"] = [
+            {"kernel": "fw_walk_zprs", "total_ms": last.walk_kernel_ms, "algorithmic_bytes": int(walk_b),
+             "achieved": walk_b / (last.walk_kernel_ms * 1e-3) / 1e9, "steps": int(last.steps - last.hub_steps)},
+            {"kernel": "fw_hub_batch", "total_ms": last.hub_kernel_ms, "algorithmic_bytes": int(hub_b),
+             "achieved": hub_b / (last.hub_kernel_ms * 1e-3) / 1e9, "steps": int(last.hub_steps)},
+        ]
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(fw, g, params, starts, args.cpu_seconds)

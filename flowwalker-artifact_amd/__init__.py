@@ -44,6 +44,8 @@ class WalkStats(C.Structure):
     _fields_ = [
         ("kernel_ms", C.c_double), ("total_ms", C.c_double), ("steps", C.c_uint64),
         ("sampled_edges", C.c_uint64), ("launches", C.c_int32), ("grid", C.c_int32),
+        ("walk_kernel_ms", C.c_double), ("hub_kernel_ms", C.c_double), ("hub_steps", C.c_uint64),
+        ("hub_sampled_edges", C.c_uint64),
     ]
 
 

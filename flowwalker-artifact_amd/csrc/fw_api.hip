@@ -567,8 +567,33 @@ static int32_t resolve_park_threshold(const fw_walk_params* p, int32_t n) {
 
 // Runs all walks of one batch on `stream`: a single walk launch, or the park / batch / resume loop.
 // `a` is complete except for the parking fields; a.dispenser / a.counters point at zeroed memory.
+struct KernelTimes {
+  double walk_ms = 0.0;
+  double hub_ms = 0.0;
+};
+
+// Records one event pair around a launch and adds its duration to *acc after the next stream sync.
+struct TimedLaunch {
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  int begin(hipStream_t s) {
+    FW_HIP(hipEventCreate(&e0));
+    FW_HIP(hipEventCreate(&e1));
+    FW_HIP(hipEventRecord(e0, s));
+    return FW_OK;
+  }
+  int end(hipStream_t s) { FW_HIP(hipEventRecord(e1, s)); return FW_OK; }
+  void collect(double* acc) {  // call after the stream has been synchronised
+    float ms = 0.0f;
+    if (e0 && e1 && hipEventElapsedTime(&ms, e0, e1) == hipSuccess) *acc += ms;
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    e0 = e1 = nullptr;
+  }
+};
+
 static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_kargs a, int32_t park_threshold,
-                             ParkBuffers* pb, hipStream_t stream, int* grid_used, int* launches) {
+                             ParkBuffers* pb, hipStream_t stream, int* grid_used, int* launches,
+                             KernelTimes* times) {
   *launches = 0;
   if (park_threshold == INT_MAX || g->n_hubs == 0 || pb == nullptr) {
     *launches = 1;
@@ -601,11 +626,16 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     FW_HIP(hipMemsetAsync(a.dispenser, 0, sizeof(uint32_t), stream));
     FW_HIP(hipMemsetAsync(pb->ctrs, 0, 4 * sizeof(uint32_t), stream));
     FW_HIP(hipMemsetAsync(pb->bucket_count, 0, (size_t)3 * pb->n_buckets * sizeof(uint32_t), stream));
-    int rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, iter == 0 ? grid_used : nullptr);
+    TimedLaunch tw;
+    int rc = tw.begin(stream);
     if (rc != FW_OK) return rc;
+    rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, iter == 0 ? grid_used : nullptr);
+    if (rc != FW_OK) return rc;
+    if ((rc = tw.end(stream)) != FW_OK) return rc;
     ++*launches;
     FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     FW_HIP(hipStreamSynchronize(stream));
+    tw.collect(&times->walk_ms);
     const uint32_t m = pb->h_ctrs[0];
     if (m == 0u) break;
     if ((size_t)m > pb->cap) { fw_set_error("internal: %u walkers parked, capacity %zu", m, pb->cap); return FW_ERR_INVALID; }
@@ -617,11 +647,15 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     hipLaunchKernelGGL(fw_scatter_parked_kernel, dim3(blocks), dim3(256), 0, stream, pb->parked, m, g->hub_index,
                        labels, p->app == FW_APP_METAPATH ? 1 : 0, bucket_offset, bucket_fill, pb->sorted_idx);
     FW_HIP(hipGetLastError());
+    TimedLaunch th;
+    if ((rc = th.begin(stream)) != FW_OK) return rc;
     rc = fw_launch_hub_batch(a, h, p->app, p->wg_threads, stream);
     if (rc != FW_OK) return rc;
+    if ((rc = th.end(stream)) != FW_OK) return rc;
     ++*launches;
     FW_HIP(hipMemcpyAsync(pb->h_ctrs + 1, pb->ctrs + 1, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     FW_HIP(hipStreamSynchronize(stream));
+    th.collect(&times->hub_ms);
     const uint32_t r = pb->h_ctrs[1];
     if (r == 0u) break;
     if ((size_t)r > pb->cap || r > (uint32_t)n_total) { fw_set_error("internal: %u walkers resumed, capacity %zu", r, pb->cap); return FW_ERR_INVALID; }
@@ -631,10 +665,10 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   return FW_OK;
 }
 
-struct Scratch {  // dispenser word + two 64-bit counters, 32 bytes per launch slot
+struct Scratch {  // dispenser word + workload counters of the two kernels, 48 bytes per launch slot
   uint32_t dispenser;
   uint32_t pad;
-  unsigned long long counters[2];
+  unsigned long long counters[4];
   unsigned long long pad2;
 };
 
@@ -690,8 +724,9 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
   a.dispenser = &d_scr->dispenser;
   a.counters = d_scr->counters;
   int grid_used = 0, launches = 0;
+  KernelTimes times;
   FW_TRY(hipEventRecord(ev0, stream));
-  rc = run_walk_launches(g, p, a, park_threshold, use_pb ? &pb : nullptr, stream, &grid_used, &launches);
+  rc = run_walk_launches(g, p, a, park_threshold, use_pb ? &pb : nullptr, stream, &grid_used, &launches, &times);
   if (rc != FW_OK) { cleanup(); return rc; }
   FW_TRY(hipEventRecord(ev1, stream));
   FW_TRY(hipStreamSynchronize(stream));
@@ -703,10 +738,14 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
   if (stats) {
     stats->kernel_ms = ms;
     stats->total_ms = now_ms() - t0;
-    stats->steps = h.counters[0];
-    stats->sampled_edges = h.counters[1];
+    stats->steps = h.counters[0] + h.counters[2];
+    stats->sampled_edges = h.counters[1] + h.counters[3];
     stats->launches = launches;
     stats->grid = grid_used;
+    stats->walk_kernel_ms = launches == 1 ? (double)ms : times.walk_ms;
+    stats->hub_kernel_ms = times.hub_ms;
+    stats->hub_steps = h.counters[2];
+    stats->hub_sampled_edges = h.counters[3];
   }
   return FW_OK;
 }
@@ -767,6 +806,7 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
   fw_kargs a;
   fill_kargs(&a, g, p);
   int grid_used = 0;
+  KernelTimes times;
   const double t0 = now_ms();
   for (int b = 0; b < nbatch; ++b) {
     const int s = b % nbuf;
@@ -784,7 +824,8 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     a.counters = d_scr[b].counters;
     FW_TRY(hipEventRecord(events[2 * b], streams[s]));
     int launches = 0;
-    rc = run_walk_launches(g, p, a, park_threshold, use_pb ? &pbs[s] : nullptr, streams[s], &grid_used, &launches);
+    rc = run_walk_launches(g, p, a, park_threshold, use_pb ? &pbs[s] : nullptr, streams[s], &grid_used, &launches,
+                           &times);
     if (rc != FW_OK) { cleanup(); return rc; }
     FW_TRY(hipEventRecord(events[2 * b + 1], streams[s]));
     FW_TRY(hipMemcpyAsync(h_paths + first * md, dp, (size_t)cnt * md * sizeof(int32_t), hipMemcpyDeviceToHost, streams[s]));
@@ -807,9 +848,18 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     stats->total_ms = total;
     stats->steps = 0;
     stats->sampled_edges = 0;
-    for (const Scratch& s : h) { stats->steps += s.counters[0]; stats->sampled_edges += s.counters[1]; }
+    stats->hub_steps = 0;
+    stats->hub_sampled_edges = 0;
+    for (const Scratch& s : h) {
+      stats->steps += s.counters[0] + s.counters[2];
+      stats->sampled_edges += s.counters[1] + s.counters[3];
+      stats->hub_steps += s.counters[2];
+      stats->hub_sampled_edges += s.counters[3];
+    }
     stats->launches = nbatch;
     stats->grid = grid_used;
+    stats->walk_kernel_ms = times.hub_ms == 0.0 && times.walk_ms == 0.0 ? kernel_ms : times.walk_ms;
+    stats->hub_kernel_ms = times.hub_ms;
   }
   return FW_OK;
 }

@@ -46,7 +46,7 @@ struct fw_kargs {
   const int32_t* starts;
   int32_t* paths;
   uint32_t* dispenser;          // one zeroed word per launch: the global query dispenser
-  unsigned long long* counters; // [0] steps, [1] sum of source degrees
+  unsigned long long* counters; // [0] steps, [1] sum of source degrees (walk kernel); [2], [3] the same for the hub batch kernel
   int32_t V;
   int32_t n;
   int32_t max_depth;

@@ -1016,9 +1016,9 @@ __global__ __launch_bounds__(kWGT) void fw_hub_batch(const fw_kargs a, const fw_
       }
     }
   }
-  if (n_steps != 0ull) {
-    atomicAdd(&a.counters[0], n_steps);
-    atomicAdd(&a.counters[1], n_edges);
+  if (n_steps != 0ull) {  // the hub kernel's share is counted apart and added up by the host
+    atomicAdd(&a.counters[2], n_steps);
+    atomicAdd(&a.counters[3], n_edges);
   }
 }
 

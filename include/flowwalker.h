@@ -74,6 +74,11 @@ typedef struct {
   uint64_t sampled_edges; /* "Total sampled edge": sum over steps of deg(source) */
   int32_t launches;       /* fw_walk_batch: batches; fw_walk_device: walk + hub-batch kernel launches */
   int32_t grid;           /* workgroups per launch actually used */
+  /* per-kernel breakdown of kernel_ms / steps / sampled_edges (hub parking splits a pass over two kernels) */
+  double walk_kernel_ms;      /* sum over fw_walk_zprs launches */
+  double hub_kernel_ms;       /* sum over fw_hub_batch launches */
+  uint64_t hub_steps;         /* steps taken in fw_hub_batch (included in steps) */
+  uint64_t hub_sampled_edges; /* their source degrees (included in sampled_edges) */
 } fw_walk_stats;
 
 typedef struct fw_graph fw_graph; /* device CSR mirror: include/gpu_graph.cuh:28-78 */
