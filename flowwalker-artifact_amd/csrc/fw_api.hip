@@ -8,9 +8,13 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <cstring>
+
 #include <chrono>
 #include <new>
 #include <vector>
+
+#include <rocprim/rocprim.hpp>
 
 #include "fw_internal.h"
 
@@ -474,95 +478,165 @@ static int ensure_hub_index(fw_graph* g, int32_t threshold) {
   return FW_OK;
 }
 
-// One workgroup: exclusive scan of the bucket counts, and one task per 64 parked walkers of a bucket.
-// ctrs[2] = number of tasks (out).
-__global__ __launch_bounds__(1024) void fw_bucket_scan_kernel(const uint32_t* __restrict__ bucket_count,
-                                                              uint32_t* bucket_offset, int n_buckets, uint2* tasks,
-                                                              uint32_t* ctrs) {
-  __shared__ uint32_t partial[1024];
-  const int tid = (int)threadIdx.x;
-  const int per = (n_buckets + 1023) / 1024;
-  const int lo = tid * per;
-  const int hi = lo + per < n_buckets ? lo + per : n_buckets;
-  uint32_t sum = 0;
-  for (int b = lo; b < hi; ++b) sum += bucket_count[b];
-  partial[tid] = sum;
-  __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {  // Hillis-Steele inclusive scan over the 1024 partial sums
-    const uint32_t add = tid >= off ? partial[tid - off] : 0u;
-    __syncthreads();
-    partial[tid] += add;
-    __syncthreads();
-  }
-  uint32_t run = partial[tid] - sum;  // exclusive prefix of this thread's chunk
-  for (int b = lo; b < hi; ++b) {
-    const uint32_t c = bucket_count[b];
-    bucket_offset[b] = run;
-    run += c;
+// Default parking rule (batches of at least kMinParkBatch queries): park on vertices where about kParkMeet or more
+// walkers of the batch stand at the same time.  With n walkers spread in proportion to degree over E adjacency
+// entries, a vertex of degree d holds about n * d / E of them, so the threshold is kParkMeet * E / n, not below
+// kMinDefaultPark (shorter lists cost less to read than a record costs to move).
+constexpr int32_t kMinParkBatch = 65536;
+constexpr double kParkMeet = 4.0;
+constexpr int32_t kMinDefaultPark = 64;
+constexpr int32_t kMinParkThreshold = 1;
+
+// One task per 64 parked walkers of a bucket: a workgroup task when the bucket's vertex is sampled at workgroup
+// granularity (degree above hub_threshold), a wave task otherwise.  ctrs[3] / ctrs[5] = number of tasks (out).
+__global__ __launch_bounds__(256) void fw_bucket_tasks_kernel(const uint32_t* __restrict__ bucket_count,
+                                       const uint32_t* __restrict__ bucket_offset, int n_buckets, int labels,
+                                       const int32_t* __restrict__ hub_vertex, const uint32_t* __restrict__ xadj,
+                                       int32_t hub_threshold, fw_batch_task* tasks, fw_batch_task* wtasks,
+                                       uint32_t* ctrs) {
+  const int stride = gridDim.x * blockDim.x;
+  const int lane = (int)(threadIdx.x & 63u);
+  const int rounds = (n_buckets + stride - 1) / stride;  // every lane runs every round: the wave scans need all 64
+  for (int r = 0; r < rounds; ++r) {
+    const int b = r * stride + (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    const uint32_t c = b < n_buckets ? bucket_count[b] : 0u;
+    fw_batch_task t;
+    t.v = 0; t.off = 0; t.deg = 0; t.slot = 0; t.rec_base = 0; t.count = 0;
+    t.pad[0] = t.pad[1] = 0;
+    bool wg = false;
     if (c != 0u) {
-      const uint32_t nb = (c + 63u) >> 6;
-      const uint32_t t0 = atomicAdd(&ctrs[2], nb);
-      for (uint32_t k = 0; k < nb; ++k) tasks[t0 + k] = make_uint2((uint32_t)b, k * 64u);
+      t.v = hub_vertex[b / labels];
+      t.off = xadj[t.v];
+      t.deg = xadj[t.v + 1] - t.off;
+      t.slot = b % labels;
+      wg = (int32_t)t.deg > hub_threshold;
+    }
+    const uint32_t nb = (c + 63u) >> 6;
+    // task slots: one counter update per wave and kind instead of one per bucket (the counters are contended)
+    uint32_t xw = wg ? nb : 0u, xs = wg ? 0u : nb;
+    uint32_t iw = xw, is = xs;  // inclusive wave scans
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const uint32_t uw = __shfl_up(iw, d);
+      const uint32_t us = __shfl_up(is, d);
+      if (lane >= d) { iw += uw; is += us; }
+    }
+    const uint32_t tw = __shfl(iw, 63), ts = __shfl(is, 63);
+    uint32_t bw = 0u, bs = 0u;
+    if (lane == 63) {
+      if (tw != 0u) bw = atomicAdd(&ctrs[3], tw);
+      if (ts != 0u) bs = atomicAdd(&ctrs[5], ts);
+    }
+    bw = __shfl(bw, 63);
+    bs = __shfl(bs, 63);
+    if (c != 0u) {
+      const uint32_t t0 = wg ? bw + iw - xw : bs + is - xs;
+      fw_batch_task* out = wg ? tasks : wtasks;
+      const uint32_t base = bucket_offset[b];
+      for (uint32_t k = 0; k < nb; ++k) {
+        t.rec_base = base + 64u * k;
+        t.count = (int32_t)(c - 64u * k < 64u ? c - 64u * k : 64u);
+        out[t0 + k] = t;
+      }
     }
   }
 }
 
-__global__ void fw_scatter_parked_kernel(const fw_walker_rec* __restrict__ parked, uint32_t m,
+// Counting-sort scatter of a round's parked walkers into `sorted`.  Two sources share a bucket's range:
+//  * the previous batch launch's output list, of which only the records tagged FW_REC_PARK are parked; they carry
+//    their position inside the bucket (taken when they were parked) and fill the range from its start;
+//  * the walk kernel's list, whose records were only counted; they take positions from the end of the range here.
+__global__ void fw_scatter_tagged_kernel(const fw_walker_rec* __restrict__ src, uint32_t m,
                                          const int32_t* __restrict__ hub_index, int labels, int metapath,
-                                         const uint32_t* __restrict__ bucket_offset, uint32_t* bucket_fill,
-                                         uint32_t* sorted_idx) {
+                                         const uint32_t* __restrict__ bucket_offset,
+                                         fw_walker_rec* __restrict__ sorted) {
   const uint32_t stride = gridDim.x * blockDim.x;
   for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < m; i += stride) {
-    const fw_walker_rec r = parked[i];
+    fw_walker_rec r = src[i];
+    if (r.q < 0 || (r.len & FW_REC_PARK) == 0) continue;
+    r.len &= ~FW_REC_PARK;
     const uint32_t slot = metapath ? (uint32_t)(r.len - 1) % (uint32_t)labels : 0u;
     const uint32_t b = (uint32_t)hub_index[r.cur] * (uint32_t)labels + slot;
-    sorted_idx[bucket_offset[b] + atomicAdd(&bucket_fill[b], 1u)] = i;
+    sorted[bucket_offset[b] + (uint32_t)r.prev] = r;
   }
 }
 
-// Device buffers of one park / batch / resume loop (one per stream in flight).
+__global__ void fw_scatter_counted_kernel(const fw_walker_rec* __restrict__ src, uint32_t m,
+                                          const int32_t* __restrict__ hub_index, int labels, int metapath,
+                                          const uint32_t* __restrict__ bucket_count,
+                                          const uint32_t* __restrict__ bucket_offset, uint32_t* bucket_fill,
+                                          fw_walker_rec* __restrict__ sorted) {
+  const uint32_t stride = gridDim.x * blockDim.x;
+  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < m; i += stride) {
+    const fw_walker_rec r = src[i];
+    const uint32_t slot = metapath ? (uint32_t)(r.len - 1) % (uint32_t)labels : 0u;
+    const uint32_t b = (uint32_t)hub_index[r.cur] * (uint32_t)labels + slot;
+    sorted[bucket_offset[b] + bucket_count[b] - 1u - atomicAdd(&bucket_fill[b], 1u)] = r;
+  }
+}
+
+// Device buffers of one park / batch / resume loop (one per stream in flight).  Three record lists: `walked`
+// (walkers parked by the walk kernel), `sorted` (a round's parked walkers grouped by bucket, the batch kernel's
+// input) and `out` (the batch kernel's output, one record per input record: finished / resumes / parked again).
+// The bucket counts are double buffered: a round's batch and walk launches count the next round's walkers.
 struct ParkBuffers {
   size_t cap = 0;       // walkers
   int n_buckets = 0;
-  fw_walker_rec* parked = nullptr;
-  fw_walker_rec* resume = nullptr;
-  uint32_t* sorted_idx = nullptr;
-  uint32_t* bucket_count = nullptr;   // [3 * n_buckets]: count, offset, fill
-  uint2* tasks = nullptr;
-  uint32_t* ctrs = nullptr;           // [0] parked, [1] resumed, [2] tasks, [3] task dispenser
-  uint32_t* h_ctrs = nullptr;         // pinned mirror of ctrs[0..1]
+  fw_walker_rec* walked = nullptr;
+  fw_walker_rec* sorted = nullptr;
+  fw_walker_rec* out = nullptr;
+  uint32_t* buckets = nullptr;        // [4 * n_buckets]: count of round parity 0, of parity 1, offset, fill
+  fw_batch_task* tasks = nullptr;
+  fw_batch_task* wtasks = nullptr;
+  uint32_t* ctrs = nullptr;           // [0] walkers in `walked`, [1] records of `out` that resume, [2] that are parked
+                                      // again, [3] workgroup tasks, [4] their dispenser, [5] wave tasks
+  uint32_t* h_ctrs = nullptr;         // pinned mirror
+  void* tmp = nullptr;                // scan temporary storage
+  size_t scan_bytes = 0;
 
-  int alloc(size_t walkers, int buckets) {
+  uint32_t* count(int parity) const { return buckets + (size_t)parity * n_buckets; }
+  uint32_t* offset() const { return buckets + (size_t)2 * n_buckets; }
+  uint32_t* fill() const { return buckets + (size_t)3 * n_buckets; }
+
+  int alloc(size_t walkers, int n) {
     cap = walkers;
-    n_buckets = buckets;
-    FW_HIP(hipMalloc(reinterpret_cast<void**>(&parked), cap * sizeof(fw_walker_rec)));
-    FW_HIP(hipMalloc(reinterpret_cast<void**>(&resume), cap * sizeof(fw_walker_rec)));
-    FW_HIP(hipMalloc(reinterpret_cast<void**>(&sorted_idx), cap * sizeof(uint32_t)));
-    FW_HIP(hipMalloc(reinterpret_cast<void**>(&bucket_count), (size_t)3 * buckets * sizeof(uint32_t)));
-    FW_HIP(hipMalloc(reinterpret_cast<void**>(&tasks), (cap / 64 + (size_t)buckets + 1) * sizeof(uint2)));
-    FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), 4 * sizeof(uint32_t)));
-    FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), 4 * sizeof(uint32_t), hipHostMallocDefault));
+    n_buckets = n;
+    const size_t ntask = cap / 64 + (size_t)n + 1;
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&walked), cap * sizeof(fw_walker_rec)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&sorted), cap * sizeof(fw_walker_rec)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&out), cap * sizeof(fw_walker_rec)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&buckets), (size_t)4 * n * sizeof(uint32_t)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&tasks), ntask * sizeof(fw_batch_task)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&wtasks), ntask * sizeof(fw_batch_task)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), 8 * sizeof(uint32_t)));
+    FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), 8 * sizeof(uint32_t), hipHostMallocDefault));
+    FW_HIP(rocprim::exclusive_scan(nullptr, scan_bytes, count(0), offset(), 0u, (size_t)n,
+                                   rocprim::plus<uint32_t>(), (hipStream_t)0));
+    FW_HIP(hipMalloc(&tmp, scan_bytes ? scan_bytes : 16));
     return FW_OK;
   }
   void release() {
-    void* dev[6] = {parked, resume, sorted_idx, bucket_count, tasks, ctrs};
+    void* dev[8] = {walked, sorted, out, buckets, tasks, wtasks, ctrs, tmp};
     for (void* p : dev) if (p) (void)hipFree(p);
     if (h_ctrs) (void)hipHostFree(h_ctrs);
-    parked = resume = nullptr; sorted_idx = bucket_count = ctrs = h_ctrs = nullptr; tasks = nullptr;
+    walked = sorted = out = nullptr;
+    buckets = ctrs = h_ctrs = nullptr;
+    tasks = wtasks = nullptr;
+    tmp = nullptr;
   }
 };
 
 // Decides whether a call parks walkers, and at which degree.  Returns INT_MAX for "no".
-static int32_t resolve_park_threshold(const fw_walk_params* p, int32_t n) {
+static int32_t resolve_park_threshold(const fw_graph* g, const fw_walk_params* p, int32_t n) {
   if (p->app == FW_APP_NODE2VEC) return INT_MAX;  // its biases depend on the walker: nothing to share
   if (p->park_threshold < 0) return INT_MAX;
   if (p->park_threshold == 0) {
-    // default: only batches large enough for walkers to meet on hubs
-    if (n < 65536) return INT_MAX;
-    return p->hub_threshold > 4096 ? p->hub_threshold : 4096;
+    if (n < kMinParkBatch) return INT_MAX;  // too few walkers to meet
+    const double t = kParkMeet * (double)g->E / (double)n;
+    if (t >= 2.0e9) return INT_MAX;
+    return t < (double)kMinDefaultPark ? kMinDefaultPark : (int32_t)t;
   }
-  // parked hubs are sampled at workgroup granularity, so they must be above the wave / workgroup threshold
-  return p->park_threshold > p->hub_threshold ? p->park_threshold : p->hub_threshold;
+  return p->park_threshold < kMinParkThreshold ? kMinParkThreshold : p->park_threshold;
 }
 
 // Runs all walks of one batch on `stream`: a single walk launch, or the park / batch / resume loop.
@@ -600,67 +674,104 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     return fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, grid_used);
   }
   const int labels = p->app == FW_APP_METAPATH ? p->schema_len : 1;
-  const int32_t n_total = a.n;
+  const int metapath = p->app == FW_APP_METAPATH ? 1 : 0;
+  const size_t bucket_bytes = (size_t)pb->n_buckets * sizeof(uint32_t);
   a.park_threshold = park_threshold;
   a.n_labels_per_hub = labels;
   a.hub_index = g->hub_index;
-  a.parked = pb->parked;
+  a.parked = pb->walked;
   a.parked_count = &pb->ctrs[0];
-  a.bucket_count = pb->bucket_count;
-  uint32_t* bucket_offset = pb->bucket_count + pb->n_buckets;
-  uint32_t* bucket_fill = pb->bucket_count + 2 * pb->n_buckets;
   fw_hub_args h;
-  h.parked = pb->parked;
-  h.sorted_idx = pb->sorted_idx;
-  h.bucket_count = pb->bucket_count;
-  h.bucket_offset = bucket_offset;
+  h.sorted = pb->sorted;
   h.tasks = pb->tasks;
-  h.ntasks = &pb->ctrs[2];
-  h.task_next = &pb->ctrs[3];
-  h.hub_vertex = g->hub_vertex;
-  h.resume = pb->resume;
-  h.resume_count = &pb->ctrs[1];
+  h.ntasks = &pb->ctrs[3];
+  h.task_next = &pb->ctrs[4];
+  h.wtasks = pb->wtasks;
+  h.nwtasks = &pb->ctrs[5];
+  h.out = pb->out;
+  h.out_counts = &pb->ctrs[1];
 
-  a.resume = nullptr;
-  for (int iter = 0;; ++iter) {
-    FW_HIP(hipMemsetAsync(a.dispenser, 0, sizeof(uint32_t), stream));
-    FW_HIP(hipMemsetAsync(pb->ctrs, 0, 4 * sizeof(uint32_t), stream));
-    FW_HIP(hipMemsetAsync(pb->bucket_count, 0, (size_t)3 * pb->n_buckets * sizeof(uint32_t), stream));
+  // One walk launch and the read-back of the counters.
+  auto walk = [&](int* grid_out) -> int {
+    FW_HIP(hipMemsetAsync(a.dispenser, 0, sizeof(uint32_t), stream));  // used by the launch of fresh queries only
+    FW_HIP(hipMemsetAsync(pb->ctrs, 0, sizeof(uint32_t), stream));
     TimedLaunch tw;
     int rc = tw.begin(stream);
     if (rc != FW_OK) return rc;
-    rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, iter == 0 ? grid_used : nullptr);
+    rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, grid_out);
     if (rc != FW_OK) return rc;
     if ((rc = tw.end(stream)) != FW_OK) return rc;
     ++*launches;
-    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, 8 * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     FW_HIP(hipStreamSynchronize(stream));
     tw.collect(&times->walk_ms);
-    const uint32_t m = pb->h_ctrs[0];
+    return FW_OK;
+  };
+
+  // first walk launch: fresh queries; the walkers it parks are counted in bucket array 0
+  int cur = 0;
+  FW_HIP(hipMemsetAsync(pb->ctrs, 0, 8 * sizeof(uint32_t), stream));
+  FW_HIP(hipMemsetAsync(pb->count(0), 0, bucket_bytes, stream));
+  a.resume = nullptr;
+  a.bucket_count = pb->count(0);
+  int rc = walk(grid_used);
+  if (rc != FW_OK) return rc;
+  uint32_t n_out = 0;  // records in `out` (the previous batch launch's input size)
+  for (;;) {
+    const uint32_t n_walked = pb->h_ctrs[0];                 // parked by the walk launch
+    const uint32_t n_again = n_out ? pb->h_ctrs[2] : 0u;     // parked again by the previous batch launch
+    const uint64_t m = (uint64_t)n_walked + n_again;
     if (m == 0u) break;
-    if ((size_t)m > pb->cap) { fw_set_error("internal: %u walkers parked, capacity %zu", m, pb->cap); return FW_ERR_INVALID; }
-    hipLaunchKernelGGL(fw_bucket_scan_kernel, dim3(1), dim3(1024), 0, stream, pb->bucket_count, bucket_offset,
-                       pb->n_buckets, pb->tasks, pb->ctrs);
+    if (m > pb->cap) { fw_set_error("internal: %llu walkers parked, capacity %zu", (unsigned long long)m, pb->cap); return FW_ERR_INVALID; }
+    const int nxt = cur ^ 1;
+    // group the round's walkers by bucket and cut the buckets into tasks; clear the next round's counts
+    FW_HIP(rocprim::exclusive_scan(pb->tmp, pb->scan_bytes, pb->count(cur), pb->offset(), 0u, (size_t)pb->n_buckets,
+                                   rocprim::plus<uint32_t>(), stream));
+    auto blocks_for = [](uint32_t cnt) {
+      unsigned blocks = (cnt + 255u) / 256u;
+      return blocks > 8192u ? 8192u : blocks;
+    };
+    if (n_out != 0u)
+      hipLaunchKernelGGL(fw_scatter_tagged_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
+                         g->hub_index, labels, metapath, pb->offset(), pb->sorted);
+    if (n_walked != 0u) {
+      FW_HIP(hipMemsetAsync(pb->fill(), 0, bucket_bytes, stream));
+      hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_walked)), dim3(256), 0, stream, pb->walked,
+                         n_walked, g->hub_index, labels, metapath, pb->count(cur), pb->offset(), pb->fill(),
+                         pb->sorted);
+    }
     FW_HIP(hipGetLastError());
-    unsigned blocks = (m + 255u) / 256u;
-    if (blocks > 4096u) blocks = 4096u;
-    hipLaunchKernelGGL(fw_scatter_parked_kernel, dim3(blocks), dim3(256), 0, stream, pb->parked, m, g->hub_index,
-                       labels, p->app == FW_APP_METAPATH ? 1 : 0, bucket_offset, bucket_fill, pb->sorted_idx);
+    FW_HIP(hipMemsetAsync(pb->ctrs + 1, 0, 7 * sizeof(uint32_t), stream));
+    FW_HIP(hipMemsetAsync(pb->count(nxt), 0, bucket_bytes, stream));
+    unsigned tblocks = ((unsigned)pb->n_buckets + 255u) / 256u;
+    if (tblocks > 2048u) tblocks = 2048u;
+    hipLaunchKernelGGL(fw_bucket_tasks_kernel, dim3(tblocks), dim3(256), 0, stream, pb->count(cur), pb->offset(),
+                       pb->n_buckets, labels, g->hub_vertex, g->xadj, p->hub_threshold, pb->tasks, pb->wtasks,
+                       pb->ctrs);
     FW_HIP(hipGetLastError());
+    h.bucket_out = pb->count(nxt);
     TimedLaunch th;
     if ((rc = th.begin(stream)) != FW_OK) return rc;
     rc = fw_launch_hub_batch(a, h, p->app, p->wg_threads, stream);
     if (rc != FW_OK) return rc;
     if ((rc = th.end(stream)) != FW_OK) return rc;
     ++*launches;
-    FW_HIP(hipMemcpyAsync(pb->h_ctrs + 1, pb->ctrs + 1, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, 8 * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     FW_HIP(hipStreamSynchronize(stream));
     th.collect(&times->hub_ms);
-    const uint32_t r = pb->h_ctrs[1];
-    if (r == 0u) break;
-    if ((size_t)r > pb->cap || r > (uint32_t)n_total) { fw_set_error("internal: %u walkers resumed, capacity %zu", r, pb->cap); return FW_ERR_INVALID; }
-    a.resume = pb->resume;
-    a.n = (int32_t)r;
+    n_out = (uint32_t)m;
+    pb->h_ctrs[0] = 0u;
+    if (pb->h_ctrs[1] != 0u) {
+      // walkers on vertices below the threshold continue in the walk kernel, which takes them from the batch
+      // output list (skipping the other records) and counts the walkers it parks in the same bucket array
+      a.resume = pb->out;
+      a.n = (int32_t)n_out;
+      a.bucket_count = pb->count(nxt);
+      const uint32_t n_again_now = pb->h_ctrs[2];
+      if ((rc = walk(nullptr)) != FW_OK) return rc;
+      pb->h_ctrs[2] = n_again_now;  // unchanged by the walk launch; kept explicit for the next round
+    }
+    cur = nxt;
   }
   return FW_OK;
 }
@@ -684,7 +795,7 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
   hipStream_t stream = reinterpret_cast<hipStream_t>(stream_v);
   const double t0 = now_ms();
 
-  const int32_t park_threshold = resolve_park_threshold(p, n);
+  const int32_t park_threshold = resolve_park_threshold(g, p, n);
   ParkBuffers pb;
   bool use_pb = false;
   if (park_threshold != INT_MAX) {
@@ -766,7 +877,7 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
   const size_t bs = batch_size;
   const size_t md = (size_t)p->max_depth;
 
-  const int32_t park_threshold = resolve_park_threshold(p, (int32_t)bs);
+  const int32_t park_threshold = resolve_park_threshold(g, p, (int32_t)bs);
   bool use_pb = false;
   if (park_threshold != INT_MAX) {
     rc = ensure_hub_index(const_cast<fw_graph*>(g), park_threshold);

@@ -33,7 +33,7 @@ constexpr int FW_EDGE_PAD = 4;
 struct fw_walker_rec {
   int32_t q;     // query index inside the launch (walker id = walker_base + q)
   int32_t cur;   // current vertex
-  int32_t prev;  // previous vertex or -1
+  int32_t prev;  // previous vertex or -1; in a parked record: its position inside the bucket of `cur`
   int32_t len;   // path entries written so far
 };
 
@@ -67,18 +67,35 @@ struct fw_kargs {
   const fw_walker_rec* resume;       // in: walkers to continue instead of fresh queries (NULL: use starts)
 };
 
-// Arguments of the hub batch kernel: one workgroup serves up to 64 parked walkers of one hub with one scan.
+// Tag in fw_walker_rec::len of a batch-kernel output record whose vertex is parked on again (stripped by readers).
+constexpr int32_t FW_REC_PARK = 0x40000000;
+
+// One batch: up to 64 walkers parked on vertex v, records sorted[rec_base .. rec_base + count).  32 bytes.
+struct fw_batch_task {
+  int32_t v;
+  uint32_t off;       // xadj[v]
+  uint32_t deg;
+  uint32_t rec_base;
+  int32_t count;
+  int32_t slot;       // metapath: position in the schema of the label these walkers want
+  int32_t pad[2];
+};
+
+// Arguments of the hub batch kernel: up to 64 walkers parked on one vertex are served with one scan of its list,
+// by a workgroup (degree above hub_threshold: workgroup-granularity sampling) or by a single wave.
 struct fw_hub_args {
-  const fw_walker_rec* parked;
-  const uint32_t* sorted_idx;        // parked record indices grouped by bucket
-  const uint32_t* bucket_count;
-  const uint32_t* bucket_offset;
-  const uint2* tasks;                // (bucket, first walker of the batch inside the bucket)
+  const fw_walker_rec* sorted;       // parked records grouped by bucket
+  const fw_batch_task* tasks;        // workgroup tasks, handed out through task_next
   const uint32_t* ntasks;
-  uint32_t* task_next;               // task dispenser
-  const int32_t* hub_vertex;
-  fw_walker_rec* resume;             // out: walkers that continue
-  uint32_t* resume_count;
+  uint32_t* task_next;
+  const fw_batch_task* wtasks;       // wave tasks, wave i of the grid takes i, i + waves, ...
+  const uint32_t* nwtasks;
+  // out[rec_base + i] = walker i of the batch after its step: q = -1 when its walk is over, len tagged with
+  // FW_REC_PARK when its new vertex is parked on again (bucket_out counts those, prev = position inside the
+  // bucket), untagged otherwise
+  fw_walker_rec* out;
+  uint32_t* bucket_out;
+  uint32_t* out_counts;              // [0] += records that resume, [1] += records parked again
 };
 
 void fw_set_error(const char* fmt, ...);

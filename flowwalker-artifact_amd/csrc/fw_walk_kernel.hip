@@ -82,6 +82,24 @@ __device__ __forceinline__ float wave_scan(float x) {
   return x;
 }
 
+// Inclusive prefix maximum over the 64 lanes of non-negative values (same network as wave_scan; max is exact,
+// so its association order does not matter).
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_max(float x) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(x), kCtrl, kRowMask, 0xF, false);
+  return fmaxf(x, __int_as_float(moved));
+}
+
+__device__ __forceinline__ float wave_prefix_max(float x) {
+  x = dpp_max<0x111, 0xF>(x);
+  x = dpp_max<0x112, 0xF>(x);
+  x = dpp_max<0x114, 0xF>(x);
+  x = dpp_max<0x118, 0xF>(x);
+  x = dpp_max<0x142, 0xA>(x);
+  x = dpp_max<0x143, 0xC>(x);
+  return x;
+}
+
 // Inclusive scan inside each 16-lane row only.
 __device__ __forceinline__ float row_scan(float x) {
   x = dpp_add<0x111, 0xF>(x);
@@ -266,8 +284,8 @@ __device__ __forceinline__ float next_uniform(DrawQueue& d, const fw_kargs& a, c
 // vertex.  Outputs: running total S of the wave's groups, selected local index (or -1), its vertex.
 template <int kApp, int kJ, bool kTrackV>
 __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c, const int lane, const uint32_t w,
-                                            const uint32_t nw, N2vScratch* scr, float& S_out, int32_t& sel_out,
-                                            int32_t& selv_out) {
+                                            const uint32_t nw, N2vScratch* scr, const DrawQueue& dq0, float& S_out,
+                                            int32_t& sel_out, int32_t& selv_out) {
   constexpr uint32_t kG = 64u * kGroupQuartets;  // quartets per group
   constexpr int kEl = 4 * kJ;
   const uint32_t a0 = c.off & ~3u;
@@ -290,7 +308,7 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
 
   float S = 0.0f, Sj = 0.0f, u = 1.0f;
   int32_t sel = -1, selv = -1;
-  DrawQueue dq;
+  DrawQueue dq = dq0;  // empty, or block 0 of this wave's stream computed ahead by the slot's own thread
   uint32_t seg_lo = 0u;  // node2vec: entries of N(prev) below this index are smaller than anything still to come
 
   for (uint32_t g = w; g < ngroups; g += nw) {
@@ -493,6 +511,9 @@ struct TaskTable {
   uint32_t prev_off[kWGT];
   int32_t prev_deg[kWGT];
   int32_t flag[kWGT];
+  // Philox block 0 of stream 0 for the slot's next step, computed by the slot's own thread in phase C (64 blocks
+  // per vector instruction instead of one block per scalar instruction stream)
+  uint32_t draw[4][kWGT];
   // per-round work lists, double buffered by round parity
   int32_t small_list[2][kWGT];
   int32_t hub_list[2][kWGT];
@@ -500,6 +521,8 @@ struct TaskTable {
   int32_t hub_count[2];
   int32_t claim[2];
   int32_t exhausted;
+  uint32_t cursor;            // resume lists: entries of this workgroup's share handed out so far
+  unsigned long long acc[2];  // steps, sum of source degrees of this workgroup
   // wave partials of the hub chunk in flight
   float hub_w[kHubChunk][16];
   int32_t hub_sel[kHubChunk][16];
@@ -570,6 +593,8 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
     tt.hub_count[0] = tt.hub_count[1] = 0;
     tt.claim[0] = tt.claim[1] = 0;
     tt.exhausted = 0;
+    tt.cursor = 0u;
+    tt.acc[0] = tt.acc[1] = 0ull;
   }
   __syncthreads();
 
@@ -590,7 +615,8 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
           if (kApp == FW_APP_METAPATH) c.want = tt.schema[c.step % (uint32_t)a.schema_len];
           float W;
           int32_t sel, selv;
-          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, (uint32_t)wave, (uint32_t)kNW, scr, W, sel, selv);
+          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, (uint32_t)wave, (uint32_t)kNW, scr, DrawQueue(), W, sel,
+                                                   selv);
           if (lane == 0) {
             tt.hub_w[h][wave] = W;
             tt.hub_sel[h][wave] = sel;
@@ -642,11 +668,18 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
         int32_t sel, selv;
         const uint32_t nq = ((c.off + (uint32_t)c.deg) - (c.off & ~3u) + 3u) >> 2;
         int32_t v = -1;
+        DrawQueue dq0;
+        dq0.q0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)tt.draw[0][slot]);
+        dq0.q1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)tt.draw[1][slot]);
+        dq0.q2 = (uint32_t)__builtin_amdgcn_readfirstlane((int)tt.draw[2][slot]);
+        dq0.q3 = (uint32_t)__builtin_amdgcn_readfirstlane((int)tt.draw[3][slot]);
+        dq0.avail = 4u;
+        dq0.blk = 1u;
         if (nq <= 64u) {  // one quartet per lane: fetch the adjacency with the biases, no dependent load
-          wave_stream<kApp, 1, true>(a, c, lane, 0u, 1u, scr, W, sel, selv);
+          wave_stream<kApp, 1, true>(a, c, lane, 0u, 1u, scr, dq0, W, sel, selv);
           v = selv;
         } else {
-          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, 0u, 1u, scr, W, sel, selv);
+          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, 0u, 1u, scr, dq0, W, sel, selv);
           if (sel >= 0) v = a.adjncy[c.off + (uint32_t)sel];
         }
         if (lane == 0) commit(a, tt, slot, c, v, sel >= 0, n_steps, n_edges);
@@ -705,6 +738,8 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
             rec.prev = tt.prev[tid];
             rec.len = len;
             a.parked[at] = rec;
+            // counted only: the wave does not wait for a position inside the bucket (the counters of the busiest
+            // vertices are contended); the counting sort hands the positions out later
             const uint32_t label_slot =
                 kApp == FW_APP_METAPATH ? (uint32_t)(len - 1) % (uint32_t)a.n_labels_per_hub : 0u;
             atomicAdd(&a.bucket_count[(uint32_t)a.hub_index[v] * (uint32_t)a.n_labels_per_hub + label_slot], 1u);
@@ -718,15 +753,29 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
         if (m == 0ull) break;
         uint32_t base = 0;
         const int leader = __builtin_ctzll(m);
-        if (lane == leader) base = atomicAdd(a.dispenser, (uint32_t)__builtin_popcountll(m));
+        if (lane == leader) {
+          // fresh queries come from the global dispenser (include/walker.cuh:1339,1423); the entries of a resume
+          // list are dealt out by position -- the workgroups take interleaved chunks of slot_limit entries -- with
+          // a workgroup-local cursor, because a list is long (it has holes) and a global counter is contended
+          base = a.resume != nullptr ? atomicAdd(&tt.cursor, (uint32_t)__builtin_popcountll(m))
+                                     : atomicAdd(a.dispenser, (uint32_t)__builtin_popcountll(m));
+        }
         base = (uint32_t)__builtin_amdgcn_readlane((int)base, leader);
         if (want) {
-          const uint32_t q = base + (uint32_t)__builtin_popcountll(m & ((1ull << lane) - 1ull));
+          uint32_t q = base + (uint32_t)__builtin_popcountll(m & ((1ull << lane) - 1ull));
+          if (a.resume != nullptr) {
+            const uint32_t chunk = q / (uint32_t)a.slot_limit;
+            const uint64_t pos = ((uint64_t)chunk * gridDim.x + blockIdx.x) * (uint64_t)a.slot_limit +
+                                 (q - chunk * (uint32_t)a.slot_limit);
+            q = pos < (uint64_t)(uint32_t)a.n ? (uint32_t)pos : 0xFFFFFFFFu;
+          }
           if (q < (uint32_t)a.n) {
             int32_t wq, sp, pv, ln;
-            if (a.resume != nullptr) {  // a walker coming back from its hub step
+            if (a.resume != nullptr) {  // a walker coming back from its batch step
               const fw_walker_rec rec = a.resume[q];
               wq = rec.q; sp = rec.cur; pv = rec.prev; ln = rec.len;
+              // the list has holes: walks that ended, and walkers that wait on their next vertex already
+              if (rec.q < 0 || (rec.len & FW_REC_PARK) != 0) sp = -1;
             } else {                    // a fresh query (include/walker.cuh:1340-1343)
               wq = (int32_t)q; sp = a.starts[q]; pv = -1; ln = 1;
               a.paths[(uint64_t)q * (uint64_t)a.max_depth] = sp;
@@ -763,6 +812,12 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
           tt.hub_list[np][atomicAdd(&tt.hub_count[np], 1)] = tid;
         } else {
           tt.small_list[np][atomicAdd(&tt.small_count[np], 1)] = tid;
+          const uint4 b = philox4x32_10(a.walker_base + (uint32_t)tt.walker[tid], (uint32_t)(len - 1), 0u, 0u,
+                                        a.seed_lo, a.seed_hi);
+          tt.draw[0][tid] = b.x;
+          tt.draw[1][tid] = b.y;
+          tt.draw[2][tid] = b.z;
+          tt.draw[3][tid] = b.w;
         }
       }
       parity = np;
@@ -770,9 +825,15 @@ __global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
     __syncthreads();
   }
 
+  // workload counters: summed inside the workgroup first, the global counters are contended
   if (n_steps != 0ull) {
-    atomicAdd(&a.counters[0], n_steps);
-    atomicAdd(&a.counters[1], n_edges);
+    atomicAdd(&tt.acc[0], n_steps);
+    atomicAdd(&tt.acc[1], n_edges);
+  }
+  __syncthreads();
+  if (tid == 0 && tt.acc[0] != 0ull) {
+    atomicAdd(&a.counters[0], tt.acc[0]);
+    atomicAdd(&a.counters[1], tt.acc[1]);
   }
 }
 
@@ -811,29 +872,204 @@ __device__ __forceinline__ float bperm_f(int byte_addr, float x) {
   return __int_as_float(__builtin_amdgcn_ds_bpermute(byte_addr, __float_as_int(x)));
 }
 
+// The groups w, w + nw, ... of one list for up to 64 walkers at once (lane i = walker i).  Outputs the total S
+// of those groups (the same in every lane) and each walker's selected local index (or -1).
+template <int kApp>
+__device__ __forceinline__ void batch_stream(const fw_kargs& a, const uint32_t* __restrict__ bias, const uint32_t off,
+                                             const uint32_t deg, const int32_t want, const uint32_t w,
+                                             const uint32_t nw, const bool have, const uint32_t walker,
+                                             const uint32_t step, const int lane, float& S_out, int32_t& sel_out) {
+  constexpr uint32_t kG = 64u * kGroupQuartets;
+  constexpr int kEl = 4 * kGroupQuartets;
+  const uint32_t a0 = off & ~3u;
+  const uint32_t nq = (off + deg - a0 + 3u) >> 2;
+  const uint32_t ngroups = (nq + kG - 1u) / kG;
+
+  float S = 0.0f;             // shared: running total of this wave's groups
+  float Sj = 0.0f, u = 1.0f;  // per walker
+  int32_t sel = -1;
+  LaneDraw dq;
+
+  for (uint32_t g = w; g < ngroups; g += nw) {
+    const uint32_t kb = g * kG + (uint32_t)lane;
+    const bool interior = g > 0u && (g + 1u) * kG < nq;
+    uint4 raw[kGroupQuartets];
+    float x[kEl];
+    if (interior) {
+#pragma unroll
+      for (int j = 0; j < kGroupQuartets; ++j)
+        raw[j] = *reinterpret_cast<const uint4*>(bias + a0 + 4u * (kb + 64u * (uint32_t)j));
+    } else {
+#pragma unroll
+      for (int j = 0; j < kGroupQuartets; ++j) {
+        const uint32_t k = kb + 64u * (uint32_t)j;
+        raw[j] = make_uint4(0, 0, 0, 0);
+        if (k < nq) raw[j] = *reinterpret_cast<const uint4*>(bias + a0 + 4u * k);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kGroupQuartets; ++j) {
+      if (kApp == FW_APP_METAPATH) {
+        x[4 * j + 0] = (int32_t)raw[j].x == want ? 1.0f : 0.0f;
+        x[4 * j + 1] = (int32_t)raw[j].y == want ? 1.0f : 0.0f;
+        x[4 * j + 2] = (int32_t)raw[j].z == want ? 1.0f : 0.0f;
+        x[4 * j + 3] = (int32_t)raw[j].w == want ? 1.0f : 0.0f;
+      } else {
+        x[4 * j + 0] = __uint_as_float(raw[j].x);
+        x[4 * j + 1] = __uint_as_float(raw[j].y);
+        x[4 * j + 2] = __uint_as_float(raw[j].z);
+        x[4 * j + 3] = __uint_as_float(raw[j].w);
+      }
+    }
+    if (!interior) {
+#pragma unroll
+      for (int j = 0; j < kGroupQuartets; ++j) {
+        const uint32_t li = a0 + 4u * (kb + 64u * (uint32_t)j) - off;  // wraps below 0 for the head quartet
+        x[4 * j + 0] = li < deg ? x[4 * j + 0] : 0.0f;
+        x[4 * j + 1] = li + 1u < deg ? x[4 * j + 1] : 0.0f;
+        x[4 * j + 2] = li + 2u < deg ? x[4 * j + 2] : 0.0f;
+        x[4 * j + 3] = li + 3u < deg ? x[4 * j + 3] : 0.0f;
+      }
+    }
+    float q = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kEl; ++i) q = q + x[i];
+    const float I = wave_scan(q);
+    const float T = readlane_f(I, 63);
+    const float Snew = S + T;
+
+    const bool acc = have && (Snew * u > Sj);  // per walker: this group enters its reservoir
+    const uint64_t macc = __ballot(acc);
+    if (macc != 0ull) {
+      float target = 0.0f;
+      if (acc) target = next_uniform_lane(dq, a, walker, step, w) * T;
+      // which lane's biases hold the target of walker k: first lane with a positive total whose prefix
+      // exceeds it, else the last lane with a positive total
+      const bool pos = q > 0.0f;
+      const uint64_t mpos = __ballot(pos);
+      // M = running maximum of the positive lanes' prefixes.  It never decreases, and the first lane where it
+      // exceeds a target is the first positive lane whose own prefix does (a lane without positive total adds 0,
+      // which exceeds no target), so every walker finds its lane with a binary search across the lanes.
+      const float M = wave_prefix_max(pos ? I : 0.0f);
+      int src = 0;
+#pragma unroll
+      for (int s = 32; s >= 1; s >>= 1) {
+        const float Mp = bperm_f((src + s - 1) << 2, M);
+        src = Mp > target ? src : src + s;
+      }
+      if (!(bperm_f(src << 2, M) > target)) src = 63 - __builtin_clzll(mpos | 1ull);  // no crossing: last positive lane
+      // every walker resolves its own target on the 16 biases of its source lane (fetched across lanes)
+      const int addr = src << 2;
+      float e = bperm_f(addr, I - q);
+      int pick = -1, last = -1;
+#pragma unroll
+      for (int i = 0; i < kEl; ++i) {
+        const float xi = bperm_f(addr, x[i]);
+        e = e + xi;
+        const bool p = xi > 0.0f;
+        pick = (p && e > target && pick < 0) ? i : pick;
+        last = p ? i : last;
+      }
+      pick = pick < 0 ? last : pick;
+      if (acc) {
+        const uint32_t abs_idx = a0 + 4u * (g * kG + (uint32_t)src) + 256u * (uint32_t)(pick >> 2) + (uint32_t)(pick & 3);
+        sel = (int32_t)(abs_idx - off);
+        Sj = Snew;
+        u = next_uniform_lane(dq, a, walker, step, w);
+      }
+    }
+    S = Snew;
+  }
+  S_out = S;
+  sel_out = sel;
+}
+
+// Step commit of a batch by one wave (lane i = walker i; include/walker.cuh:1410-1417).  Every walker's record
+// goes back to its own position of the output list, so no list counter is contended: finished walks are marked
+// (q = -1), walkers whose new vertex is parked on again are tagged and carry their position inside that vertex's
+// bucket, the others are picked up from the same list by the next walk launch.
+template <int kApp>
+__device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_args& h, const int32_t v,
+                                             const uint32_t off, const uint32_t deg, const uint32_t rec_base,
+                                             const fw_walker_rec rec, const bool have, const int32_t pick,
+                                             const uint32_t walker, const uint32_t step, const int lane,
+                                             unsigned long long& n_steps, unsigned long long& n_edges,
+                                             uint32_t (&n_out)[2]) {
+  const bool moved = have && pick >= 0;
+  bool go_on = false;
+  int32_t nv = -1;
+  if (moved) {
+    nv = a.adjncy[off + (uint32_t)pick];
+    a.paths[(uint64_t)(uint32_t)rec.q * (uint64_t)a.max_depth + (uint64_t)rec.len] = nv;
+    go_on = rec.len + 1 < a.max_depth;
+    if (kApp == FW_APP_PPR && go_on) {
+      const uint32_t bits = philox4x32_10(walker, step, kStreamStop, 0u, a.seed_lo, a.seed_hi).x;
+      go_on = !(u24(bits) < a.tp);
+    }
+  }
+  const uint64_t mmoved = __ballot(moved);
+  if (lane == 0) {
+    const unsigned long long c = (unsigned long long)__builtin_popcountll(mmoved);
+    n_steps += c;
+    n_edges += c * (unsigned long long)deg;
+  }
+  bool park = false;
+  if (go_on) {
+    const int32_t ndeg = (int32_t)(a.xadj[nv + 1] - a.xadj[nv]);
+    go_on = ndeg > 0;  // a dead end finishes the walk (include/walker.cuh:1373-1374)
+    park = ndeg > a.park_threshold;
+  }
+  if (have) {
+    fw_walker_rec out;
+    out.q = go_on ? rec.q : -1;
+    out.cur = nv;
+    out.prev = v;
+    out.len = rec.len + 1;
+    if (go_on && park) {
+      const uint32_t label_slot = kApp == FW_APP_METAPATH ? (uint32_t)rec.len % (uint32_t)a.n_labels_per_hub : 0u;
+      out.prev = (int32_t)atomicAdd(
+          &h.bucket_out[(uint32_t)a.hub_index[nv] * (uint32_t)a.n_labels_per_hub + label_slot], 1u);
+      out.len |= FW_REC_PARK;
+    }
+    h.out[rec_base + (uint32_t)lane] = out;
+  }
+  const uint64_t mpark = __ballot(go_on && park);
+  const uint64_t mres = __ballot(go_on && !park);
+  if (lane == 0) {
+    n_out[0] += (uint32_t)__builtin_popcountll(mres);
+    n_out[1] += (uint32_t)__builtin_popcountll(mpark);
+  }
+}
+
 template <int kApp, int kWGT>
 __global__ __launch_bounds__(kWGT) void fw_hub_batch(const fw_kargs a, const fw_hub_args h) {
   constexpr int kNW = kWGT / 64;
-  constexpr uint32_t kG = 64u * kGroupQuartets;
-  constexpr int kEl = 4 * kGroupQuartets;
   __shared__ int32_t s_sel[kNW][64];
   __shared__ float s_w[16];
   __shared__ uint32_t s_task;
   __shared__ int32_t s_schema[kApp == FW_APP_METAPATH ? FW_MAX_SCHEMA : 1];
+  __shared__ unsigned long long s_acc[2];
+  __shared__ uint32_t s_out[2];
 
   const int tid = (int)threadIdx.x;
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (tid == 0) {
+    s_acc[0] = s_acc[1] = 0ull;
+    s_out[0] = s_out[1] = 0u;
+  }
   if (kApp == FW_APP_METAPATH && threadIdx.x == 0) {
 #pragma unroll
     for (int i = 0; i < FW_MAX_SCHEMA; ++i) s_schema[i] = a.schema[i];
   }
   const uint32_t ntasks = *h.ntasks;
-  const uint32_t labels = (uint32_t)a.n_labels_per_hub;
+  const uint32_t nwtasks = *h.nwtasks;
   const uint32_t* __restrict__ bias =
       reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
   unsigned long long n_steps = 0ull, n_edges = 0ull;
+  uint32_t n_out[2] = {0u, 0u};  // walkers that resume / that are parked again
 
+  // ---- workgroup tasks: lists above hub_threshold, sampled at workgroup granularity ----
   for (;;) {
     if (tid == 0) s_task = atomicAdd(h.task_next, 1u);
     __syncthreads();
@@ -841,121 +1077,21 @@ __global__ __launch_bounds__(kWGT) void fw_hub_batch(const fw_kargs a, const fw_
     __syncthreads();  // everyone has read s_task before it is overwritten; also fences s_sel / s_w reuse
     if (t >= ntasks) break;
 
-    const uint2 task = h.tasks[t];
-    const uint32_t bucket = task.x;
-    const uint32_t in_bucket = h.bucket_count[bucket] - task.y;
-    const int count = (int)(in_bucket < 64u ? in_bucket : 64u);
-    const uint32_t rec_base = h.bucket_offset[bucket] + task.y;
-    const int32_t v = h.hub_vertex[bucket / labels];
-    const int32_t want = kApp == FW_APP_METAPATH ? s_schema[bucket % labels] : 0;
-    const uint32_t off = a.xadj[v];
-    const uint32_t deg = a.xadj[v + 1] - off;
-    const uint32_t a0 = off & ~3u;
-    const uint32_t end = off + deg;
-    const uint32_t nq = (end - a0 + 3u) >> 2;
-    const uint32_t ngroups = (nq + kG - 1u) / kG;
+    const fw_batch_task task = h.tasks[t];
+    const int32_t want = kApp == FW_APP_METAPATH ? s_schema[task.slot] : 0;
 
     // lane i carries walker i of the batch
-    const bool have = lane < count;
+    const bool have = lane < task.count;
     fw_walker_rec rec;
-    rec.q = 0; rec.cur = v; rec.prev = -1; rec.len = 1;
-    if (have) rec = h.parked[h.sorted_idx[rec_base + (uint32_t)lane]];
+    rec.q = 0; rec.cur = task.v; rec.prev = -1; rec.len = 1;
+    if (have) rec = h.sorted[task.rec_base + (uint32_t)lane];
     const uint32_t walker = a.walker_base + (uint32_t)rec.q;
     const uint32_t step = (uint32_t)(rec.len - 1);
 
-    float S = 0.0f;                      // shared: running total of this wave's groups
-    float Sj = 0.0f, u = 1.0f;           // per walker
-    int32_t sel = -1;
-    LaneDraw dq;
-
-    for (uint32_t g = (uint32_t)wave; g < ngroups; g += (uint32_t)kNW) {
-      const uint32_t kb = g * kG + (uint32_t)lane;
-      const bool interior = g > 0u && (g + 1u) * kG < nq;
-      uint4 raw[kGroupQuartets];
-      float x[kEl];
-      if (interior) {
-#pragma unroll
-        for (int j = 0; j < kGroupQuartets; ++j)
-          raw[j] = *reinterpret_cast<const uint4*>(bias + a0 + 4u * (kb + 64u * (uint32_t)j));
-      } else {
-#pragma unroll
-        for (int j = 0; j < kGroupQuartets; ++j) {
-          const uint32_t k = kb + 64u * (uint32_t)j;
-          raw[j] = make_uint4(0, 0, 0, 0);
-          if (k < nq) raw[j] = *reinterpret_cast<const uint4*>(bias + a0 + 4u * k);
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < kGroupQuartets; ++j) {
-        if (kApp == FW_APP_METAPATH) {
-          x[4 * j + 0] = (int32_t)raw[j].x == want ? 1.0f : 0.0f;
-          x[4 * j + 1] = (int32_t)raw[j].y == want ? 1.0f : 0.0f;
-          x[4 * j + 2] = (int32_t)raw[j].z == want ? 1.0f : 0.0f;
-          x[4 * j + 3] = (int32_t)raw[j].w == want ? 1.0f : 0.0f;
-        } else {
-          x[4 * j + 0] = __uint_as_float(raw[j].x);
-          x[4 * j + 1] = __uint_as_float(raw[j].y);
-          x[4 * j + 2] = __uint_as_float(raw[j].z);
-          x[4 * j + 3] = __uint_as_float(raw[j].w);
-        }
-      }
-      if (!interior) {
-#pragma unroll
-        for (int j = 0; j < kGroupQuartets; ++j) {
-          const uint32_t li = a0 + 4u * (kb + 64u * (uint32_t)j) - off;  // wraps below 0 for the head quartet
-          x[4 * j + 0] = li < deg ? x[4 * j + 0] : 0.0f;
-          x[4 * j + 1] = li + 1u < deg ? x[4 * j + 1] : 0.0f;
-          x[4 * j + 2] = li + 2u < deg ? x[4 * j + 2] : 0.0f;
-          x[4 * j + 3] = li + 3u < deg ? x[4 * j + 3] : 0.0f;
-        }
-      }
-      float q = 0.0f;
-#pragma unroll
-      for (int i = 0; i < kEl; ++i) q = q + x[i];
-      const float I = wave_scan(q);
-      const float T = readlane_f(I, 63);
-      const float Snew = S + T;
-
-      const bool acc = have && (Snew * u > Sj);  // per walker: this group enters its reservoir
-      const uint64_t macc = __ballot(acc);
-      if (macc != 0ull) {
-        float target = 0.0f;
-        if (acc) target = next_uniform_lane(dq, a, walker, step, (uint32_t)wave) * T;
-        // which lane's biases hold the target of walker k: first lane with a positive total whose prefix
-        // exceeds it, else the last lane with a positive total
-        const bool pos = q > 0.0f;
-        const uint64_t mpos = __ballot(pos);
-        int src = 0;
-        for (uint64_t mm = macc; mm != 0ull; mm &= mm - 1ull) {
-          const int k = __builtin_ctzll(mm);
-          const float tk = readlane_f(target, k);
-          const uint64_t mk = __ballot(pos && I > tk);
-          const int lk = mk != 0ull ? __builtin_ctzll(mk) : 63 - __builtin_clzll(mpos);
-          src = (lane == k) ? lk : src;
-        }
-        // every walker resolves its own target on the 16 biases of its source lane (fetched across lanes)
-        const int addr = src << 2;
-        float e = bperm_f(addr, I - q);
-        int pick = -1, last = -1;
-#pragma unroll
-        for (int i = 0; i < kEl; ++i) {
-          const float xi = bperm_f(addr, x[i]);
-          e = e + xi;
-          const bool p = xi > 0.0f;
-          pick = (p && e > target && pick < 0) ? i : pick;
-          last = p ? i : last;
-        }
-        pick = pick < 0 ? last : pick;
-        if (acc) {
-          const uint32_t abs_idx = a0 + 4u * (g * kG + (uint32_t)src) + 256u * (uint32_t)(pick >> 2) + (uint32_t)(pick & 3);
-          sel = (int32_t)(abs_idx - off);
-          Sj = Snew;
-          u = next_uniform_lane(dq, a, walker, step, (uint32_t)wave);
-        }
-      }
-      S = Snew;
-    }
-
+    float S;
+    int32_t sel;
+    batch_stream<kApp>(a, bias, task.off, task.deg, want, (uint32_t)wave, (uint32_t)kNW, have, walker, step, lane, S,
+                       sel);
     s_sel[wave][lane] = sel;
     if (lane == 0) s_w[wave] = S;
     __syncthreads();
@@ -981,44 +1117,50 @@ __global__ __launch_bounds__(kWGT) void fw_hub_batch(const fw_kargs a, const fw_
         wsel = wsel < 0 ? wlast : wsel;
         if (wsel >= 0) pick = s_sel[wsel][lane];
       }
-      const bool moved = have && pick >= 0;
-      bool go_on = false;
-      int32_t nv = -1;
-      if (moved) {  // step commit: include/walker.cuh:1410-1417
-        nv = a.adjncy[off + (uint32_t)pick];
-        a.paths[(uint64_t)(uint32_t)rec.q * (uint64_t)a.max_depth + (uint64_t)rec.len] = nv;
-        go_on = rec.len + 1 < a.max_depth;
-        if (kApp == FW_APP_PPR && go_on) {
-          const uint32_t bits = philox4x32_10(walker, step, kStreamStop, 0u, a.seed_lo, a.seed_hi).x;
-          go_on = !(u24(bits) < a.tp);
-        }
-      }
-      const uint64_t mmoved = __ballot(moved);
-      if (lane == 0) {
-        const unsigned long long c = (unsigned long long)__builtin_popcountll(mmoved);
-        n_steps += c;
-        n_edges += c * (unsigned long long)deg;
-      }
-      const uint64_t mgo = __ballot(go_on);
-      if (mgo != 0ull) {  // survivors resume in the next walk launch
-        uint32_t rbase = 0;
-        const int leader = __builtin_ctzll(mgo);
-        if (lane == leader) rbase = atomicAdd(h.resume_count, (uint32_t)__builtin_popcountll(mgo));
-        rbase = (uint32_t)__builtin_amdgcn_readlane((int)rbase, leader);
-        if (go_on) {
-          fw_walker_rec out;
-          out.q = rec.q;
-          out.cur = nv;
-          out.prev = v;
-          out.len = rec.len + 1;
-          h.resume[rbase + (uint32_t)__builtin_popcountll(mgo & ((1ull << lane) - 1ull))] = out;
-        }
-      }
+      batch_commit<kApp>(a, h, task.v, task.off, task.deg, task.rec_base, rec, have, pick, walker, step, lane,
+                         n_steps, n_edges, n_out);
     }
   }
-  if (n_steps != 0ull) {  // the hub kernel's share is counted apart and added up by the host
-    atomicAdd(&a.counters[2], n_steps);
-    atomicAdd(&a.counters[3], n_edges);
+
+  // ---- wave tasks: lists up to hub_threshold, sampled at wave granularity, one batch per wave; the tasks are
+  //      short and many, so they are dealt out by position instead of through a contended counter ----
+  const uint32_t nwaves = gridDim.x * (uint32_t)kNW;
+  for (uint32_t t = blockIdx.x * (uint32_t)kNW + (uint32_t)wave; t < nwtasks; t += nwaves) {
+    const fw_batch_task* tp = h.wtasks + t;
+    const int32_t v = __builtin_amdgcn_readfirstlane(tp->v);
+    const uint32_t off = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->off);
+    const uint32_t deg = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->deg);
+    const uint32_t rec_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->rec_base);
+    const int count = __builtin_amdgcn_readfirstlane(tp->count);
+    const int32_t want = kApp == FW_APP_METAPATH ? s_schema[__builtin_amdgcn_readfirstlane(tp->slot)] : 0;
+
+    const bool have = lane < count;
+    fw_walker_rec rec;
+    rec.q = 0; rec.cur = v; rec.prev = -1; rec.len = 1;
+    if (have) rec = h.sorted[rec_base + (uint32_t)lane];
+    const uint32_t walker = a.walker_base + (uint32_t)rec.q;
+    const uint32_t step = (uint32_t)(rec.len - 1);
+
+    float S;
+    int32_t sel;
+    batch_stream<kApp>(a, bias, off, deg, want, 0u, 1u, have, walker, step, lane, S, sel);
+    batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, have, sel, walker, step, lane, n_steps, n_edges, n_out);
+  }
+
+  // counters: summed inside the workgroup first (the global ones are contended); the batch kernel's share of the
+  // workload is counted apart and added up by the host
+  if (n_steps != 0ull) {
+    atomicAdd(&s_acc[0], n_steps);
+    atomicAdd(&s_acc[1], n_edges);
+    atomicAdd(&s_out[0], n_out[0]);
+    atomicAdd(&s_out[1], n_out[1]);
+  }
+  __syncthreads();
+  if (tid == 0 && s_acc[0] != 0ull) {
+    atomicAdd(&a.counters[2], s_acc[0]);
+    atomicAdd(&a.counters[3], s_acc[1]);
+    if (s_out[0] != 0u) atomicAdd(&h.out_counts[0], s_out[0]);
+    if (s_out[1] != 0u) atomicAdd(&h.out_counts[1], s_out[1]);
   }
 }
 

@@ -62,8 +62,8 @@ typedef struct {
   int32_t grid;          /* workgroups to launch; 0 = library default (src/walk.cu:84-92 analogue) */
   int32_t park_threshold; /* hub parking, an execution strategy that never changes results: walkers that arrive on a
                             vertex of larger degree wait there and are served 64 at a time by one shared scan of its
-                            list.  0 = library default (on for batches >= 65536 queries), < 0 = off, > 0 = degree
-                            (raised to hub_threshold if smaller).  Not used by node2vec. */
+                            list (by a workgroup above hub_threshold, by one wave below).  0 = library default (on
+                            for batches >= 65536 queries), < 0 = off, > 0 = degree.  Not used by node2vec. */
 } fw_walk_params;
 
 /* What src/main.cu:82-113 (calculate_workload) and the timing code of src/walk.cu report. */

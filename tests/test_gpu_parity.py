@@ -85,9 +85,12 @@ def test_hub_parking_does_not_change_results(gpu, hub, app, wg):
     kw = dict(deepwalk=dict(app=gpu.APP_DEEPWALK, max_depth=41),
               ppr=dict(app=gpu.APP_PPR, max_depth=81, tp=0.15),
               metapath=dict(app=gpu.APP_METAPATH, max_depth=11, schema=[1, 3, 0]))[app]
-    for hub_thr, park in ((1000, 1000), (64, 2000), (500, 8000)):
+    # park threshold at / above the hub threshold: workgroup batches only; below it: vertices in between are served
+    # by single waves (wave-granularity sampling); 3: nearly every vertex of the graph is parked on
+    for hub_thr, park in ((1000, 1000), (64, 2000), (500, 8000), (4096, 3), (100000, 600), (1000, 12)):
         _, st = _check(gpu, hub, starts, wg_threads=wg, hub_threshold=hub_thr, park_threshold=park, seed=77, **kw)
         assert st.launches >= 3                      # walk, hub batch, walk ...
+        assert 0 < st.hub_steps <= st.steps
 
 
 def test_hub_parking_through_the_batch_driver(gpu, hub):
