@@ -6,6 +6,7 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <cstring>
@@ -759,6 +760,9 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, 8 * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     FW_HIP(hipStreamSynchronize(stream));
     th.collect(&times->hub_ms);
+    if (getenv("FW_DEBUG_ROUNDS"))
+      fprintf(stderr, "round: parked %llu (walk %u + again %u) wg_tasks %u wave_tasks %u -> resume %u again %u\n",
+              (unsigned long long)m, n_walked, n_again, pb->h_ctrs[3], pb->h_ctrs[5], pb->h_ctrs[1], pb->h_ctrs[2]);
     n_out = (uint32_t)m;
     pb->h_ctrs[0] = 0u;
     if (pb->h_ctrs[1] != 0u) {

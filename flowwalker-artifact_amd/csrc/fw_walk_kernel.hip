@@ -61,33 +61,46 @@ __device__ __forceinline__ float u24(uint32_t bits) { return (float)(bits >> 8) 
 
 // ---- wave64 scans on the DPP network -----------------------------------------------------------
 
-// x + (value of the lane selected by the DPP control, 0 where the control has no source lane or the
-// row is masked off).
-template <int kCtrl, int kRowMask>
+// x + (value of the lane selected by the DPP control; lanes without a source lane add 0).  For values that are
+// not -0 (sums of non-negative biases never are) x + 0 == x bit for bit.
+template <int kCtrl>
 __device__ __forceinline__ float dpp_add(float x) {
-  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(x), kCtrl, kRowMask, 0xF, false);
+  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(x), kCtrl, 0xF, 0xF, true);
   return x + __int_as_float(moved);
+}
+
+// x += (lane 15 of the previous row) in rows 1 and 3; x += (lane 31) in rows 2 and 3.  The other rows keep x: the
+// instruction does not write them.  (Written out because the compiler only folds a lane movement into an add
+// when the skipped lanes can be given the operation's identity, which it does not do for float adds.)
+__device__ __forceinline__ float dpp_add_bcast15(float x) {
+  asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf" : "+v"(x));
+  return x;
+}
+__device__ __forceinline__ float dpp_add_bcast31(float x) {
+  asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf" : "+v"(x));
+  return x;
 }
 
 // Inclusive scan over the 64 lanes: Kogge-Stone inside each 16-lane row (row_shr 1,2,4,8), then
 // row_bcast:15 into rows 1 and 3, then row_bcast:31 into rows 2 and 3.  The association order is part
 // of the sampler's definition.
 __device__ __forceinline__ float wave_scan(float x) {
-  x = dpp_add<0x111, 0xF>(x);
-  x = dpp_add<0x112, 0xF>(x);
-  x = dpp_add<0x114, 0xF>(x);
-  x = dpp_add<0x118, 0xF>(x);
-  x = dpp_add<0x142, 0xA>(x);
-  x = dpp_add<0x143, 0xC>(x);
+  x = dpp_add<0x111>(x);
+  x = dpp_add<0x112>(x);
+  x = dpp_add<0x114>(x);
+  x = dpp_add<0x118>(x);
+  x = dpp_add_bcast15(x);
+  x = dpp_add_bcast31(x);
   return x;
 }
 
-// Inclusive prefix maximum over the 64 lanes of non-negative values (same network as wave_scan; max is exact,
-// so its association order does not matter).
+// Inclusive prefix maximum over the 64 lanes of non-negative floats (same network as wave_scan).  Non-negative
+// floats order like their bit patterns, so the maximum is taken on the integers (exact, no NaN handling).
 template <int kCtrl, int kRowMask>
 __device__ __forceinline__ float dpp_max(float x) {
-  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(x), kCtrl, kRowMask, 0xF, false);
-  return fmaxf(x, __int_as_float(moved));
+  const uint32_t xi = __float_as_uint(x);
+  const uint32_t moved = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)xi, kCtrl, kRowMask, 0xF, false);
+  return __uint_as_float(xi > moved ? xi : moved);
 }
 
 __device__ __forceinline__ float wave_prefix_max(float x) {
@@ -102,10 +115,10 @@ __device__ __forceinline__ float wave_prefix_max(float x) {
 
 // Inclusive scan inside each 16-lane row only.
 __device__ __forceinline__ float row_scan(float x) {
-  x = dpp_add<0x111, 0xF>(x);
-  x = dpp_add<0x112, 0xF>(x);
-  x = dpp_add<0x114, 0xF>(x);
-  x = dpp_add<0x118, 0xF>(x);
+  x = dpp_add<0x111>(x);
+  x = dpp_add<0x112>(x);
+  x = dpp_add<0x114>(x);
+  x = dpp_add<0x118>(x);
   return x;
 }
 
@@ -463,17 +476,19 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
       } else {  // rounding in the scan tree left no crossing: last lane with a positive total
         l = 63 - __builtin_clzll(__ballot(pos));
       }
-      // every lane resolves its own elements; the answer of lane l is the one that is read
+      // Every lane resolves its own elements; the answer of lane l is the one that is read.  The running sum
+      // e never decreases (the biases are not negative), so "first positive element whose running sum exceeds
+      // the target" is the first positive element at or after position #(sums <= target); none: last positive.
       float e = I - q;
-      int pick = -1, last = -1;
+      uint32_t cnt = 0u, pm = 0u;
 #pragma unroll
       for (int i = 0; i < kEl; ++i) {
         e = e + x[i];
-        const bool p = x[i] > 0.0f;
-        pick = (p && e > target && pick < 0) ? i : pick;
-        last = p ? i : last;
+        cnt += e <= target ? 1u : 0u;
+        pm |= (x[i] > 0.0f ? 1u : 0u) << i;
       }
-      pick = pick < 0 ? last : pick;
+      const uint32_t cand = pm >> cnt;
+      const int pick = cand != 0u ? (int)cnt + __builtin_ctz(cand) : 31 - __builtin_clz(pm | 1u);
       const uint32_t abs_idx = a0 + 4u * kb + 256u * (uint32_t)(pick >> 2) + (uint32_t)(pick & 3);
       sel = __builtin_amdgcn_readlane((int32_t)(abs_idx - c.off), l);
       if (kTrackV) {
@@ -572,7 +587,7 @@ __device__ __forceinline__ void commit(const fw_kargs& a, TaskTable<kWGT, kApp>&
 // ---- the kernel --------------------------------------------------------------------------------
 
 template <int kApp, int kWGT>
-__global__ __launch_bounds__(kWGT) void fw_walk_zprs(const fw_kargs a) {
+__global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk_zprs(const fw_kargs a) {
   constexpr int kNW = kWGT / 64;
   __shared__ TaskTable<kWGT, kApp> tt;
 
@@ -958,19 +973,23 @@ __device__ __forceinline__ void batch_stream(const fw_kargs& a, const uint32_t* 
         src = Mp > target ? src : src + s;
       }
       if (!(bperm_f(src << 2, M) > target)) src = 63 - __builtin_clzll(mpos | 1ull);  // no crossing: last positive lane
-      // every walker resolves its own target on the 16 biases of its source lane (fetched across lanes)
+      // Every walker resolves its own target on the 16 biases of its source lane (fetched across lanes, all
+      // fetches in flight together).  The running sum never decreases, so the element is the first positive one
+      // at or after position #(sums <= target); none: the last positive one.
       const int addr = src << 2;
+      float xs[kEl];
       float e = bperm_f(addr, I - q);
-      int pick = -1, last = -1;
+#pragma unroll
+      for (int i = 0; i < kEl; ++i) xs[i] = bperm_f(addr, x[i]);
+      uint32_t cnt = 0u, pm = 0u;
 #pragma unroll
       for (int i = 0; i < kEl; ++i) {
-        const float xi = bperm_f(addr, x[i]);
-        e = e + xi;
-        const bool p = xi > 0.0f;
-        pick = (p && e > target && pick < 0) ? i : pick;
-        last = p ? i : last;
+        e = e + xs[i];
+        cnt += e <= target ? 1u : 0u;
+        pm |= (xs[i] > 0.0f ? 1u : 0u) << i;
       }
-      pick = pick < 0 ? last : pick;
+      const uint32_t cand = pm >> cnt;
+      const int pick = cand != 0u ? (int)cnt + __builtin_ctz(cand) : 31 - __builtin_clz(pm | 1u);
       if (acc) {
         const uint32_t abs_idx = a0 + 4u * (g * kG + (uint32_t)src) + 256u * (uint32_t)(pick >> 2) + (uint32_t)(pick & 3);
         sel = (int32_t)(abs_idx - off);
@@ -1042,7 +1061,7 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
 }
 
 template <int kApp, int kWGT>
-__global__ __launch_bounds__(kWGT) void fw_hub_batch(const fw_kargs a, const fw_hub_args h) {
+__global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const fw_hub_args h) {
   constexpr int kNW = kWGT / 64;
   __shared__ int32_t s_sel[kNW][64];
   __shared__ float s_w[16];
