@@ -222,7 +222,7 @@ extern "C" int fw_graph_destroy(fw_graph* g) {
       if (p && hipFree(p) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
     }
   }
-  void* index_ptrs[2] = {g->hub_index, g->hub_vertex};
+  void* index_ptrs[2] = {g->hub_index, g->hub_info};
   for (void* p : index_ptrs) {
     if (p && hipFree(p) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
   }
@@ -440,23 +440,28 @@ __global__ void fw_hub_count_kernel(const uint32_t* __restrict__ xadj, int32_t V
 }
 
 __global__ void fw_hub_index_kernel(const uint32_t* __restrict__ xadj, int32_t V, int32_t threshold, unsigned* next,
-                                    int32_t* hub_index, int32_t* hub_vertex) {
+                                    int32_t* hub_index, fw_hub_info* hub_info) {
   const int stride = gridDim.x * blockDim.x;
   for (int v = blockIdx.x * blockDim.x + threadIdx.x; v < V; v += stride) {
     int32_t idx = -1;
     if ((int32_t)(xadj[v + 1] - xadj[v]) > threshold) {
       idx = (int32_t)atomicAdd(next, 1u);
-      hub_vertex[idx] = v;
+      fw_hub_info hi;
+      hi.v = v;
+      hi.off = xadj[v];
+      hi.deg = xadj[v + 1] - hi.off;
+      hi.pad = 0u;
+      hub_info[idx] = hi;
     }
     hub_index[v] = idx;
   }
 }
 
-// (Re)builds g->hub_index / hub_vertex for `threshold`; cached in the graph.
+// (Re)builds g->hub_index / hub_info for `threshold`; cached in the graph.
 static int ensure_hub_index(fw_graph* g, int32_t threshold) {
   if (g->hub_index_threshold == threshold && g->hub_index) return FW_OK;
   if (g->hub_index) { (void)hipFree(g->hub_index); g->hub_index = nullptr; }
-  if (g->hub_vertex) { (void)hipFree(g->hub_vertex); g->hub_vertex = nullptr; }
+  if (g->hub_info) { (void)hipFree(g->hub_info); g->hub_info = nullptr; }
   g->hub_index_threshold = -1;
   g->n_hubs = 0;
   unsigned* d_cnt = nullptr;
@@ -466,10 +471,10 @@ static int ensure_hub_index(fw_graph* g, int32_t threshold) {
   unsigned n_hubs = 0;
   int rc = fw_check_hip(hipMemcpy(&n_hubs, d_cnt, sizeof(unsigned), hipMemcpyDeviceToHost), "hipMemcpy(hub count)", __FILE__, __LINE__);
   if (rc == FW_OK) rc = fw_check_hip(hipMalloc(reinterpret_cast<void**>(&g->hub_index), (size_t)g->V * sizeof(int32_t)), "hipMalloc(hub_index)", __FILE__, __LINE__);
-  if (rc == FW_OK) rc = fw_check_hip(hipMalloc(reinterpret_cast<void**>(&g->hub_vertex), (size_t)(n_hubs ? n_hubs : 1) * sizeof(int32_t)), "hipMalloc(hub_vertex)", __FILE__, __LINE__);
+  if (rc == FW_OK) rc = fw_check_hip(hipMalloc(reinterpret_cast<void**>(&g->hub_info), (size_t)(n_hubs ? n_hubs : 1) * sizeof(fw_hub_info)), "hipMalloc(hub_info)", __FILE__, __LINE__);
   if (rc == FW_OK) {
     hipLaunchKernelGGL(fw_hub_index_kernel, dim3(1024), dim3(256), 0, 0, g->xadj, g->V, threshold, d_cnt + 1,
-                       g->hub_index, g->hub_vertex);
+                       g->hub_index, g->hub_info);
     rc = fw_check_hip(hipDeviceSynchronize(), "hub index", __FILE__, __LINE__);
   }
   (void)hipFree(d_cnt);
@@ -484,6 +489,7 @@ static int ensure_hub_index(fw_graph* g, int32_t threshold) {
 // entries, a vertex of degree d holds about n * d / E of them, so the threshold is kParkMeet * E / n, not below
 // kMinDefaultPark (shorter lists cost less to read than a record costs to move).
 constexpr int32_t kMinParkBatch = 65536;
+constexpr uint32_t kParkTail = 32768;  // fewer walkers than this finish in one walk launch without parking
 constexpr double kParkMeet = 4.0;
 constexpr int32_t kMinDefaultPark = 64;
 constexpr int32_t kMinParkThreshold = 1;
@@ -492,8 +498,7 @@ constexpr int32_t kMinParkThreshold = 1;
 // granularity (degree above hub_threshold), a wave task otherwise.  ctrs[3] / ctrs[5] = number of tasks (out).
 __global__ __launch_bounds__(256) void fw_bucket_tasks_kernel(const uint32_t* __restrict__ bucket_count,
                                        const uint32_t* __restrict__ bucket_offset, int n_buckets, int labels,
-                                       const int32_t* __restrict__ hub_vertex, const uint32_t* __restrict__ xadj,
-                                       int32_t hub_threshold, fw_batch_task* tasks, fw_batch_task* wtasks,
+                                       const fw_hub_info* __restrict__ hub_info, int32_t hub_threshold, fw_batch_task* tasks, fw_batch_task* wtasks,
                                        uint32_t* ctrs) {
   const int stride = gridDim.x * blockDim.x;
   const int lane = (int)(threadIdx.x & 63u);
@@ -506,9 +511,10 @@ __global__ __launch_bounds__(256) void fw_bucket_tasks_kernel(const uint32_t* __
     t.pad[0] = t.pad[1] = 0;
     bool wg = false;
     if (c != 0u) {
-      t.v = hub_vertex[b / labels];
-      t.off = xadj[t.v];
-      t.deg = xadj[t.v + 1] - t.off;
+      const fw_hub_info hi = hub_info[b / labels];
+      t.v = hi.v;
+      t.off = hi.off;
+      t.deg = hi.deg;
       t.slot = b % labels;
       wg = (int32_t)t.deg > hub_threshold;
     }
@@ -545,10 +551,9 @@ __global__ __launch_bounds__(256) void fw_bucket_tasks_kernel(const uint32_t* __
 
 // Counting-sort scatter of a round's parked walkers into `sorted`.  Two sources share a bucket's range:
 //  * the previous batch launch's output list, of which only the records tagged FW_REC_PARK are parked; they carry
-//    their position inside the bucket (taken when they were parked) and fill the range from its start;
+//    their bucket and their position inside it (taken when they were parked) and fill the range from its start;
 //  * the walk kernel's list, whose records were only counted; they take positions from the end of the range here.
 __global__ void fw_scatter_tagged_kernel(const fw_walker_rec* __restrict__ src, uint32_t m,
-                                         const int32_t* __restrict__ hub_index, int labels, int metapath,
                                          const uint32_t* __restrict__ bucket_offset,
                                          fw_walker_rec* __restrict__ sorted) {
   const uint32_t stride = gridDim.x * blockDim.x;
@@ -556,24 +561,28 @@ __global__ void fw_scatter_tagged_kernel(const fw_walker_rec* __restrict__ src, 
     fw_walker_rec r = src[i];
     if (r.q < 0 || (r.len & FW_REC_PARK) == 0) continue;
     r.len &= ~FW_REC_PARK;
-    const uint32_t slot = metapath ? (uint32_t)(r.len - 1) % (uint32_t)labels : 0u;
-    const uint32_t b = (uint32_t)hub_index[r.cur] * (uint32_t)labels + slot;
-    sorted[bucket_offset[b] + (uint32_t)r.prev] = r;
+    sorted[bucket_offset[r.cur] + (uint32_t)r.prev] = r;
   }
 }
 
 __global__ void fw_scatter_counted_kernel(const fw_walker_rec* __restrict__ src, uint32_t m,
-                                          const int32_t* __restrict__ hub_index, int labels, int metapath,
                                           const uint32_t* __restrict__ bucket_count,
                                           const uint32_t* __restrict__ bucket_offset, uint32_t* bucket_fill,
                                           fw_walker_rec* __restrict__ sorted) {
   const uint32_t stride = gridDim.x * blockDim.x;
   for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < m; i += stride) {
     const fw_walker_rec r = src[i];
-    const uint32_t slot = metapath ? (uint32_t)(r.len - 1) % (uint32_t)labels : 0u;
-    const uint32_t b = (uint32_t)hub_index[r.cur] * (uint32_t)labels + slot;
+    const uint32_t b = (uint32_t)r.cur;
     sorted[bucket_offset[b] + bucket_count[b] - 1u - atomicAdd(&bucket_fill[b], 1u)] = r;
   }
+}
+
+// Parked records name their bucket; the walk kernel wants the vertex (used when the last few walkers leave the
+// park / batch loop).
+__global__ void fw_bucket_to_vertex_kernel(fw_walker_rec* recs, uint32_t m, const fw_hub_info* __restrict__ hub_info,
+                                           int labels) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < m) recs[i].cur = hub_info[(uint32_t)recs[i].cur / (uint32_t)labels].v;
 }
 
 // Device buffers of one park / batch / resume loop (one per stream in flight).  Three record lists: `walked`
@@ -675,7 +684,6 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     return fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, grid_used);
   }
   const int labels = p->app == FW_APP_METAPATH ? p->schema_len : 1;
-  const int metapath = p->app == FW_APP_METAPATH ? 1 : 0;
   const size_t bucket_bytes = (size_t)pb->n_buckets * sizeof(uint32_t);
   a.park_threshold = park_threshold;
   a.n_labels_per_hub = labels;
@@ -734,20 +742,30 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     };
     if (n_out != 0u)
       hipLaunchKernelGGL(fw_scatter_tagged_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
-                         g->hub_index, labels, metapath, pb->offset(), pb->sorted);
+                         pb->offset(), pb->sorted);
     if (n_walked != 0u) {
       FW_HIP(hipMemsetAsync(pb->fill(), 0, bucket_bytes, stream));
       hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_walked)), dim3(256), 0, stream, pb->walked,
-                         n_walked, g->hub_index, labels, metapath, pb->count(cur), pb->offset(), pb->fill(),
-                         pb->sorted);
+                         n_walked, pb->count(cur), pb->offset(), pb->fill(), pb->sorted);
     }
     FW_HIP(hipGetLastError());
+    if (p->park_threshold == 0 && m < kParkTail) {
+      // default rule only (an explicit threshold keeps every round in the loop): too few walkers are left to
+      // meet anywhere, so they finish in one walk launch that does not park
+      hipLaunchKernelGGL(fw_bucket_to_vertex_kernel, dim3(((unsigned)m + 255u) / 256u), dim3(256), 0, stream,
+                         pb->sorted, (uint32_t)m, g->hub_info, labels);
+      FW_HIP(hipGetLastError());
+      a.resume = pb->sorted;
+      a.n = (int32_t)m;
+      a.park_threshold = INT_MAX;
+      return walk(nullptr);
+    }
     FW_HIP(hipMemsetAsync(pb->ctrs + 1, 0, 7 * sizeof(uint32_t), stream));
     FW_HIP(hipMemsetAsync(pb->count(nxt), 0, bucket_bytes, stream));
     unsigned tblocks = ((unsigned)pb->n_buckets + 255u) / 256u;
     if (tblocks > 2048u) tblocks = 2048u;
     hipLaunchKernelGGL(fw_bucket_tasks_kernel, dim3(tblocks), dim3(256), 0, stream, pb->count(cur), pb->offset(),
-                       pb->n_buckets, labels, g->hub_vertex, g->xadj, p->hub_threshold, pb->tasks, pb->wtasks,
+                       pb->n_buckets, labels, g->hub_info, p->hub_threshold, pb->tasks, pb->wtasks,
                        pb->ctrs);
     FW_HIP(hipGetLastError());
     h.bucket_out = pb->count(nxt);

@@ -6,6 +6,14 @@
 
 #include "flowwalker.h"
 
+// A vertex that walkers are parked on: its CSR range, so that building batch tasks is a streaming pass.
+struct fw_hub_info {
+  int32_t v;
+  uint32_t off;  // xadj[v]
+  uint32_t deg;
+  uint32_t pad;
+};
+
 // Device CSR mirror (include/gpu_graph.cuh:28-36 in the reference).  Edge arrays are allocated with
 // FW_EDGE_PAD extra elements so that aligned 16-byte loads of the last quartet stay in bounds.
 struct fw_graph {
@@ -23,8 +31,8 @@ struct fw_graph {
   // lazily built index of the vertices whose degree exceeds hub_index_threshold (hub parking)
   int32_t hub_index_threshold = -1;
   int32_t n_hubs = 0;
-  int32_t* hub_index = nullptr;   // int32[V]: position in hub_vertex, or -1
-  int32_t* hub_vertex = nullptr;  // int32[n_hubs]
+  int32_t* hub_index = nullptr;       // int32[V]: position in hub_info, or -1
+  struct fw_hub_info* hub_info = nullptr;  // [n_hubs]
 };
 
 constexpr int FW_EDGE_PAD = 4;
@@ -32,7 +40,7 @@ constexpr int FW_EDGE_PAD = 4;
 // A walker in transit between kernels (parked on a hub, or resuming after its hub step): 16 bytes.
 struct fw_walker_rec {
   int32_t q;     // query index inside the launch (walker id = walker_base + q)
-  int32_t cur;   // current vertex
+  int32_t cur;   // current vertex; in a parked record: the bucket (hub index * labels + label slot) it waits in
   int32_t prev;  // previous vertex or -1; in a parked record: its position inside the bucket of `cur`
   int32_t len;   // path entries written so far
 };

@@ -747,17 +747,18 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
           if (park) {
             const uint32_t at = pbase + (uint32_t)__builtin_popcountll(pm & ((1ull << lane) - 1ull));
             const int32_t v = tt.cur[tid];
+            const uint32_t label_slot =
+                kApp == FW_APP_METAPATH ? (uint32_t)(len - 1) % (uint32_t)a.n_labels_per_hub : 0u;
+            const uint32_t bucket = (uint32_t)a.hub_index[v] * (uint32_t)a.n_labels_per_hub + label_slot;
             fw_walker_rec rec;
             rec.q = tt.walker[tid];
-            rec.cur = v;
+            rec.cur = (int32_t)bucket;  // the vertex follows from the bucket
             rec.prev = tt.prev[tid];
             rec.len = len;
             a.parked[at] = rec;
             // counted only: the wave does not wait for a position inside the bucket (the counters of the busiest
             // vertices are contended); the counting sort hands the positions out later
-            const uint32_t label_slot =
-                kApp == FW_APP_METAPATH ? (uint32_t)(len - 1) % (uint32_t)a.n_labels_per_hub : 0u;
-            atomicAdd(&a.bucket_count[(uint32_t)a.hub_index[v] * (uint32_t)a.n_labels_per_hub + label_slot], 1u);
+            atomicAdd(&a.bucket_count[bucket], 1u);
             park = false;
             need = true;
             len = -1;
@@ -1046,8 +1047,9 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
     out.len = rec.len + 1;
     if (go_on && park) {
       const uint32_t label_slot = kApp == FW_APP_METAPATH ? (uint32_t)rec.len % (uint32_t)a.n_labels_per_hub : 0u;
-      out.prev = (int32_t)atomicAdd(
-          &h.bucket_out[(uint32_t)a.hub_index[nv] * (uint32_t)a.n_labels_per_hub + label_slot], 1u);
+      const uint32_t bucket = (uint32_t)a.hub_index[nv] * (uint32_t)a.n_labels_per_hub + label_slot;
+      out.cur = (int32_t)bucket;  // the vertex follows from the bucket
+      out.prev = (int32_t)atomicAdd(&h.bucket_out[bucket], 1u);
       out.len |= FW_REC_PARK;
     }
     h.out[rec_base + (uint32_t)lane] = out;

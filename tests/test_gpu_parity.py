@@ -93,6 +93,26 @@ def test_hub_parking_does_not_change_results(gpu, hub, app, wg):
         assert 0 < st.hub_steps <= st.steps
 
 
+def test_default_parking_rule_and_its_tail(gpu, hub):
+    """park_threshold = 0: the library decides (batches of at least 65,536 queries park where about four walkers
+    meet), and once few walkers are left they finish in one launch without parking.  Same paths either way."""
+    xadj, adj, w, lab = hub
+    starts = np.random.RandomState(8).randint(0, 12000, size=600000).astype(np.int32)  # ~50,000 of them park per round
+    og = _oracle.Graph(xadj, adj, w, lab)
+    g = gpu.Graph.from_csr(xadj, adj, w, lab)
+    try:
+        for kw in (dict(app=gpu.APP_PPR, max_depth=61, tp=0.3), dict(app=gpu.APP_DEEPWALK, max_depth=9)):
+            p = gpu.default_params(seed=21, **kw)
+            assert p.park_threshold == 0
+            ref, steps, edges = _oracle.walk(og, _oracle.from_walk_params(p), starts)
+            paths, st = g.walk(p, starts)
+            assert (paths == ref).all()
+            assert (st.steps, st.sampled_edges) == (steps, edges)
+            assert st.launches >= 3 and 0 < st.hub_steps < st.steps
+    finally:
+        g.destroy()
+
+
 def test_hub_parking_through_the_batch_driver(gpu, hub):
     xadj, adj, w, lab = hub
     starts = np.random.RandomState(5).randint(0, 12000, size=9000).astype(np.int32)
