@@ -496,13 +496,18 @@ constexpr int32_t kMinParkThreshold = 1;
 
 // One task per 64 parked walkers of a bucket: a workgroup task when the bucket's vertex is sampled at workgroup
 // granularity (degree above hub_threshold), a wave task otherwise.  ctrs[3] / ctrs[5] = number of tasks (out).
-__global__ __launch_bounds__(256) void fw_bucket_tasks_kernel(const uint32_t* __restrict__ bucket_count,
+__global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* __restrict__ bucket_count,
                                        const uint32_t* __restrict__ bucket_offset, int n_buckets, int labels,
-                                       const fw_hub_info* __restrict__ hub_info, int32_t hub_threshold, fw_batch_task* tasks, fw_batch_task* wtasks,
-                                       uint32_t* ctrs) {
+                                       const fw_hub_info* __restrict__ hub_info, int32_t hub_threshold,
+                                       fw_batch_task* tasks, fw_batch_task* wtasks, uint32_t* ctrs) {
+  // task slots: one update of the (contended) global counters per workgroup and kind; inside the workgroup the
+  // slots are dealt out by a scan over the waves' totals
+  __shared__ uint32_t s_tot[2][16];
+  __shared__ uint32_t s_base[2];
   const int stride = gridDim.x * blockDim.x;
   const int lane = (int)(threadIdx.x & 63u);
-  const int rounds = (n_buckets + stride - 1) / stride;  // every lane runs every round: the wave scans need all 64
+  const int wave = (int)(threadIdx.x >> 6);
+  const int rounds = (n_buckets + stride - 1) / stride;  // every thread runs every round: scans and barriers
   for (int r = 0; r < rounds; ++r) {
     const int b = r * stride + (int)(blockIdx.x * blockDim.x + threadIdx.x);
     const uint32_t c = b < n_buckets ? bucket_count[b] : 0u;
@@ -519,8 +524,7 @@ __global__ __launch_bounds__(256) void fw_bucket_tasks_kernel(const uint32_t* __
       wg = (int32_t)t.deg > hub_threshold;
     }
     const uint32_t nb = (c + 63u) >> 6;
-    // task slots: one counter update per wave and kind instead of one per bucket (the counters are contended)
-    uint32_t xw = wg ? nb : 0u, xs = wg ? 0u : nb;
+    const uint32_t xw = wg ? nb : 0u, xs = wg ? 0u : nb;
     uint32_t iw = xw, is = xs;  // inclusive wave scans
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -528,16 +532,23 @@ __global__ __launch_bounds__(256) void fw_bucket_tasks_kernel(const uint32_t* __
       const uint32_t us = __shfl_up(is, d);
       if (lane >= d) { iw += uw; is += us; }
     }
-    const uint32_t tw = __shfl(iw, 63), ts = __shfl(is, 63);
-    uint32_t bw = 0u, bs = 0u;
     if (lane == 63) {
-      if (tw != 0u) bw = atomicAdd(&ctrs[3], tw);
-      if (ts != 0u) bs = atomicAdd(&ctrs[5], ts);
+      s_tot[0][wave] = iw;
+      s_tot[1][wave] = is;
     }
-    bw = __shfl(bw, 63);
-    bs = __shfl(bs, 63);
+    __syncthreads();
+    if (threadIdx.x < 2) {
+      uint32_t total = 0u;
+      for (int w = 0; w < 16; ++w) {  // exclusive prefix over the waves, in place
+        const uint32_t v = s_tot[threadIdx.x][w];
+        s_tot[threadIdx.x][w] = total;
+        total += v;
+      }
+      s_base[threadIdx.x] = total != 0u ? atomicAdd(&ctrs[threadIdx.x == 0 ? 3 : 5], total) : 0u;
+    }
+    __syncthreads();
     if (c != 0u) {
-      const uint32_t t0 = wg ? bw + iw - xw : bs + is - xs;
+      const uint32_t t0 = wg ? s_base[0] + s_tot[0][wave] + iw - xw : s_base[1] + s_tot[1][wave] + is - xs;
       fw_batch_task* out = wg ? tasks : wtasks;
       const uint32_t base = bucket_offset[b];
       for (uint32_t k = 0; k < nb; ++k) {
@@ -546,6 +557,7 @@ __global__ __launch_bounds__(256) void fw_bucket_tasks_kernel(const uint32_t* __
         out[t0 + k] = t;
       }
     }
+    __syncthreads();  // s_tot / s_base are reused by the next round
   }
 }
 
@@ -762,9 +774,9 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     }
     FW_HIP(hipMemsetAsync(pb->ctrs + 1, 0, 7 * sizeof(uint32_t), stream));
     FW_HIP(hipMemsetAsync(pb->count(nxt), 0, bucket_bytes, stream));
-    unsigned tblocks = ((unsigned)pb->n_buckets + 255u) / 256u;
-    if (tblocks > 2048u) tblocks = 2048u;
-    hipLaunchKernelGGL(fw_bucket_tasks_kernel, dim3(tblocks), dim3(256), 0, stream, pb->count(cur), pb->offset(),
+    unsigned tblocks = ((unsigned)pb->n_buckets + 1023u) / 1024u;
+    if (tblocks > 1024u) tblocks = 1024u;
+    hipLaunchKernelGGL(fw_bucket_tasks_kernel, dim3(tblocks), dim3(1024), 0, stream, pb->count(cur), pb->offset(),
                        pb->n_buckets, labels, g->hub_info, p->hub_threshold, pb->tasks, pb->wtasks,
                        pb->ctrs);
     FW_HIP(hipGetLastError());

@@ -128,6 +128,11 @@ __device__ __forceinline__ float readlane_f(float x, int l) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), l));
 }
 
+// Value of x in the lane whose number is byte_addr / 4 (any lane may read any lane).
+__device__ __forceinline__ float bperm_f(int byte_addr, float x) {
+  return __int_as_float(__builtin_amdgcn_ds_bpermute(byte_addr, __float_as_int(x)));
+}
+
 // ---- per-step context (wave-uniform) -----------------------------------------------------------
 
 struct StepCtx {
@@ -529,11 +534,19 @@ struct TaskTable {
   // Philox block 0 of stream 0 for the slot's next step, computed by the slot's own thread in phase C (64 blocks
   // per vector instruction instead of one block per scalar instruction stream)
   uint32_t draw[4][kWGT];
-  // per-round work lists, double buffered by round parity
-  int32_t small_list[2][kWGT];
-  int32_t hub_list[2][kWGT];
+  // per-round work lists, double buffered by round parity.  Lists of at most 16 (32) quartets use one (two) 16-lane
+  // rows of a wave, so four (two) of them are sampled by one wave at the same time; the others take a whole wave
+  // (small) or the whole workgroup (hub).
+  uint16_t tiny_list[2][kWGT];
+  uint16_t half_list[2][kWGT];
+  uint16_t small_list[2][kWGT];
+  uint16_t hub_list[2][kWGT];
+  int32_t tiny_count[2];
+  int32_t half_count[2];
   int32_t small_count[2];
   int32_t hub_count[2];
+  int32_t claim_tiny[2];
+  int32_t claim_half[2];
   int32_t claim[2];
   int32_t exhausted;
   uint32_t cursor;            // resume lists: entries of this workgroup's share handed out so far
@@ -546,6 +559,7 @@ struct TaskTable {
   // metapath only: the schema, so that the per-step label is an LDS read (a dynamic index into the
   // by-value kernel arguments would force a private copy of the whole array)
   int32_t schema[kApp == FW_APP_METAPATH ? FW_MAX_SCHEMA : 1];
+  int32_t want[kApp == FW_APP_METAPATH ? kWGT : 1];  // the label the slot's next step looks for
 };
 
 // The slot index is wave-uniform; readfirstlane tells the compiler so (scalar registers, scalar Philox).
@@ -584,6 +598,106 @@ __device__ __forceinline__ void commit(const fw_kargs& a, TaskTable<kWGT, kApp>&
   n_edges += (unsigned long long)(uint32_t)c.deg;
 }
 
+// One sampling step for 64 / kSeg task slots at once: slot s of the bundle owns the kSeg lanes starting at
+// s * kSeg (kSeg = 16 or 32, lists of at most kSeg quartets, one quartet per lane).  The arithmetic is the wave
+// sampler's: inside a 16-lane row the scan network is the same, row_bcast:15 joins the two rows of a 32-lane
+// segment exactly as it joins rows 0 and 1 of a whole wave, and the steps of the whole-wave scan that are left out
+// only ever add zeros for such a list, so every slot gets the element it would get from a wave of its own.
+// `slot` is this lane's slot or -1.  Not for node2vec (its biases need the adjacency test).
+template <int kApp, int kSeg, int kWGT>
+__device__ __forceinline__ void packed_step(const fw_kargs& a, TaskTable<kWGT, kApp>& tt, const int lane,
+                                            const int slot, unsigned long long& n_steps,
+                                            unsigned long long& n_edges) {
+  static_assert(kSeg == 16 || kSeg == 32, "a segment is one or two DPP rows");
+  const bool active = slot >= 0;
+  const int c = lane & (kSeg - 1);
+  const int seg_first = lane & ~(kSeg - 1);
+  uint32_t off = 0u, deg = 0u, d0 = 0u;
+  int32_t len = 1, want = 0;
+  if (active) {
+    off = tt.off[slot];
+    deg = (uint32_t)tt.deg[slot];
+    len = tt.len[slot];
+    d0 = tt.draw[0][slot];
+    if (kApp == FW_APP_METAPATH) want = tt.want[slot];
+  }
+  const uint32_t a0 = off & ~3u;
+  const uint32_t nq = (off + deg - a0 + 3u) >> 2;
+  const bool have = active && (uint32_t)c < nq;
+  const uint32_t base = a0 + 4u * (uint32_t)c;
+  const uint32_t* __restrict__ bias =
+      reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
+  uint4 raw = make_uint4(0, 0, 0, 0);
+  int4 adj = make_int4(-1, -1, -1, -1);
+  if (have) {
+    raw = *reinterpret_cast<const uint4*>(bias + base);
+    adj = *reinterpret_cast<const int4*>(a.adjncy + base);
+  }
+  float x[4];
+  if (kApp == FW_APP_METAPATH) {  // include/app.cuh:141-146
+    x[0] = (int32_t)raw.x == want ? 1.0f : 0.0f;
+    x[1] = (int32_t)raw.y == want ? 1.0f : 0.0f;
+    x[2] = (int32_t)raw.z == want ? 1.0f : 0.0f;
+    x[3] = (int32_t)raw.w == want ? 1.0f : 0.0f;
+  } else {
+    x[0] = __uint_as_float(raw.x);
+    x[1] = __uint_as_float(raw.y);
+    x[2] = __uint_as_float(raw.z);
+    x[3] = __uint_as_float(raw.w);
+  }
+  const uint32_t li = base - off;  // local index of the quartet's first slot (wraps below 0 for the head quartet)
+  const uint32_t lim = have ? deg : 0u;
+  x[0] = li < lim ? x[0] : 0.0f;
+  x[1] = li + 1u < lim ? x[1] : 0.0f;
+  x[2] = li + 2u < lim ? x[2] : 0.0f;
+  x[3] = li + 3u < lim ? x[3] : 0.0f;
+  float q = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) q = q + x[i];
+  float I = row_scan(q);
+  if (kSeg == 32) I = dpp_add_bcast15(I);
+  const float T = bperm_f((lane | (kSeg - 1)) << 2, I);  // the segment's total
+  const bool accept = T > 0.0f;                          // first group of an empty reservoir: S * 1 > 0
+  const float target = u24(d0) * T;
+  const bool pos = q > 0.0f;
+  const uint64_t mhit = __ballot(pos && I > target);
+  const uint64_t mpos = __ballot(pos);
+  const uint32_t seg_mask = kSeg == 32 ? 0xFFFFFFFFu : 0xFFFFu;
+  const uint32_t hit = (uint32_t)(mhit >> seg_first) & seg_mask;
+  const uint32_t any = (uint32_t)(mpos >> seg_first) & seg_mask;
+  // first lane of the segment with a positive total whose prefix exceeds the target, else the last positive one
+  const int l = hit != 0u ? __builtin_ctz(hit) : 31 - __builtin_clz(any | 1u);
+  // every lane resolves its own four elements; the answer of lane l of the segment is the one that is read
+  float e = I - q;
+  uint32_t cnt = 0u, pm = 0u;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    e = e + x[i];
+    cnt += e <= target ? 1u : 0u;
+    pm |= (x[i] > 0.0f ? 1u : 0u) << i;
+  }
+  const uint32_t cand = pm >> cnt;
+  const int pick = cand != 0u ? (int)cnt + __builtin_ctz(cand) : 31 - __builtin_clz(pm | 1u);
+  int32_t v = adj.x;
+  v = pick == 1 ? adj.y : v;
+  v = pick == 2 ? adj.z : v;
+  v = pick == 3 ? adj.w : v;
+  const int32_t selv = __builtin_amdgcn_ds_bpermute((seg_first + l) << 2, v);
+  if (active && c == 0) {  // commit (include/walker.cuh:1372-1385, Task::update include/gpu_task.cuh:70-77)
+    if (!accept) {
+      tt.flag[slot] = kFlagDead;
+    } else {
+      a.paths[(uint64_t)(uint32_t)tt.walker[slot] * (uint64_t)a.max_depth + (uint64_t)len] = selv;
+      tt.prev[slot] = tt.cur[slot];
+      tt.cur[slot] = selv;
+      tt.len[slot] = len + 1;
+      tt.flag[slot] = kFlagMoved;
+      n_steps += 1ull;
+      n_edges += (unsigned long long)deg;
+    }
+  }
+}
+
 // ---- the kernel --------------------------------------------------------------------------------
 
 template <int kApp, int kWGT>
@@ -604,8 +718,12 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
     for (int i = 0; i < FW_MAX_SCHEMA; ++i) tt.schema[i] = a.schema[i];
   }
   if (tid == 0) {
+    tt.tiny_count[0] = tt.tiny_count[1] = 0;
+    tt.half_count[0] = tt.half_count[1] = 0;
     tt.small_count[0] = tt.small_count[1] = 0;
     tt.hub_count[0] = tt.hub_count[1] = 0;
+    tt.claim_tiny[0] = tt.claim_tiny[1] = 0;
+    tt.claim_half[0] = tt.claim_half[1] = 0;
     tt.claim[0] = tt.claim[1] = 0;
     tt.exhausted = 0;
     tt.cursor = 0u;
@@ -619,7 +737,9 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
     if (!first) {
       const int nh = tt.hub_count[parity];
       const int ns = tt.small_count[parity];
-      if (nh + ns == 0) break;  // uniform: read after the barrier that closed phase C
+      const int nt = tt.tiny_count[parity];
+      const int nf = tt.half_count[parity];
+      if (nh + ns + nt + nf == 0) break;  // uniform: read after the barrier that closed phase C
 
       // ---- phase B: hubs, whole workgroup ----
       for (int hb = 0; hb < nh; hb += kHubChunk) {
@@ -670,7 +790,27 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
         if (hb + kHubChunk < nh) __syncthreads();  // the partial buffers are reused by the next chunk
       }
 
-      // ---- phase A: remaining slots, one wave each, claimed dynamically ----
+      // ---- phase A: remaining slots, claimed dynamically: four or two short lists per wave, else one ----
+      if (kApp != FW_APP_NODE2VEC) {
+        for (;;) {
+          int idx = 0;
+          if (lane == 0) idx = atomicAdd(&tt.claim_tiny[parity], 4);
+          idx = __builtin_amdgcn_readfirstlane(idx);
+          if (idx >= nt) break;
+          const int entry = idx + (lane >> 4);
+          const int slot = entry < nt ? (int)tt.tiny_list[parity][entry] : -1;
+          packed_step<kApp, 16, kWGT>(a, tt, lane, slot, n_steps, n_edges);
+        }
+        for (;;) {
+          int idx = 0;
+          if (lane == 0) idx = atomicAdd(&tt.claim_half[parity], 2);
+          idx = __builtin_amdgcn_readfirstlane(idx);
+          if (idx >= nf) break;
+          const int entry = idx + (lane >> 5);
+          const int slot = entry < nf ? (int)tt.half_list[parity][entry] : -1;
+          packed_step<kApp, 32, kWGT>(a, tt, lane, slot, n_steps, n_edges);
+        }
+      }
       for (;;) {
         int idx = 0;
         if (lane == 0) idx = atomicAdd(&tt.claim[parity], 1);
@@ -701,8 +841,12 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
       }
       __syncthreads();
       if (tid == 0) {  // this round's lists are drained; they become the lists produced two rounds later
+        tt.tiny_count[parity] = 0;
+        tt.half_count[parity] = 0;
         tt.small_count[parity] = 0;
         tt.hub_count[parity] = 0;
+        tt.claim_tiny[parity] = 0;
+        tt.claim_half[parity] = 0;
         tt.claim[parity] = 0;
       }
       parity ^= 1;
@@ -825,9 +969,18 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
         tt.len[tid] = len;
         tt.flag[tid] = 0;
         if (deg > a.hub_threshold) {
-          tt.hub_list[np][atomicAdd(&tt.hub_count[np], 1)] = tid;
+          tt.hub_list[np][atomicAdd(&tt.hub_count[np], 1)] = (uint16_t)tid;
         } else {
-          tt.small_list[np][atomicAdd(&tt.small_count[np], 1)] = tid;
+          const uint32_t o = tt.off[tid];
+          const uint32_t nq = (o + (uint32_t)deg - (o & ~3u) + 3u) >> 2;
+          if (kApp != FW_APP_NODE2VEC && nq <= 16u) {
+            tt.tiny_list[np][atomicAdd(&tt.tiny_count[np], 1)] = (uint16_t)tid;
+          } else if (kApp != FW_APP_NODE2VEC && nq <= 32u) {
+            tt.half_list[np][atomicAdd(&tt.half_count[np], 1)] = (uint16_t)tid;
+          } else {
+            tt.small_list[np][atomicAdd(&tt.small_count[np], 1)] = (uint16_t)tid;
+          }
+          if (kApp == FW_APP_METAPATH) tt.want[tid] = tt.schema[(uint32_t)(len - 1) % (uint32_t)a.schema_len];
           const uint4 b = philox4x32_10(a.walker_base + (uint32_t)tt.walker[tid], (uint32_t)(len - 1), 0u, 0u,
                                         a.seed_lo, a.seed_hi);
           tt.draw[0][tid] = b.x;
@@ -882,10 +1035,6 @@ __device__ __forceinline__ float next_uniform_lane(LaneDraw& d, const fw_kargs& 
   d.q0 = d.q1; d.q1 = d.q2; d.q2 = d.q3;
   --d.avail;
   return u;
-}
-
-__device__ __forceinline__ float bperm_f(int byte_addr, float x) {
-  return __int_as_float(__builtin_amdgcn_ds_bpermute(byte_addr, __float_as_int(x)));
 }
 
 // The groups w, w + nw, ... of one list for up to 64 walkers at once (lane i = walker i).  Outputs the total S
