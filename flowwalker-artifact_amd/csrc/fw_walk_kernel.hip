@@ -219,11 +219,21 @@ __device__ __forceinline__ uint32_t coop_lower_bound(const int32_t* __restrict__
   return lo + (uint32_t)__builtin_popcountll(__ballot(lt));
 }
 
-// Per-wave LDS scratch of the reversed adjacency test (entries of N(prev) looked up in N(cur)).
-constexpr int kN2vChunk = 256;  // entries of N(prev) resolved per refill: 4 per lane
+// Per-wave LDS scratch of the adjacency test.  Forward test (neighbours of cur looked up in N(prev)): `window`
+// holds the part of N(prev) that can contain the current group's vertices, so the per-lane searches run in LDS.
+// Reversed test (entries of N(prev) looked up in N(cur)): `match` and `mask` share the same memory.
+constexpr int kN2vChunk = 256;    // entries of N(prev) resolved per refill: 4 per lane
+constexpr int kN2vWindow = 1024;  // entries of N(prev) staged per group
+constexpr int kN2vMaxWindows = 16;   // longer stretches of N(prev) per group are searched in place
+constexpr uint64_t kN2vReverseRatio = 8;  // reversed test when N(prev) is at least this many times shorter than N(cur)
 struct N2vScratch {
-  int32_t match[kN2vChunk];  // local indices in N(cur) of common neighbours, ascending
-  uint32_t mask[64];         // per lane: bit i set = the lane's i-th bias of the current group is a common neighbour
+  union {
+    int32_t window[kN2vWindow];
+    struct {
+      int32_t match[kN2vChunk];  // local indices in N(cur) of common neighbours, ascending
+      uint32_t mask[64];         // per lane: bit i set = the lane's i-th bias of the current group is a common neighbour
+    };
+  };
 };
 
 // Wave-uniform cursor of the reversed test.
@@ -314,7 +324,7 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
       reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
   const bool n2v = kApp == FW_APP_NODE2VEC && c.prev != -1;
   // reversed adjacency test: look the entries of the shorter list N(prev) up in N(cur) (wave granularity only)
-  const bool reversed = n2v && nw == 1u && c.prev_deg <= c.deg;
+  const bool reversed = n2v && nw == 1u && (uint64_t)(uint32_t)c.prev_deg * kN2vReverseRatio <= (uint64_t)(uint32_t)c.deg;
   const bool need_adj = kTrackV || (n2v && !reversed);
   N2vCursor cur;
   int32_t ret_idx = -1;  // local index of prev in N(cur): the return edge (include/app.cuh:113-114)
@@ -446,19 +456,103 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
       }
       vmax = wave_max_i32(vmax);
       // N(prev)[seg_lo, seg_hi) can hold this group's vertices; later groups only hold larger ones
+      if (nw > 1u) {  // this wave skipped the groups of the other waves: drop the entries below this group's first vertex
+        const int32_t gs = (int32_t)(a0 + 4u * g * kG - c.off);
+        const int32_t vmin = a.adjncy[c.off + (uint32_t)(gs > 0 ? gs : 0)];
+        seg_lo = coop_lower_bound(plist, seg_lo, (uint32_t)c.prev_deg, vmin, lane);
+      }
       const uint32_t seg_hi = coop_upper_bound(plist, seg_lo, (uint32_t)c.prev_deg, vmax, lane);
-      uint32_t pos = seg_lo;
+      const uint32_t p_lo = c.prev_off + seg_lo, p_hi = c.prev_off + seg_hi;  // the segment as CSR indices
+      const uint32_t wa = p_lo & ~3u;
+      if (p_hi - wa <= (uint32_t)kN2vWindow) {
+        // the segment fits the window: stage it with aligned 16-byte loads, then search in LDS
+        __builtin_amdgcn_wave_barrier();  // the previous group's searches are done
 #pragma unroll
-      for (int j = 0; j < kJ; ++j) {
-        const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
+        for (int k = 0; k < kN2vWindow / 256; ++k) {
+          const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
+          if (wa + wi < p_hi)
+            *reinterpret_cast<int4*>(&scr->window[wi]) = *reinterpret_cast<const int4*>(a.adjncy + wa + wi);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int32_t* win = scr->window;
+        const uint32_t hi_w = p_hi - wa;
+        uint32_t pos = p_lo - wa;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (post[e] == c.prev) {
-            x[4 * j + e] = x[4 * j + e] * a.inv_p;
-          } else {
-            pos = gallop_lower_bound(plist, pos, seg_hi, post[e]);
-            const bool common = pos < seg_hi && plist[pos] == post[e];
-            x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
+        for (int j = 0; j < kJ; ++j) {
+          const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (post[e] == c.prev) {
+              x[4 * j + e] = x[4 * j + e] * a.inv_p;
+            } else {
+              pos = gallop_lower_bound(win, pos, hi_w, post[e]);
+              const bool common = pos < hi_w && win[pos] == post[e];
+              x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
+            }
+          }
+        }
+      } else if (p_hi - wa <= (uint32_t)(kN2vMaxWindows * kN2vWindow)) {
+        // the segment is a few windows long: stream it through the window; a neighbour is resolved in the first
+        // window whose last entry is not smaller (both lists ascend, so a lane's neighbours come up in order)
+        uint32_t done = 0u;  // bit i: bias i is final
+#pragma unroll
+        for (int j = 0; j < kJ; ++j) {
+          const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (post[e] == c.prev) {
+              x[4 * j + e] = x[4 * j + e] * a.inv_p;
+              done |= 1u << (4 * j + e);
+            }
+          }
+        }
+        for (uint32_t ws = wa; ws < p_hi; ws += (uint32_t)kN2vWindow) {
+          __builtin_amdgcn_wave_barrier();  // the previous window's searches are done
+#pragma unroll
+          for (int k = 0; k < kN2vWindow / 256; ++k) {
+            const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
+            if (ws + wi < p_hi)
+              *reinterpret_cast<int4*>(&scr->window[wi]) = *reinterpret_cast<const int4*>(a.adjncy + ws + wi);
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          const int32_t* win = scr->window;
+          const uint32_t hi_w = (p_hi - ws) < (uint32_t)kN2vWindow ? (p_hi - ws) : (uint32_t)kN2vWindow;
+          const bool last = ws + (uint32_t)kN2vWindow >= p_hi;
+          const int32_t wmax = win[hi_w - 1u];
+          uint32_t pos = ws == wa ? p_lo - wa : 0u;
+#pragma unroll
+          for (int j = 0; j < kJ; ++j) {
+            const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int i = 4 * j + e;
+              if (((done >> i) & 1u) == 0u && (post[e] <= wmax || last)) {
+                pos = gallop_lower_bound(win, pos, hi_w, post[e]);
+                const bool common = pos < hi_w && win[pos] == post[e];
+                x[i] = common ? x[i] : x[i] * a.inv_q;
+                done |= 1u << i;
+              }
+            }
+          }
+        }
+      } else {  // a long stretch of N(prev) against few neighbours: search it in place, galloping from hit to hit
+        uint32_t pos = seg_lo;
+#pragma unroll
+        for (int j = 0; j < kJ; ++j) {
+          const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (post[e] == c.prev) {
+              x[4 * j + e] = x[4 * j + e] * a.inv_p;
+            } else {
+              pos = gallop_lower_bound(plist, pos, seg_hi, post[e]);
+              const bool common = pos < seg_hi && plist[pos] == post[e];
+              x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
+            }
           }
         }
       }

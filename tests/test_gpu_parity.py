@@ -68,6 +68,20 @@ def test_node2vec(gpu, hub):
     _check(gpu, hub, starts, app=gpu.APP_NODE2VEC, max_depth=16, p=2.0, q=0.5, hub_threshold=1000, seed=6)
 
 
+def test_node2vec_adjacency_test_strategies(gpu):
+    """The node2vec bias needs "is this neighbour of cur also a neighbour of prev?".  The kernel answers it in four
+    ways depending on the two list lengths (N(prev) entries looked up in N(cur); the stretch of N(prev) staged in LDS,
+    one window or several; searched in place) at wave and at workgroup granularity.  All must give the oracle's walks."""
+    csr = _graphs.hub_graph(V=40000, hub_degrees=(30000, 20000, 5000, 600, 70), base_degree=4, seed=23)
+    starts = np.random.RandomState(6).randint(0, 40000, size=4000).astype(np.int32)
+    starts[:300] = 0    # 30000-degree hub: its neighbours see it as prev (a stretch of many windows, or in place)
+    starts[300:500] = 1
+    starts[500:600] = 2
+    for thr in (64, 4096, 1 << 30):
+        _check(gpu, csr, starts, app=gpu.APP_NODE2VEC, max_depth=9, p=0.5, q=2.0, hub_threshold=thr, seed=31)
+    _check(gpu, csr, starts, app=gpu.APP_NODE2VEC, max_depth=9, p=4.0, q=0.25, hub_threshold=1000, wg_threads=256, seed=32)
+
+
 def test_metapath(gpu, hub):
     starts = np.arange(0, 12000, 2, dtype=np.int32)
     _check(gpu, hub, starts, app=gpu.APP_METAPATH, max_depth=6, schema=[0, 1, 2, 3, 4], hub_threshold=1000, seed=7)
