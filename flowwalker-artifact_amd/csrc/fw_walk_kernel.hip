@@ -251,21 +251,38 @@ __device__ __forceinline__ void n2v_refill(const int32_t* __restrict__ clist, ui
                                            N2vCursor& k, int lane) {
   const uint32_t cnt = (dp - k.pc) < (uint32_t)kN2vChunk ? (dp - k.pc) : (uint32_t)kN2vChunk;
   const uint32_t base = k.pc + 4u * (uint32_t)lane;
-  uint32_t pos = k.cov;
+  // The four look-ups of a lane do not depend on each other, and the entries of a short N(prev) lie far apart in
+  // N(cur): plain binary searches over the unresolved part, advancing together (one memory latency per round
+  // for all four, instead of galloping from hit to hit).
   uint32_t hit_pos[4];
   bool hit[4];
+  int32_t y[4];
+  bool valid[4];
+  uint32_t lo[4], hi[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    valid[e] = base + (uint32_t)e < k.pc + cnt;
+    y[e] = valid[e] ? plist[base + (uint32_t)e] : 0;
+    lo[e] = k.cov;
+    hi[e] = valid[e] ? dc : k.cov;
+  }
+  for (uint32_t span = dc - k.cov; span != 0u; span >>= 1) {  // ceil(log2(span + 1)) rounds close every search
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const bool open = lo[e] < hi[e];
+      const uint32_t mid = (lo[e] + hi[e]) >> 1;
+      const int32_t val = open ? clist[mid] : 0;
+      const bool less = open && val < y[e];
+      lo[e] = less ? mid + 1u : lo[e];
+      hi[e] = (open && !less) ? mid : hi[e];
+    }
+  }
   uint32_t resolved = k.cov;  // after this lane's last entry: indices below are resolved
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    hit[e] = false;
-    hit_pos[e] = 0u;
-    if (base + (uint32_t)e < k.pc + cnt) {
-      const int32_t y = plist[base + (uint32_t)e];
-      pos = gallop_lower_bound(clist, pos, dc, y);
-      hit[e] = pos < dc && clist[pos] == y;
-      hit_pos[e] = pos;
-      resolved = pos + (hit[e] ? 1u : 0u);
-    }
+    hit_pos[e] = lo[e];
+    hit[e] = valid[e] && lo[e] < dc && clist[lo[e]] == y[e];
+    if (valid[e]) resolved = lo[e] + (hit[e] ? 1u : 0u);
   }
   const uint64_t m0 = __ballot(hit[0]), m1 = __ballot(hit[1]), m2 = __ballot(hit[2]), m3 = __ballot(hit[3]);
   const uint64_t below = (1ull << lane) - 1ull;
