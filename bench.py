@@ -41,7 +41,7 @@ HEADLINE = "deepwalk_rmat24_sym"
 # HBM-side bytes of one pass (all fw_walk_zprs + fw_hub_batch launches) from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs, each scaled by what the same counter reads for the 1 GiB copy kernel (profiles/).
 # None for workloads that have not been measured.
-MEASURED_TRAFFIC_BYTES = {"deepwalk_rmat24_sym": 2.225e12}
+MEASURED_TRAFFIC_BYTES = {"deepwalk_rmat24_sym": 6.58e11}
 
 
 def algorithmic_bytes(app, steps, sampled_edges, queries, probe_terms=0):
@@ -161,7 +161,8 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload if not args.scale else None),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(
+                args.workload if not args.scale and args.park_threshold == 0 and last.launches > 1 else None),
             "kernel": "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_batch pipeline",
             "kernel_ms": avg_kernel_ms,
             "algorithmic_bytes": int(alg_bytes),
