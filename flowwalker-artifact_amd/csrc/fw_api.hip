@@ -453,7 +453,8 @@ __global__ void fw_hub_index_kernel(const uint32_t* __restrict__ xadj, int32_t V
       hi.pad = 0u;
       hub_info[idx] = hi;
     }
-    hub_index[v] = idx;
+    // -1: not parked on; -2: no neighbours at all (a walker that arrives there is finished)
+    hub_index[v] = idx >= 0 ? idx : (xadj[v + 1] == xadj[v] ? -2 : -1);
   }
 }
 
@@ -589,6 +590,53 @@ __global__ void fw_scatter_counted_kernel(const fw_walker_rec* __restrict__ src,
   }
 }
 
+// Copies the records of a batch launch's output list that continue in the walk kernel (not finished, not parked
+// again) to a dense list, so that the walk kernel's refill rounds do not scan the holes.  One update of the
+// (contended) list counter per 4096 records.
+__global__ __launch_bounds__(1024) void fw_compact_resume_kernel(const fw_walker_rec* __restrict__ out, uint32_t m,
+                                                                 fw_walker_rec* __restrict__ resume, uint32_t* count) {
+  __shared__ uint32_t s_wave[16];
+  __shared__ uint32_t s_base;
+  const int lane = (int)(threadIdx.x & 63u);
+  const int wave = (int)(threadIdx.x >> 6);
+  for (uint32_t base = blockIdx.x * 4096u; base < m; base += gridDim.x * 4096u) {  // uniform per workgroup
+    fw_walker_rec r[4];
+    uint32_t n = 0u;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t i = base + (uint32_t)k * 1024u + threadIdx.x;
+      r[k].q = -1; r[k].cur = 0; r[k].prev = 0; r[k].len = 0;
+      if (i < m) r[k] = out[i];
+      if (r[k].q < 0 || (r[k].len & FW_REC_PARK) != 0) r[k].q = -1;
+      n += r[k].q >= 0 ? 1u : 0u;
+    }
+    uint32_t incl = n;  // inclusive wave scan
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const uint32_t up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      uint32_t total = 0u;
+      for (int w = 0; w < 16; ++w) {
+        const uint32_t v = s_wave[w];
+        s_wave[w] = total;
+        total += v;
+      }
+      s_base = total != 0u ? atomicAdd(count, total) : 0u;
+    }
+    __syncthreads();
+    uint32_t at = s_base + s_wave[wave] + incl - n;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (r[k].q >= 0) resume[at++] = r[k];
+    }
+    __syncthreads();  // s_wave / s_base are reused by the next chunk
+  }
+}
+
 // Parked records name their bucket; the walk kernel wants the vertex (used when the last few walkers leave the
 // park / batch loop).
 __global__ void fw_bucket_to_vertex_kernel(fw_walker_rec* recs, uint32_t m, const fw_hub_info* __restrict__ hub_info,
@@ -607,11 +655,12 @@ struct ParkBuffers {
   fw_walker_rec* walked = nullptr;
   fw_walker_rec* sorted = nullptr;
   fw_walker_rec* out = nullptr;
+  fw_walker_rec* resume = nullptr;    // the records of `out` that continue in the walk kernel, dense
   uint32_t* buckets = nullptr;        // [4 * n_buckets]: count of round parity 0, of parity 1, offset, fill
   fw_batch_task* tasks = nullptr;
   fw_batch_task* wtasks = nullptr;
   uint32_t* ctrs = nullptr;           // [0] walkers in `walked`, [1] records of `out` that resume, [2] that are parked
-                                      // again, [3] workgroup tasks, [4] their dispenser, [5] wave tasks
+                                      // again, [3] workgroup tasks, [4] their dispenser, [5] wave tasks, [6] records in `resume`
   uint32_t* h_ctrs = nullptr;         // pinned mirror
   void* tmp = nullptr;                // scan temporary storage
   size_t scan_bytes = 0;
@@ -627,6 +676,7 @@ struct ParkBuffers {
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&walked), cap * sizeof(fw_walker_rec)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&sorted), cap * sizeof(fw_walker_rec)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&out), cap * sizeof(fw_walker_rec)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&resume), cap * sizeof(fw_walker_rec)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&buckets), (size_t)4 * n * sizeof(uint32_t)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&tasks), ntask * sizeof(fw_batch_task)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&wtasks), ntask * sizeof(fw_batch_task)));
@@ -638,10 +688,10 @@ struct ParkBuffers {
     return FW_OK;
   }
   void release() {
-    void* dev[8] = {walked, sorted, out, buckets, tasks, wtasks, ctrs, tmp};
+    void* dev[9] = {walked, sorted, out, resume, buckets, tasks, wtasks, ctrs, tmp};
     for (void* p : dev) if (p) (void)hipFree(p);
     if (h_ctrs) (void)hipHostFree(h_ctrs);
-    walked = sorted = out = nullptr;
+    walked = sorted = out = resume = nullptr;
     buckets = ctrs = h_ctrs = nullptr;
     tasks = wtasks = nullptr;
     tmp = nullptr;
@@ -787,6 +837,13 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     if (rc != FW_OK) return rc;
     if ((rc = th.end(stream)) != FW_OK) return rc;
     ++*launches;
+    {
+      unsigned cblocks = ((unsigned)m + 4095u) / 4096u;
+      if (cblocks > 1024u) cblocks = 1024u;
+      hipLaunchKernelGGL(fw_compact_resume_kernel, dim3(cblocks), dim3(1024), 0, stream, pb->out, (uint32_t)m,
+                         pb->resume, pb->ctrs + 6);
+      FW_HIP(hipGetLastError());
+    }
     FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, 8 * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     FW_HIP(hipStreamSynchronize(stream));
     th.collect(&times->hub_ms);
@@ -795,11 +852,11 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
               (unsigned long long)m, n_walked, n_again, pb->h_ctrs[3], pb->h_ctrs[5], pb->h_ctrs[1], pb->h_ctrs[2]);
     n_out = (uint32_t)m;
     pb->h_ctrs[0] = 0u;
-    if (pb->h_ctrs[1] != 0u) {
-      // walkers on vertices below the threshold continue in the walk kernel, which takes them from the batch
-      // output list (skipping the other records) and counts the walkers it parks in the same bucket array
-      a.resume = pb->out;
-      a.n = (int32_t)n_out;
+    if (pb->h_ctrs[6] != 0u) {
+      // walkers on vertices below the threshold continue in the walk kernel, which counts the walkers it parks in
+      // the same bucket array as the batch launch did
+      a.resume = pb->resume;
+      a.n = (int32_t)pb->h_ctrs[6];
       a.bucket_count = pb->count(nxt);
       const uint32_t n_again_now = pb->h_ctrs[2];
       if ((rc = walk(nullptr)) != FW_OK) return rc;

@@ -31,7 +31,7 @@ struct fw_graph {
   // lazily built index of the vertices whose degree exceeds hub_index_threshold (hub parking)
   int32_t hub_index_threshold = -1;
   int32_t n_hubs = 0;
-  int32_t* hub_index = nullptr;       // int32[V]: position in hub_info, or -1
+  int32_t* hub_index = nullptr;       // int32[V]: position in hub_info, -1 (not parked on) or -2 (degree 0)
   struct fw_hub_info* hub_info = nullptr;  // [n_hubs]
 };
 
@@ -68,7 +68,7 @@ struct fw_kargs {
   // hub parking (park_threshold = INT32_MAX switches it off)
   int32_t park_threshold;            // a walker that arrives on a vertex of larger degree is parked
   int32_t n_labels_per_hub;          // buckets per hub: 1, or schema_len for metapath (walkers wanting one label share a scan)
-  const int32_t* hub_index;          // int32[V]
+  const int32_t* hub_index;          // int32[V]: index of the vertex among the parked-on ones, -1, or -2 = degree 0
   fw_walker_rec* parked;             // out: parked walkers
   uint32_t* parked_count;
   uint32_t* bucket_count;            // [n_hubs * n_labels_per_hub]

@@ -970,12 +970,16 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
       int32_t len = tt.len[tid];
       bool need = tid < a.slot_limit;  // slot wants a new walker
       bool park = false;               // the slot's walker has reached a hub that is served by the batch kernel
+      int32_t hidx = -1;               // that vertex's index among the parked-on ones (read together with its CSR range)
+      const bool parking = a.park_threshold != 0x7FFFFFFF;
+      const bool by_position = parking || a.resume != nullptr;
       int32_t deg = 0;
       if (len >= 0) {
         if (tt.flag[tid] == kFlagMoved) {
           const int32_t v = tt.cur[tid];
           const uint32_t o = a.xadj[v];
           const uint32_t e = a.xadj[v + 1];
+          if (parking) hidx = a.hub_index[v];
           deg = (int32_t)(e - o);
           tt.off[tid] = o;
           tt.deg[tid] = deg;
@@ -986,7 +990,7 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
             stop = u24(bits) < a.tp;
           }
           need = stop;
-          park = !stop && deg > a.park_threshold;
+          park = !stop && hidx >= 0;  // same as deg > park_threshold
         }
         // kFlagDead: dead end (no neighbour with positive bias), include/walker.cuh:1373-1374
       }
@@ -1004,7 +1008,7 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
             const int32_t v = tt.cur[tid];
             const uint32_t label_slot =
                 kApp == FW_APP_METAPATH ? (uint32_t)(len - 1) % (uint32_t)a.n_labels_per_hub : 0u;
-            const uint32_t bucket = (uint32_t)a.hub_index[v] * (uint32_t)a.n_labels_per_hub + label_slot;
+            const uint32_t bucket = (uint32_t)hidx * (uint32_t)a.n_labels_per_hub + label_slot;
             fw_walker_rec rec;
             rec.q = tt.walker[tid];
             rec.cur = (int32_t)bucket;  // the vertex follows from the bucket
@@ -1025,16 +1029,18 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
         uint32_t base = 0;
         const int leader = __builtin_ctzll(m);
         if (lane == leader) {
-          // fresh queries come from the global dispenser (include/walker.cuh:1339,1423); the entries of a resume
-          // list are dealt out by position -- the workgroups take interleaved chunks of slot_limit entries -- with
-          // a workgroup-local cursor, because a list is long (it has holes) and a global counter is contended
-          base = a.resume != nullptr ? atomicAdd(&tt.cursor, (uint32_t)__builtin_popcountll(m))
-                                     : atomicAdd(a.dispenser, (uint32_t)__builtin_popcountll(m));
+          // Without parking a walker stays in its slot for its whole walk, and queries come from the global
+          // dispenser (include/walker.cuh:1339,1423) so that the workgroups balance.  With parking every launch
+          // is short and there are many: the entries (fresh queries or a resume list) are dealt out by position
+          // -- the workgroups take interleaved chunks of slot_limit entries -- with a workgroup-local cursor,
+          // because a global counter is contended (about 13 ns per update).
+          base = by_position ? atomicAdd(&tt.cursor, (uint32_t)__builtin_popcountll(m))
+                             : atomicAdd(a.dispenser, (uint32_t)__builtin_popcountll(m));
         }
         base = (uint32_t)__builtin_amdgcn_readlane((int)base, leader);
         if (want) {
           uint32_t q = base + (uint32_t)__builtin_popcountll(m & ((1ull << lane) - 1ull));
-          if (a.resume != nullptr) {
+          if (by_position) {
             const uint32_t chunk = q / (uint32_t)a.slot_limit;
             const uint64_t pos = ((uint64_t)chunk * gridDim.x + blockIdx.x) * (uint64_t)a.slot_limit +
                                  (q - chunk * (uint32_t)a.slot_limit);
@@ -1054,6 +1060,7 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
             if ((uint32_t)sp < (uint32_t)a.V && ln < a.max_depth) {
               const uint32_t o = a.xadj[sp];
               const uint32_t e = a.xadj[sp + 1];
+              if (parking) hidx = a.hub_index[sp];
               deg = (int32_t)(e - o);
               if (deg > 0) {
                 tt.walker[tid] = wq;
@@ -1065,7 +1072,7 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
                 tt.prev_deg[tid] = 0;
                 len = ln;
                 need = false;
-                park = deg > a.park_threshold;
+                park = hidx >= 0;  // same as deg > park_threshold
               }
             }
           } else {
@@ -1294,10 +1301,13 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
     n_edges += c * (unsigned long long)deg;
   }
   bool park = false;
+  int32_t hidx = -1;
   if (go_on) {
-    const int32_t ndeg = (int32_t)(a.xadj[nv + 1] - a.xadj[nv]);
-    go_on = ndeg > 0;  // a dead end finishes the walk (include/walker.cuh:1373-1374)
-    park = ndeg > a.park_threshold;
+    // one look-up tells both what the step commit needs to know about the new vertex: parked on (index >= 0),
+    // a dead end that finishes the walk (-2, include/walker.cuh:1373-1374), or neither
+    hidx = a.hub_index[nv];
+    go_on = hidx != -2;
+    park = hidx >= 0;
   }
   if (have) {
     fw_walker_rec out;
@@ -1307,7 +1317,7 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
     out.len = rec.len + 1;
     if (go_on && park) {
       const uint32_t label_slot = kApp == FW_APP_METAPATH ? (uint32_t)rec.len % (uint32_t)a.n_labels_per_hub : 0u;
-      const uint32_t bucket = (uint32_t)a.hub_index[nv] * (uint32_t)a.n_labels_per_hub + label_slot;
+      const uint32_t bucket = (uint32_t)hidx * (uint32_t)a.n_labels_per_hub + label_slot;
       out.cur = (int32_t)bucket;  // the vertex follows from the bucket
       out.prev = (int32_t)atomicAdd(&h.bucket_out[bucket], 1u);
       out.len |= FW_REC_PARK;
