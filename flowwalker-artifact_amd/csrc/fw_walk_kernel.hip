@@ -355,6 +355,29 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
   int32_t sel = -1, selv = -1;
   DrawQueue dq = dq0;  // empty, or block 0 of this wave's stream computed ahead by the slot's own thread
   uint32_t seg_lo = 0u;  // node2vec: entries of N(prev) below this index are smaller than anything still to come
+  // node2vec, forward test, N(prev) short enough for the window: stage all of it once per step; every lane then
+  // gallops through it in LDS from where its previous neighbour ended (a lane's neighbours ascend across groups too)
+  bool p_staged = false;
+  uint32_t st_hi = 0u, lane_pos = 0u;
+  if (kApp == FW_APP_NODE2VEC && n2v && !reversed) {
+    const uint32_t wa = c.prev_off & ~3u;
+    const uint32_t p_end = c.prev_off + (uint32_t)c.prev_deg;
+    if (p_end - wa <= (uint32_t)kN2vWindow) {
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int k = 0; k < kN2vWindow / 256; ++k) {
+        const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
+        if (wa + wi < p_end)
+          *reinterpret_cast<int4*>(&scr->window[wi]) = *reinterpret_cast<const int4*>(a.adjncy + wa + wi);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      p_staged = true;
+      lane_pos = c.prev_off - wa;
+      st_hi = p_end - wa;
+    }
+  }
 
   for (uint32_t g = w; g < ngroups; g += nw) {
     const uint32_t kb = g * kG + (uint32_t)lane;  // this lane's quartet for j = 0
@@ -459,6 +482,22 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
         const float wq = x[i] * a.inv_q;
         const float wp = x[i] * a.inv_p;
         x[i] = (i == ret_slot) ? wp : (((common >> i) & 1u) ? x[i] : wq);
+      }
+    } else if (n2v && p_staged) {  // include/app.cuh:108-123 against the staged N(prev)
+      const int32_t* win = scr->window;
+#pragma unroll
+      for (int j = 0; j < kJ; ++j) {
+        const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (post[e] == c.prev) {  // the return edge, or an entry outside the list (bias 0 already)
+            x[4 * j + e] = x[4 * j + e] * a.inv_p;
+          } else {
+            lane_pos = gallop_lower_bound(win, lane_pos, st_hi, post[e]);
+            const bool common = lane_pos < st_hi && win[lane_pos] == post[e];
+            x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
+          }
+        }
       }
     } else if (n2v) {  // include/app.cuh:108-123: w/p back to prev, w for common neighbours, w/q otherwise
       const int32_t* __restrict__ plist = a.adjncy + c.prev_off;
