@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the walk path: one "step" = one pass of the walk kernel over the whole query batch.
 
-Default workload = the headline of BASELINE.json: DeepWalk, length 80, one query per vertex, on the
+Default workload = the headline configuration: DeepWalk, length 80, one query per vertex, on the
 symmetrised R-MAT scale-24 graph (edge factor 16, a/b/c/d = .57/.19/.19/.05, weights U[1,100)).
 Inputs (CSR, start vertices, path matrix) are resident in HBM before the timed region starts.
 
@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
-# name -> generator / walk settings.  Scales follow BASELINE.json's configs; "headline" is the metric's.
+# name -> generator / walk settings of the five benchmark configurations; "headline" is the one the metric is quoted on.
 WORKLOADS = {
     "deepwalk_rmat24_sym": dict(scale=24, sym=True, app="deepwalk", depth=80, queries="all", labels=0),
     "deepwalk_rmat22": dict(scale=22, sym=False, app="deepwalk", depth=80, queries="all", labels=0),

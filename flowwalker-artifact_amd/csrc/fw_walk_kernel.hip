@@ -1399,7 +1399,35 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
   unsigned long long n_steps = 0ull, n_edges = 0ull;
   uint32_t n_out[2] = {0u, 0u};  // walkers that resume / that are parked again
 
-  // ---- workgroup tasks: lists above hub_threshold, sampled at workgroup granularity ----
+  __syncthreads();  // the shared initialisation above is visible
+
+  // ---- wave tasks first: lists up to hub_threshold, sampled at wave granularity, one batch per wave; the tasks are
+  //      short and many, so they are dealt out by position instead of through a contended counter ----
+  const uint32_t nwaves = gridDim.x * (uint32_t)kNW;
+  for (uint32_t t = blockIdx.x * (uint32_t)kNW + (uint32_t)wave; t < nwtasks; t += nwaves) {
+    const fw_batch_task* tp = h.wtasks + t;
+    const int32_t v = __builtin_amdgcn_readfirstlane(tp->v);
+    const uint32_t off = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->off);
+    const uint32_t deg = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->deg);
+    const uint32_t rec_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->rec_base);
+    const int count = __builtin_amdgcn_readfirstlane(tp->count);
+    const int32_t want = kApp == FW_APP_METAPATH ? s_schema[__builtin_amdgcn_readfirstlane(tp->slot)] : 0;
+
+    const bool have = lane < count;
+    fw_walker_rec rec;
+    rec.q = 0; rec.cur = v; rec.prev = -1; rec.len = 1;
+    if (have) rec = h.sorted[rec_base + (uint32_t)lane];
+    const uint32_t walker = a.walker_base + (uint32_t)rec.q;
+    const uint32_t step = (uint32_t)(rec.len - 1);
+
+    float S;
+    int32_t sel;
+    batch_stream<kApp>(a, bias, off, deg, want, 0u, 1u, have, walker, step, lane, S, sel);
+    batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, have, sel, walker, step, lane, n_steps, n_edges, n_out);
+  }
+
+  // ---- then workgroup tasks: lists above hub_threshold, sampled at workgroup granularity.  They are handed out
+  //      dynamically, which evens out what the fixed deal of the wave tasks left uneven ----
   for (;;) {
     if (tid == 0) s_task = atomicAdd(h.task_next, 1u);
     __syncthreads();
@@ -1450,31 +1478,6 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
       batch_commit<kApp>(a, h, task.v, task.off, task.deg, task.rec_base, rec, have, pick, walker, step, lane,
                          n_steps, n_edges, n_out);
     }
-  }
-
-  // ---- wave tasks: lists up to hub_threshold, sampled at wave granularity, one batch per wave; the tasks are
-  //      short and many, so they are dealt out by position instead of through a contended counter ----
-  const uint32_t nwaves = gridDim.x * (uint32_t)kNW;
-  for (uint32_t t = blockIdx.x * (uint32_t)kNW + (uint32_t)wave; t < nwtasks; t += nwaves) {
-    const fw_batch_task* tp = h.wtasks + t;
-    const int32_t v = __builtin_amdgcn_readfirstlane(tp->v);
-    const uint32_t off = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->off);
-    const uint32_t deg = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->deg);
-    const uint32_t rec_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->rec_base);
-    const int count = __builtin_amdgcn_readfirstlane(tp->count);
-    const int32_t want = kApp == FW_APP_METAPATH ? s_schema[__builtin_amdgcn_readfirstlane(tp->slot)] : 0;
-
-    const bool have = lane < count;
-    fw_walker_rec rec;
-    rec.q = 0; rec.cur = v; rec.prev = -1; rec.len = 1;
-    if (have) rec = h.sorted[rec_base + (uint32_t)lane];
-    const uint32_t walker = a.walker_base + (uint32_t)rec.q;
-    const uint32_t step = (uint32_t)(rec.len - 1);
-
-    float S;
-    int32_t sel;
-    batch_stream<kApp>(a, bias, off, deg, want, 0u, 1u, have, walker, step, lane, S, sel);
-    batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, have, sel, walker, step, lane, n_steps, n_edges, n_out);
   }
 
   // counters: summed inside the workgroup first (the global ones are contended); the batch kernel's share of the

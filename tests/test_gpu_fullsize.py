@@ -1,4 +1,4 @@
-"""The configurations of BASELINE.json at their real sizes, checked through size-independent properties
+"""The benchmark configurations at their real sizes, checked through size-independent properties
 (the oracle would need minutes to hours at these sizes): start column, -1 suffix, every hop a CSR edge, workload
 counters recomputed from the paths, and byte-identical output under a different launch shape."""
 import numpy as np

@@ -40,7 +40,7 @@ def hub():
 
 
 def test_config1_deepwalk(gpu, c1_graph):
-    """BASELINE config 1: 7,115 vertices, 103,689 edges, 100 seeded starts, length 80."""
+    """Benchmark configuration 1: 7,115 vertices, 103,689 edges, 100 seeded starts, length 80."""
     starts = np.random.RandomState(1).randint(0, 7115, size=100).astype(np.int32)
     paths, st = _check(gpu, c1_graph, starts, app=gpu.APP_DEEPWALK, max_depth=81, seed=1)
     assert (paths[:, 0] == starts).all()

@@ -260,7 +260,7 @@ def test_metapath_follows_schema_and_is_uniform_among_matches(hub_csr):
 
 
 def test_config1_plumbing_on_the_cpu_path():
-    """BASELINE config 1 on the CPU reference path: 7,115 vertices, 103,689 edges, 100 seeded starts, length 80."""
+    """Benchmark configuration 1 on the CPU reference path: 7,115 vertices, 103,689 edges, 100 seeded starts, length 80."""
     xadj, adj, w, lab = _graphs.uniform_graph(7115, 103689, seed=1)
     assert len(xadj) == 7116 and len(adj) == 103689 and w.min() >= 1.0 and w.max() < 5.0
     g = orc.Graph(xadj, adj, w, lab)
