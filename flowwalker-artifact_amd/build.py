@@ -29,7 +29,8 @@ HIP_FLAGS = [
 ]
 
 KERNEL_SOURCES = ["fw_walk_kernel.hip", "fw_api.hip", "fw_gen.hip", "fw_csr_io.hip"]
-HOST_TOOLS = {"flowwalker": ["flowwalker_main.cpp"], "fw_gen": ["fw_gen_main.cpp"], "fw_convert": ["fw_convert_main.cpp"]}
+HOST_TOOLS = {"flowwalker": ["flowwalker_main.cpp"], "fw_gen": ["fw_gen_main.cpp"], "fw_convert": ["fw_convert_main.cpp"],
+              "fw_sampler_bench": ["fw_sampler_bench_main.cpp"]}
 
 
 def _run(cmd):

@@ -910,7 +910,11 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
   } while (0)
   if (use_pb) {
     rc = pb.alloc((size_t)n, g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1));
-    if (rc != FW_OK) { cleanup(); return rc; }
+    if (rc != FW_OK) {  // no room for the parking lists: walk without parking (same results, one launch)
+      pb.release();
+      use_pb = false;
+      (void)hipGetLastError();
+    }
   }
   FW_TRY(hipEventCreate(&ev0));
   FW_TRY(hipEventCreate(&ev1));
@@ -962,6 +966,13 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     if (rc != FW_OK) return rc;
     batch_size = fw_autobatch_size(free_b, 512, p->max_depth, sync, (uint32_t)n);
     if (batch_size == 0) { fw_set_error("autobatch: not enough free device memory"); return FW_ERR_NOMEM; }
+    if (resolve_park_threshold(g, p, (int32_t)batch_size) != INT_MAX) {
+      // the reference's rule counts the path matrix only; the parking lists take about 72 bytes per query more
+      const size_t per_query = 4u * ((size_t)p->max_depth + 1u) + 72u;
+      size_t bs2 = (free_b > ((size_t)512 << 20) ? free_b - ((size_t)512 << 20) : 0) / per_query;
+      if (!sync) bs2 /= 2;
+      if (bs2 >= 1 && bs2 < (size_t)batch_size) batch_size = (uint32_t)bs2;
+    }
   }
   if (batch_size > (uint32_t)n) batch_size = (uint32_t)n;
   const int nbuf = sync ? 1 : 2;
@@ -990,14 +1001,19 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     pbs[0].release();
     pbs[1].release();
   };
-  if (use_pb) {
-    for (int i = 0; i < nbuf; ++i) {
-      rc = pbs[i].alloc(bs, g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1));
-      if (rc != FW_OK) { cleanup(); return rc; }
-    }
-  }
   FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_starts), bs * nbuf * sizeof(int32_t)));
   FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_paths), bs * nbuf * md * sizeof(int32_t)));
+  if (use_pb) {
+    for (int i = 0; i < nbuf && use_pb; ++i) {
+      rc = pbs[i].alloc(bs, g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1));
+      if (rc != FW_OK) {  // no room for the parking lists: walk without parking (same results)
+        pbs[0].release();
+        pbs[1].release();
+        use_pb = false;
+        (void)hipGetLastError();
+      }
+    }
+  }
   const int nbatch = (int)(((size_t)n + bs - 1) / bs);
   FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_scr), sizeof(Scratch) * (size_t)nbatch));
   FW_TRY(hipMemset(d_scr, 0, sizeof(Scratch) * (size_t)nbatch));

@@ -81,3 +81,29 @@ def test_metapath_and_ppr(gpu, graph_files, tmp_path):
     assert (got == ref).all()
     _run("--input", prefix, "--ppr", "--n=300", "--seq", "--pprstart=seq", "--savepaths", out)
     assert (np.fromfile(out, dtype=np.int32).reshape(300, 81)[:, 0] == np.arange(300)).all()
+
+
+def test_sampler_micro_benchmark_and_converter(gpu, tmp_path):
+    """fw_sampler_bench (one sampling step at fixed list lengths, both granularities) runs and reports every sample;
+    a graph written by fw_convert loads and walks."""
+    tool = os.path.join(ROOT, "flowwalker-artifact_amd", "bin", "fw_sampler_bench")
+    r = subprocess.run([tool, "--elements", "1048576", "--samples", "20000", "--gran", "16,1024", "--reps", "1"],
+                       stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    rows = [ln.split() for ln in r.stdout.splitlines()[1:]]
+    assert [(row[0], row[1]) for row in rows] == [("16", "wave"), ("16", "workgroup"), ("1024", "wave"), ("1024", "workgroup")]
+    assert all(int(row[2]) == 20000 and float(row[3]) > 0 for row in rows)
+
+    conv = os.path.join(ROOT, "flowwalker-artifact_amd", "bin", "fw_convert")
+    rng = np.random.RandomState(11)
+    src = tmp_path / "edges.txt"
+    src.write_text("".join("%d %d\n" % (a, b) for a, b in rng.randint(0, 500, size=(6000, 2))))
+    prefix = str(tmp_path / "conv")
+    subprocess.run([conv, str(src), prefix, "5", "--sorted", "--seed", "3"], check=True, capture_output=True)
+    xadj, adj, w, lab = gpu.csr_read(prefix)
+    out = str(tmp_path / "p.bin")
+    _run("--input", prefix, "--node2vec", "--n=200", "--seq", "--d=10", "--seed=9", "--savepaths", out)
+    paths = np.fromfile(out, dtype=np.int32).reshape(200, 11)
+    ref, _, _ = orc.walk(orc.Graph(xadj, adj, w, lab), orc.make_params(app=2, max_depth=11, seed=9, p=2.0, q=0.5),
+                         np.arange(200, dtype=np.int32))
+    assert (paths == ref).all()
