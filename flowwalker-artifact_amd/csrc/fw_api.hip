@@ -892,7 +892,9 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
   if (park_threshold != INT_MAX) {
     rc = ensure_hub_index(const_cast<fw_graph*>(g), park_threshold);
     if (rc != FW_OK) return rc;
-    use_pb = g->n_hubs > 0;
+    // buckets = parked-on vertices x labels must stay a 30-bit count (bucket ids travel in 32-bit record fields)
+    use_pb = g->n_hubs > 0 &&
+             (int64_t)g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1) <= ((int64_t)1 << 30);
   }
   Scratch* d_scr = nullptr;
   FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_scr), sizeof(Scratch)));
@@ -984,7 +986,9 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
   if (park_threshold != INT_MAX) {
     rc = ensure_hub_index(const_cast<fw_graph*>(g), park_threshold);
     if (rc != FW_OK) return rc;
-    use_pb = g->n_hubs > 0;
+    // buckets = parked-on vertices x labels must stay a 30-bit count (bucket ids travel in 32-bit record fields)
+    use_pb = g->n_hubs > 0 &&
+             (int64_t)g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1) <= ((int64_t)1 << 30);
   }
   ParkBuffers pbs[2];
   int32_t* d_starts = nullptr;
