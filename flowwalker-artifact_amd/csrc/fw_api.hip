@@ -73,7 +73,7 @@ extern "C" void fw_walk_params_default(fw_walk_params* p) {
   p->sampler = FW_SAMPLER_ZPRS;
   p->max_depth = 81;
   p->wg_threads = 512;
-  p->hub_threshold = 4096;
+  p->hub_threshold = 16384;
   p->schema_len = 5;
   for (int i = 0; i < 5; ++i) p->schema[i] = i;
   p->tp = 0.2f;
@@ -213,6 +213,8 @@ static int alloc_edge_array(T** out, uint64_t E) {
   return FW_OK;
 }
 
+static void release_park_cache(fw_graph* g);  // defined with the parking buffers below
+
 extern "C" int fw_graph_destroy(fw_graph* g) {
   if (!g) return FW_OK;
   int rc = FW_OK;
@@ -222,6 +224,7 @@ extern "C" int fw_graph_destroy(fw_graph* g) {
       if (p && hipFree(p) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
     }
   }
+  release_park_cache(g);
   void* index_ptrs[2] = {g->hub_index, g->hub_info};
   for (void* p : index_ptrs) {
     if (p && hipFree(p) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
@@ -698,6 +701,34 @@ struct ParkBuffers {
   }
 };
 
+static void release_park_cache(fw_graph* g) {
+  ParkBuffers* c = static_cast<ParkBuffers*>(g->park_cache);
+  if (c) {
+    c->release();
+    delete c;
+  }
+  g->park_cache = nullptr;
+}
+
+// The parking lists for a call over n queries with n_buckets buckets: the graph keeps the last set (a call pays ten
+// allocations otherwise, which is a fifth of a 7 ms pass); it is replaced when it is too small or shaped differently.
+// NULL when the memory is not there (the caller then walks without parking).
+static ParkBuffers* cached_park_buffers(fw_graph* g, size_t n, int n_buckets) {
+  ParkBuffers* c = static_cast<ParkBuffers*>(g->park_cache);
+  if (c && c->cap >= n && c->n_buckets == n_buckets) return c;
+  release_park_cache(g);
+  c = new (std::nothrow) ParkBuffers;
+  if (!c) return nullptr;
+  if (c->alloc(n, n_buckets) != FW_OK) {
+    c->release();
+    delete c;
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  g->park_cache = c;
+  return c;
+}
+
 // Decides whether a call parks walkers, and at which degree.  Returns INT_MAX for "no".
 static int32_t resolve_park_threshold(const fw_graph* g, const fw_walk_params* p, int32_t n) {
   if (p->app == FW_APP_NODE2VEC) return INT_MAX;  // its biases depend on the walker: nothing to share
@@ -887,7 +918,7 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
   const double t0 = now_ms();
 
   const int32_t park_threshold = resolve_park_threshold(g, p, n);
-  ParkBuffers pb;
+  ParkBuffers* pb = nullptr;
   bool use_pb = false;
   if (park_threshold != INT_MAX) {
     rc = ensure_hub_index(const_cast<fw_graph*>(g), park_threshold);
@@ -896,6 +927,11 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
     use_pb = g->n_hubs > 0 &&
              (int64_t)g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1) <= ((int64_t)1 << 30);
   }
+  if (use_pb) {
+    pb = cached_park_buffers(const_cast<fw_graph*>(g), (size_t)n,
+                             g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1));
+    use_pb = pb != nullptr;  // no room for the parking lists: walk without parking (same results, one launch)
+  }
   Scratch* d_scr = nullptr;
   FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_scr), sizeof(Scratch)));
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -903,21 +939,12 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
     if (ev0) (void)hipEventDestroy(ev0);
     if (ev1) (void)hipEventDestroy(ev1);
     if (d_scr) (void)hipFree(d_scr);
-    pb.release();
   };
 #define FW_TRY(call)                                                 \
   do {                                                               \
     int rc_ = fw_check_hip((call), #call, __FILE__, __LINE__);       \
     if (rc_ != FW_OK) { cleanup(); return rc_; }                     \
   } while (0)
-  if (use_pb) {
-    rc = pb.alloc((size_t)n, g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1));
-    if (rc != FW_OK) {  // no room for the parking lists: walk without parking (same results, one launch)
-      pb.release();
-      use_pb = false;
-      (void)hipGetLastError();
-    }
-  }
   FW_TRY(hipEventCreate(&ev0));
   FW_TRY(hipEventCreate(&ev1));
   FW_TRY(hipMemsetAsync(d_scr, 0, sizeof(Scratch), stream));
@@ -934,7 +961,7 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
   int grid_used = 0, launches = 0;
   KernelTimes times;
   FW_TRY(hipEventRecord(ev0, stream));
-  rc = run_walk_launches(g, p, a, park_threshold, use_pb ? &pb : nullptr, stream, &grid_used, &launches, &times);
+  rc = run_walk_launches(g, p, a, park_threshold, use_pb ? pb : nullptr, stream, &grid_used, &launches, &times);
   if (rc != FW_OK) { cleanup(); return rc; }
   FW_TRY(hipEventRecord(ev1, stream));
   FW_TRY(hipStreamSynchronize(stream));

@@ -33,6 +33,7 @@ struct fw_graph {
   int32_t n_hubs = 0;
   int32_t* hub_index = nullptr;       // int32[V]: position in hub_info, -1 (not parked on) or -2 (degree 0)
   struct fw_hub_info* hub_info = nullptr;  // [n_hubs]
+  void* park_cache = nullptr;         // the parking lists of the last fw_walk_device call, kept for the next one
 };
 
 constexpr int FW_EDGE_PAD = 4;
