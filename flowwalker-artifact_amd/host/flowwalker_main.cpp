@@ -10,8 +10,8 @@
 // reference, on purpose: random start vertices come from --seed instead of time(NULL) (src/main.cu:284),
 // the first min(100, n) walkers are printed (the reference always prints 100 and reads out of bounds for
 // smaller n: src/main.cu:165), errors return a non-zero status with a message instead of exit() inside a
-// macro, and --walkmode / --umgraph / --lognorm / --save_degree / --b_file (ablation and debug switches)
-// are accepted and ignored with a note.
+// macro, --lognorm draws its weights from a seeded host generator, and --walkmode / --umgraph (ablation and
+// out-of-core switches) are accepted and ignored with a note.
 
 #include <stdint.h>
 #include <stdio.h>
@@ -21,6 +21,7 @@
 #include <algorithm>
 #include <chrono>
 #include <map>
+#include <random>
 #include <string>
 #include <vector>
 
@@ -194,9 +195,8 @@ int main(int argc, char** argv) {
          "------------------------------------\n");
   Flags F;
   if (!parse_flags(argc, argv, &F)) return 2;
-  for (const char* ignored : {"walkmode", "umgraph", "lognorm", "save_degree"}) {
-    const bool set = (!strcmp(ignored, "walkmode") && F.walkmode >= 0) || (!strcmp(ignored, "umgraph") && F.umgraph) ||
-                     (!strcmp(ignored, "lognorm") && F.lognorm) || (!strcmp(ignored, "save_degree") && F.save_degree);
+  for (const char* ignored : {"walkmode", "umgraph"}) {
+    const bool set = (!strcmp(ignored, "walkmode") && F.walkmode >= 0) || (!strcmp(ignored, "umgraph") && F.umgraph);
     if (set) fprintf(stderr, "flowwalker: --%s selects an ablation / debug mode that this build does not have; ignored\n", ignored);
   }
   if (!(F.deepwalk || F.ppr || F.node2vec || F.metapath)) {  // src/walk.cu:565-568
@@ -221,6 +221,13 @@ int main(int argc, char** argv) {
   if (fw_csr_load(F.input.c_str(), V, E, xadj.data(), adjncy.data(), F.metapath ? nullptr : weight.data(),
                   F.metapath ? label.data() : nullptr) != FW_OK)
     return fail("loading the graph");
+  if (F.lognorm && !F.metapath) {
+    // include/graph.cuh:79-91, :164-165: the weights of the file are replaced by log-normal(0, 3) draws (the
+    // reference draws them with cuRAND, seed 1234; here a seeded host generator: same law, other numbers)
+    std::mt19937_64 gen(1234ULL);
+    std::lognormal_distribution<float> dist(0.0f, 3.0f);
+    for (size_t i = 0; i < weight.size(); ++i) weight[i] = dist(gen);
+  }
   printf("Graph load (success): %d verts, %llu edges %g second(s)\n", V, (unsigned long long)E, now_s() - t_load);
   printf("Read Graph!\n");
   int32_t max_deg = 0, max_idx = 0;
@@ -332,6 +339,17 @@ int main(int argc, char** argv) {
            (double)st.sampled_edges / (sample_ms * 1e-3));
     printf("walk steps per s: %f (kernel only: %f)\n", (double)st.steps / (sample_ms * 1e-3),
            (double)st.steps / (st.kernel_ms * 1e-3));
+  }
+  if (F.save_degree) {  // src/main.cu:115-149, :373: how many steps left a vertex of each degree, "degree,count" per line
+    std::map<uint32_t, uint64_t> hist;
+    for (int i = 0; i < sample_size; ++i) {
+      const int32_t* row = paths + (size_t)i * (size_t)depth;
+      for (int j = 1; j < depth && row[j] != -1; ++j) ++hist[xadj[(size_t)row[j - 1] + 1] - xadj[(size_t)row[j - 1]]];
+    }
+    FILE* f = fopen(F.b_file.c_str(), "w");
+    if (!f) { fprintf(stderr, "flowwalker: cannot write %s\n", F.b_file.c_str()); return 4; }
+    for (const auto& kv : hist) fprintf(f, "%u,%llu\n", kv.first, (unsigned long long)kv.second);
+    fclose(f);
   }
   if (!F.savepaths.empty()) {
     FILE* f = fopen(F.savepaths.c_str(), "wb");

@@ -107,3 +107,32 @@ def test_sampler_micro_benchmark_and_converter(gpu, tmp_path):
     ref, _, _ = orc.walk(orc.Graph(xadj, adj, w, lab), orc.make_params(app=2, max_depth=11, seed=9, p=2.0, q=0.5),
                          np.arange(200, dtype=np.int32))
     assert (paths == ref).all()
+
+
+def test_save_degree_and_lognorm(gpu, graph_files, tmp_path):
+    """--save_degree writes how many steps left a vertex of each degree (src/main.cu:115-149); --lognorm replaces
+    the file's weights by log-normal(0, 3) draws (include/graph.cuh:79-91), so the walks change but stay walks."""
+    prefix, (xadj, adj, w, lab) = graph_files
+    out, hist = str(tmp_path / "p.bin"), str(tmp_path / "bucket.csv")
+    _run("--input", prefix, "--deepwalk", "--n=300", "--seq", "--d=12", "--seed=4", "--save_degree", "--b_file", hist,
+         "--savepaths", out)
+    paths = np.fromfile(out, dtype=np.int32).reshape(300, 13)
+    deg = np.diff(xadj.astype(np.int64))
+    want = {}
+    for row in paths:
+        for j in range(1, 13):
+            if row[j] < 0:
+                break
+            want[int(deg[row[j - 1]])] = want.get(int(deg[row[j - 1]]), 0) + 1
+    got = {int(a): int(b) for a, b in (ln.split(",") for ln in open(hist).read().split())}
+    assert got == want and list(got) == sorted(got)
+
+    out2 = str(tmp_path / "p2.bin")
+    _run("--input", prefix, "--deepwalk", "--n=300", "--seq", "--d=12", "--seed=4", "--lognorm", "--savepaths", out2)
+    p2 = np.fromfile(out2, dtype=np.int32).reshape(300, 13)
+    assert (p2[:, 0] == paths[:, 0]).all() and (p2 != paths).any()
+    for row in p2[:50]:                                    # every hop is an edge of the graph
+        for j in range(1, 13):
+            if row[j] < 0:
+                break
+            assert row[j] in adj[xadj[row[j - 1]]:xadj[row[j - 1] + 1]]
