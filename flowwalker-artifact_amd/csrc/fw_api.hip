@@ -497,68 +497,138 @@ constexpr uint32_t kParkTail = 32768;  // fewer walkers than this finish in one 
 constexpr double kParkMeet = 4.0;
 constexpr int32_t kMinDefaultPark = 64;
 constexpr int32_t kMinParkThreshold = 1;
+constexpr int kParkCtrs = 16;                    // counters of a parking round
+// Two-pass steps: buckets with more than kTwoPassWalkers walkers on lists of at least kTwoPassDegree elements
+constexpr uint32_t kTwoPassWalkers = 256;
+constexpr uint32_t kTwoPassDegree = 2048;
+constexpr uint64_t kMaxRows = (2ull << 30) / 520u;  // 2 GiB of rows at most
 
-// One task per 64 parked walkers of a bucket: a workgroup task when the bucket's vertex is sampled at workgroup
-// granularity (degree above hub_threshold), a wave task otherwise.  ctrs[3] / ctrs[5] = number of tasks (out).
+// Cuts the round's buckets into tasks.  A bucket with more than two_pass_walkers walkers on a list of at least
+// two_pass_degree elements is served in two passes (scan tasks of up to kScanRun groups that make the list's rows,
+// one table task per 64 walkers) when its rows still fit; every other bucket gets one batch task per 64 walkers:
+// a workgroup task when its vertex is sampled at workgroup granularity (degree above hub_threshold), a wave task
+// otherwise.  ctrs (out): [3] workgroup tasks, [5] wave tasks, [7] table tasks, [8] scan tasks, [9] rows handed out.
+constexpr uint32_t kScanRun = 16;
+
+struct TaskPlan {
+  int32_t hub_threshold;
+  uint32_t two_pass_walkers;  // 0xFFFFFFFF: never
+  uint32_t two_pass_degree;
+  uint32_t rows_cap;
+};
+
 __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* __restrict__ bucket_count,
                                        const uint32_t* __restrict__ bucket_offset, int n_buckets, int labels,
-                                       const fw_hub_info* __restrict__ hub_info, int32_t hub_threshold,
-                                       fw_batch_task* tasks, fw_batch_task* wtasks, uint32_t* ctrs) {
-  // task slots: one update of the (contended) global counters per workgroup and kind; inside the workgroup the
-  // slots are dealt out by a scan over the waves' totals
-  __shared__ uint32_t s_tot[2][16];
-  __shared__ uint32_t s_base[2];
+                                       const fw_hub_info* __restrict__ hub_info, const TaskPlan plan,
+                                       fw_batch_task* tasks, fw_batch_task* wtasks, fw_batch_task* ttasks,
+                                       fw_batch_task* stasks, uint32_t* ctrs) {
+  // slots and rows: one update of the (contended) global counters per workgroup and kind; inside the workgroup
+  // they are dealt out by a scan over the waves' totals
+  constexpr int kKinds = 4;  // workgroup, wave, table, scan
+  __shared__ uint32_t s_tot[kKinds][16];
+  __shared__ uint32_t s_base[kKinds];
+  const int ctr_of[kKinds] = {3, 5, 7, 8};
   const int stride = gridDim.x * blockDim.x;
   const int lane = (int)(threadIdx.x & 63u);
   const int wave = (int)(threadIdx.x >> 6);
   const int rounds = (n_buckets + stride - 1) / stride;  // every thread runs every round: scans and barriers
+
+  // exclusive position of x among the workgroup's threads, plus a base from the global counter `ctr`
+  auto place = [&](uint32_t x, int ctr) -> uint32_t {
+    uint32_t inc = x;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const uint32_t up = __shfl_up(inc, d);
+      if (lane >= d) inc += up;
+    }
+    if (lane == 63) s_tot[0][wave] = inc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      uint32_t total = 0u;
+      for (int w = 0; w < 16; ++w) {
+        const uint32_t v = s_tot[0][w];
+        s_tot[0][w] = total;
+        total += v;
+      }
+      s_base[0] = total != 0u ? atomicAdd(&ctrs[ctr], total) : 0u;
+    }
+    __syncthreads();
+    const uint32_t at = s_base[0] + s_tot[0][wave] + inc - x;
+    __syncthreads();  // s_tot / s_base are reused
+    return at;
+  };
+
   for (int r = 0; r < rounds; ++r) {
     const int b = r * stride + (int)(blockIdx.x * blockDim.x + threadIdx.x);
     const uint32_t c = b < n_buckets ? bucket_count[b] : 0u;
     fw_batch_task t;
-    t.v = 0; t.off = 0; t.deg = 0; t.slot = 0; t.rec_base = 0; t.count = 0;
-    t.pad[0] = t.pad[1] = 0;
-    bool wg = false;
+    t.v = 0; t.off = 0; t.deg = 0; t.slot = 0; t.rec_base = 0; t.count = 0; t.row = 0; t.pad = 0;
+    uint32_t ngroups = 0u;
     if (c != 0u) {
       const fw_hub_info hi = hub_info[b / labels];
       t.v = hi.v;
       t.off = hi.off;
       t.deg = hi.deg;
       t.slot = b % labels;
-      wg = (int32_t)t.deg > hub_threshold;
+      ngroups = ((((t.off & 3u) + t.deg + 3u) >> 2) + 255u) / 256u;
     }
+    // rows first: a bucket whose rows do not fit any more falls back to batch tasks
+    bool two_pass = c > plan.two_pass_walkers && t.deg >= plan.two_pass_degree;
+    if (plan.two_pass_walkers != 0xFFFFFFFFu) {  // the same for every thread
+      const uint32_t row = place(two_pass ? ngroups : 0u, 9);
+      two_pass = two_pass && row <= plan.rows_cap && ngroups <= plan.rows_cap - row;
+      t.row = row;
+    }
+    const bool wg = (int32_t)t.deg > plan.hub_threshold;
     const uint32_t nb = (c + 63u) >> 6;
-    const uint32_t xw = wg ? nb : 0u, xs = wg ? 0u : nb;
-    uint32_t iw = xw, is = xs;  // inclusive wave scans
+    uint32_t x[kKinds];
+    x[0] = !two_pass && wg ? nb : 0u;
+    x[1] = !two_pass && !wg ? nb : 0u;
+    x[2] = two_pass ? nb : 0u;
+    x[3] = two_pass ? (ngroups + kScanRun - 1u) / kScanRun : 0u;
+    uint32_t inc[kKinds];
+#pragma unroll
+    for (int k = 0; k < kKinds; ++k) inc[k] = x[k];
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
-      const uint32_t uw = __shfl_up(iw, d);
-      const uint32_t us = __shfl_up(is, d);
-      if (lane >= d) { iw += uw; is += us; }
+#pragma unroll
+      for (int k = 0; k < kKinds; ++k) {
+        const uint32_t up = __shfl_up(inc[k], d);
+        if (lane >= d) inc[k] += up;
+      }
     }
     if (lane == 63) {
-      s_tot[0][wave] = iw;
-      s_tot[1][wave] = is;
+#pragma unroll
+      for (int k = 0; k < kKinds; ++k) s_tot[k][wave] = inc[k];
     }
     __syncthreads();
-    if (threadIdx.x < 2) {
+    if (threadIdx.x < kKinds) {
       uint32_t total = 0u;
       for (int w = 0; w < 16; ++w) {  // exclusive prefix over the waves, in place
         const uint32_t v = s_tot[threadIdx.x][w];
         s_tot[threadIdx.x][w] = total;
         total += v;
       }
-      s_base[threadIdx.x] = total != 0u ? atomicAdd(&ctrs[threadIdx.x == 0 ? 3 : 5], total) : 0u;
+      s_base[threadIdx.x] = total != 0u ? atomicAdd(&ctrs[ctr_of[threadIdx.x]], total) : 0u;
     }
     __syncthreads();
     if (c != 0u) {
-      const uint32_t t0 = wg ? s_base[0] + s_tot[0][wave] + iw - xw : s_base[1] + s_tot[1][wave] + is - xs;
-      fw_batch_task* out = wg ? tasks : wtasks;
+      const int kind = two_pass ? 2 : (wg ? 0 : 1);
+      const uint32_t t0 = s_base[kind] + s_tot[kind][wave] + inc[kind] - x[kind];
+      fw_batch_task* out = kind == 0 ? tasks : (kind == 1 ? wtasks : ttasks);
       const uint32_t base = bucket_offset[b];
       for (uint32_t k = 0; k < nb; ++k) {
         t.rec_base = base + 64u * k;
         t.count = (int32_t)(c - 64u * k < 64u ? c - 64u * k : 64u);
         out[t0 + k] = t;
+      }
+      if (two_pass) {
+        const uint32_t s0 = s_base[3] + s_tot[3][wave] + inc[3] - x[3];
+        for (uint32_t k = 0; k < x[3]; ++k) {
+          t.rec_base = k * kScanRun;
+          t.count = (int32_t)((k + 1u) * kScanRun < ngroups ? (k + 1u) * kScanRun : ngroups);
+          stasks[s0 + k] = t;
+        }
       }
     }
     __syncthreads();  // s_tot / s_base are reused by the next round
@@ -586,10 +656,15 @@ __global__ void fw_scatter_counted_kernel(const fw_walker_rec* __restrict__ src,
                                           const uint32_t* __restrict__ bucket_offset, uint32_t* bucket_fill,
                                           fw_walker_rec* __restrict__ sorted) {
   const uint32_t stride = gridDim.x * blockDim.x;
-  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < m; i += stride) {
-    const fw_walker_rec r = src[i];
+  for (uint32_t i0 = blockIdx.x * blockDim.x; i0 < m; i0 += stride) {  // uniform in the wave: the ranks are taken together
+    const uint32_t i = i0 + threadIdx.x;
+    const bool have = i < m;
+    fw_walker_rec r;
+    r.q = 0; r.cur = 0; r.prev = 0; r.len = 0;
+    if (have) r = src[i];
     const uint32_t b = (uint32_t)r.cur;
-    sorted[bucket_offset[b] + bucket_count[b] - 1u - atomicAdd(&bucket_fill[b], 1u)] = r;
+    const uint32_t rank = fw_wave_count_keys<true>(bucket_fill, b, have);
+    if (have) sorted[bucket_offset[b] + bucket_count[b] - 1u - rank] = r;
   }
 }
 
@@ -663,7 +738,14 @@ struct ParkBuffers {
   fw_batch_task* tasks = nullptr;
   fw_batch_task* wtasks = nullptr;
   uint32_t* ctrs = nullptr;           // [0] walkers in `walked`, [1] records of `out` that resume, [2] that are parked
-                                      // again, [3] workgroup tasks, [4] their dispenser, [5] wave tasks, [6] records in `resume`
+                                      // again, [3] workgroup tasks, [4] their dispenser, [5] wave tasks, [6] records in
+                                      // `resume`, [7] table tasks, [8] scan tasks, [9] rows handed out
+  fw_batch_task* ttasks = nullptr;    // two-pass steps: table tasks, scan tasks and the rows between them
+  fw_batch_task* stasks = nullptr;
+  float* totals = nullptr;
+  float* rows = nullptr;
+  int32_t* lastpos = nullptr;
+  uint32_t rows_cap = 0;              // rows allocated (0: no two-pass steps)
   uint32_t* h_ctrs = nullptr;         // pinned mirror
   void* tmp = nullptr;                // scan temporary storage
   size_t scan_bytes = 0;
@@ -672,7 +754,7 @@ struct ParkBuffers {
   uint32_t* offset() const { return buckets + (size_t)2 * n_buckets; }
   uint32_t* fill() const { return buckets + (size_t)3 * n_buckets; }
 
-  int alloc(size_t walkers, int n) {
+  int alloc(size_t walkers, int n, uint64_t rows_wanted) {
     cap = walkers;
     n_buckets = n;
     const size_t ntask = cap / 64 + (size_t)n + 1;
@@ -683,14 +765,40 @@ struct ParkBuffers {
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&buckets), (size_t)4 * n * sizeof(uint32_t)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&tasks), ntask * sizeof(fw_batch_task)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&wtasks), ntask * sizeof(fw_batch_task)));
-    FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), 8 * sizeof(uint32_t)));
-    FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), 8 * sizeof(uint32_t), hipHostMallocDefault));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), kParkCtrs * sizeof(uint32_t)));
+    FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), kParkCtrs * sizeof(uint32_t), hipHostMallocDefault));
+    // the rows are an extra: without room for them every bucket is served by batch tasks
+    if (rows_wanted > kMaxRows) rows_wanted = kMaxRows;
+    if (rows_wanted != 0u) {
+      // scan tasks: a list of G groups is cut into at most G / kScanRun + 1 runs, and no more lists are scanned in
+      // a round than there are buckets or walkers
+      const size_t nscan = (size_t)(rows_wanted / kScanRun) + ((size_t)n < cap ? (size_t)n : cap) + 1;
+      if (hipMalloc(reinterpret_cast<void**>(&ttasks), ntask * sizeof(fw_batch_task)) == hipSuccess &&
+          hipMalloc(reinterpret_cast<void**>(&stasks), nscan * sizeof(fw_batch_task)) == hipSuccess &&
+          hipMalloc(reinterpret_cast<void**>(&totals), (size_t)rows_wanted * sizeof(float)) == hipSuccess &&
+          hipMalloc(reinterpret_cast<void**>(&lastpos), (size_t)rows_wanted * sizeof(int32_t)) == hipSuccess &&
+          hipMalloc(reinterpret_cast<void**>(&rows), (size_t)rows_wanted * 128 * sizeof(float)) == hipSuccess) {
+        rows_cap = (uint32_t)rows_wanted;
+      } else {
+        (void)hipGetLastError();
+        release_rows();
+      }
+    }
     FW_HIP(rocprim::exclusive_scan(nullptr, scan_bytes, count(0), offset(), 0u, (size_t)n,
                                    rocprim::plus<uint32_t>(), (hipStream_t)0));
     FW_HIP(hipMalloc(&tmp, scan_bytes ? scan_bytes : 16));
     return FW_OK;
   }
+  void release_rows() {
+    void* dev[5] = {ttasks, stasks, totals, lastpos, rows};
+    for (void* p : dev) if (p) (void)hipFree(p);
+    ttasks = stasks = nullptr;
+    totals = rows = nullptr;
+    lastpos = nullptr;
+    rows_cap = 0;
+  }
   void release() {
+    release_rows();
     void* dev[9] = {walked, sorted, out, resume, buckets, tasks, wtasks, ctrs, tmp};
     for (void* p : dev) if (p) (void)hipFree(p);
     if (h_ctrs) (void)hipHostFree(h_ctrs);
@@ -713,13 +821,13 @@ static void release_park_cache(fw_graph* g) {
 // The parking lists for a call over n queries with n_buckets buckets: the graph keeps the last set (a call pays ten
 // allocations otherwise, which is a fifth of a 7 ms pass); it is replaced when it is too small or shaped differently.
 // NULL when the memory is not there (the caller then walks without parking).
-static ParkBuffers* cached_park_buffers(fw_graph* g, size_t n, int n_buckets) {
+static ParkBuffers* cached_park_buffers(fw_graph* g, size_t n, int n_buckets, uint64_t rows_wanted) {
   ParkBuffers* c = static_cast<ParkBuffers*>(g->park_cache);
   if (c && c->cap >= n && c->n_buckets == n_buckets) return c;
   release_park_cache(g);
   c = new (std::nothrow) ParkBuffers;
   if (!c) return nullptr;
-  if (c->alloc(n, n_buckets) != FW_OK) {
+  if (c->alloc(n, n_buckets, rows_wanted) != FW_OK) {
     c->release();
     delete c;
     (void)hipGetLastError();
@@ -727,6 +835,17 @@ static ParkBuffers* cached_park_buffers(fw_graph* g, size_t n, int n_buckets) {
   }
   g->park_cache = c;
   return c;
+}
+
+// Rows to set aside for two-pass steps.  A list of d elements has at most d / 1024 + 2 groups, so all lists of
+// kTwoPassDegree elements or more together have at most E / 512 per label a walker can want; a quarter of that is
+// set aside, because only the lists that are crowded in the same round need rows at the same time, and a bucket
+// whose rows do not fit is served by batches like any other.
+static uint64_t two_pass_rows(const fw_graph* g, int labels) {
+  int32_t max_degree = 0;
+  if (fw_graph_info(g, nullptr, nullptr, &max_degree, nullptr) != FW_OK) return 0;
+  if ((uint32_t)max_degree < kTwoPassDegree) return 0;
+  return (uint64_t)labels * (g->E / 2048u + 1024u);
 }
 
 // Decides whether a call parks walkers, and at which degree.  Returns INT_MAX for "no".
@@ -792,6 +911,18 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   h.nwtasks = &pb->ctrs[5];
   h.out = pb->out;
   h.out_counts = &pb->ctrs[1];
+  h.stasks = pb->stasks;
+  h.nstasks = &pb->ctrs[8];
+  h.ttasks = pb->ttasks;
+  h.nttasks = &pb->ctrs[7];
+  h.totals = pb->totals;
+  h.rows = pb->rows;
+  h.lastpos = pb->lastpos;
+  TaskPlan plan;
+  plan.hub_threshold = p->hub_threshold;
+  plan.two_pass_walkers = pb->rows_cap != 0u ? kTwoPassWalkers : 0xFFFFFFFFu;
+  plan.two_pass_degree = kTwoPassDegree;
+  plan.rows_cap = pb->rows_cap;
 
   // One walk launch and the read-back of the counters.
   auto walk = [&](int* grid_out) -> int {
@@ -804,7 +935,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     if (rc != FW_OK) return rc;
     if ((rc = tw.end(stream)) != FW_OK) return rc;
     ++*launches;
-    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, 8 * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, kParkCtrs * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     FW_HIP(hipStreamSynchronize(stream));
     tw.collect(&times->walk_ms);
     return FW_OK;
@@ -812,7 +943,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
 
   // first walk launch: fresh queries; the walkers it parks are counted in bucket array 0
   int cur = 0;
-  FW_HIP(hipMemsetAsync(pb->ctrs, 0, 8 * sizeof(uint32_t), stream));
+  FW_HIP(hipMemsetAsync(pb->ctrs, 0, kParkCtrs * sizeof(uint32_t), stream));
   FW_HIP(hipMemsetAsync(pb->count(0), 0, bucket_bytes, stream));
   a.resume = nullptr;
   a.bucket_count = pb->count(0);
@@ -853,17 +984,21 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
       a.park_threshold = INT_MAX;
       return walk(nullptr);
     }
-    FW_HIP(hipMemsetAsync(pb->ctrs + 1, 0, 7 * sizeof(uint32_t), stream));
+    FW_HIP(hipMemsetAsync(pb->ctrs + 1, 0, (kParkCtrs - 1) * sizeof(uint32_t), stream));
     FW_HIP(hipMemsetAsync(pb->count(nxt), 0, bucket_bytes, stream));
     unsigned tblocks = ((unsigned)pb->n_buckets + 1023u) / 1024u;
     if (tblocks > 1024u) tblocks = 1024u;
     hipLaunchKernelGGL(fw_bucket_tasks_kernel, dim3(tblocks), dim3(1024), 0, stream, pb->count(cur), pb->offset(),
-                       pb->n_buckets, labels, g->hub_info, p->hub_threshold, pb->tasks, pb->wtasks,
+                       pb->n_buckets, labels, g->hub_info, plan, pb->tasks, pb->wtasks, pb->ttasks, pb->stasks,
                        pb->ctrs);
     FW_HIP(hipGetLastError());
     h.bucket_out = pb->count(nxt);
     TimedLaunch th;
     if ((rc = th.begin(stream)) != FW_OK) return rc;
+    if (plan.two_pass_walkers != 0xFFFFFFFFu) {
+      rc = fw_launch_hub_scan(a, h, p->app, stream);  // finds its task count on the device; often none
+      if (rc != FW_OK) return rc;
+    }
     rc = fw_launch_hub_batch(a, h, p->app, p->wg_threads, stream);
     if (rc != FW_OK) return rc;
     if ((rc = th.end(stream)) != FW_OK) return rc;
@@ -875,12 +1010,13 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
                          pb->resume, pb->ctrs + 6);
       FW_HIP(hipGetLastError());
     }
-    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, 8 * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, kParkCtrs * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     FW_HIP(hipStreamSynchronize(stream));
     th.collect(&times->hub_ms);
     if (getenv("FW_DEBUG_ROUNDS"))
-      fprintf(stderr, "round: parked %llu (walk %u + again %u) wg_tasks %u wave_tasks %u -> resume %u again %u\n",
-              (unsigned long long)m, n_walked, n_again, pb->h_ctrs[3], pb->h_ctrs[5], pb->h_ctrs[1], pb->h_ctrs[2]);
+      fprintf(stderr, "round: parked %llu (walk %u + again %u) wg_tasks %u wave_tasks %u table_tasks %u scan_tasks %u rows %u -> resume %u again %u\n",
+              (unsigned long long)m, n_walked, n_again, pb->h_ctrs[3], pb->h_ctrs[5], pb->h_ctrs[7], pb->h_ctrs[8],
+              pb->h_ctrs[9], pb->h_ctrs[1], pb->h_ctrs[2]);
     n_out = (uint32_t)m;
     pb->h_ctrs[0] = 0u;
     if (pb->h_ctrs[6] != 0u) {
@@ -928,8 +1064,8 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
              (int64_t)g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1) <= ((int64_t)1 << 30);
   }
   if (use_pb) {
-    pb = cached_park_buffers(const_cast<fw_graph*>(g), (size_t)n,
-                             g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1));
+    const int labels = p->app == FW_APP_METAPATH ? p->schema_len : 1;
+    pb = cached_park_buffers(const_cast<fw_graph*>(g), (size_t)n, g->n_hubs * labels, two_pass_rows(g, labels));
     use_pb = pb != nullptr;  // no room for the parking lists: walk without parking (same results, one launch)
   }
   Scratch* d_scr = nullptr;
@@ -1036,7 +1172,8 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
   FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_paths), bs * nbuf * md * sizeof(int32_t)));
   if (use_pb) {
     for (int i = 0; i < nbuf && use_pb; ++i) {
-      rc = pbs[i].alloc(bs, g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1));
+      rc = pbs[i].alloc(bs, g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1),
+                        two_pass_rows(g, p->app == FW_APP_METAPATH ? p->schema_len : 1));
       if (rc != FW_OK) {  // no room for the parking lists: walk without parking (same results)
         pbs[0].release();
         pbs[1].release();

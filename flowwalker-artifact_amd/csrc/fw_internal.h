@@ -87,7 +87,8 @@ struct fw_batch_task {
   uint32_t rec_base;
   int32_t count;
   int32_t slot;       // metapath: position in the schema of the label these walkers want
-  int32_t pad[2];
+  uint32_t row;       // two-pass steps: first row of the list's groups
+  int32_t pad;
 };
 
 // Arguments of the hub batch kernel: up to 64 walkers parked on one vertex are served with one scan of its list,
@@ -105,7 +106,57 @@ struct fw_hub_args {
   fw_walker_rec* out;
   uint32_t* bucket_out;
   uint32_t* out_counts;              // [0] += records that resume, [1] += records parked again
+  // Two-pass steps of crowded hubs.  The scan launch works through stasks (rec_base = first group of the run,
+  // count = one past its last, row = the list's first row) and fills, per group of a list, totals[row],
+  // rows[row * 128 ..] (64 running maxima, 64 prefixes) and lastpos[row]; the batch launch then serves ttasks
+  // (a batch task plus row = the list's first row) from them.
+  const fw_batch_task* stasks;
+  const uint32_t* nstasks;
+  const fw_batch_task* ttasks;
+  const uint32_t* nttasks;
+  float* totals;
+  float* rows;
+  int32_t* lastpos;
 };
+
+#ifdef __HIPCC__
+// counter[key] += 1 for every lane with pred; returns the value the lane's own increment found (its rank among the
+// increments of that counter).  When several lanes of the wave share the first active lane's key (then the first
+// remaining lane's), they are served by one atomic of their count: a wave whose walkers mostly move to one vertex
+// would otherwise update that vertex's counter 64 times in a row, and updates of one address cost about 13 ns
+// each wherever they come from.  Call from wave-uniform control flow.
+template <bool kReturn>
+__device__ __forceinline__ uint32_t fw_wave_count_keys(uint32_t* counter, uint32_t key, bool pred) {
+  const int lane = (int)__lane_id();
+  uint32_t rank = 0u;
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const uint64_t m = __ballot(pred);
+    if (m == 0ull) break;
+    const int leader = __builtin_ctzll(m);
+    const uint32_t k = (uint32_t)__builtin_amdgcn_readlane((int)key, leader);
+    const bool same = pred && key == k;
+    const uint64_t ms = __ballot(same);
+    const uint32_t cnt = (uint32_t)__builtin_popcountll(ms);
+    if (cnt < 4u) break;
+    uint32_t old = 0u;
+    if (lane == leader) {
+      if (kReturn) old = atomicAdd(&counter[k], cnt);
+      else atomicAdd(&counter[k], cnt);
+    }
+    if (kReturn) {
+      old = (uint32_t)__builtin_amdgcn_readlane((int)old, leader);
+      if (same) rank = old + (uint32_t)__builtin_popcountll(ms & ((1ull << lane) - 1ull));
+    }
+    pred = pred && !same;
+  }
+  if (pred) {
+    if (kReturn) rank = atomicAdd(&counter[key], 1u);
+    else atomicAdd(&counter[key], 1u);
+  }
+  return rank;
+}
+#endif
 
 void fw_set_error(const char* fmt, ...);
 int fw_check_hip(hipError_t e, const char* what, const char* file, int line);
@@ -122,3 +173,5 @@ int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int 
 
 // Launches the hub batch kernel (persistent grid, tasks taken from h.task_next).
 int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, hipStream_t stream);
+// Launches the scan kernel of the two-pass steps (it finds its task count in h.nstasks on the device).
+int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, hipStream_t stream);

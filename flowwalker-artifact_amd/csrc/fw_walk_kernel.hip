@@ -1042,21 +1042,20 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
           const int pleader = __builtin_ctzll(pm);
           if (lane == pleader) pbase = atomicAdd(a.parked_count, (uint32_t)__builtin_popcountll(pm));
           pbase = (uint32_t)__builtin_amdgcn_readlane((int)pbase, pleader);
+          const uint32_t label_slot =
+              kApp == FW_APP_METAPATH ? (uint32_t)(len - 1) % (uint32_t)a.n_labels_per_hub : 0u;
+          const uint32_t bucket = (uint32_t)hidx * (uint32_t)a.n_labels_per_hub + label_slot;
+          // counted only: the wave does not wait for a position inside the bucket (the counters of the busiest
+          // vertices are contended); the counting sort hands the positions out later
+          fw_wave_count_keys<false>(a.bucket_count, bucket, park);
           if (park) {
             const uint32_t at = pbase + (uint32_t)__builtin_popcountll(pm & ((1ull << lane) - 1ull));
-            const int32_t v = tt.cur[tid];
-            const uint32_t label_slot =
-                kApp == FW_APP_METAPATH ? (uint32_t)(len - 1) % (uint32_t)a.n_labels_per_hub : 0u;
-            const uint32_t bucket = (uint32_t)hidx * (uint32_t)a.n_labels_per_hub + label_slot;
             fw_walker_rec rec;
             rec.q = tt.walker[tid];
             rec.cur = (int32_t)bucket;  // the vertex follows from the bucket
             rec.prev = tt.prev[tid];
             rec.len = len;
             a.parked[at] = rec;
-            // counted only: the wave does not wait for a position inside the bucket (the counters of the busiest
-            // vertices are contended); the counting sort hands the positions out later
-            atomicAdd(&a.bucket_count[bucket], 1u);
             park = false;
             need = true;
             len = -1;
@@ -1310,6 +1309,234 @@ __device__ __forceinline__ void batch_stream(const fw_kargs& a, const uint32_t* 
   sel_out = sel;
 }
 
+// ---- Two-pass steps for crowded hubs ----------------------------------------------------------------------------------
+// A hub with many parked walkers is scanned once per 64 of them by the batches above.  Nothing in a group's part
+// of the sampler depends on the walker except two uniforms, so the walker-independent part can be made once per
+// hub and round: for every group its total T, the running maximum M of its positive lanes' prefixes, every
+// lane's prefix before its own 16 biases (E), and its last positive lane.  A walker then runs its reservoir over
+// the totals alone (same additions, same tests, same draws in the same order) and resolves its final target
+// inside one group from M, E and the 16 biases of one lane.  Same vertex as from the full stream, bit for bit.
+
+// The 16 biases of this lane in group g of a list (elements outside the list read as 0).
+template <int kApp>
+__device__ __forceinline__ void group_load(const uint32_t* __restrict__ bias, const uint32_t off, const uint32_t deg,
+                                           const int32_t want, const uint32_t g, const int lane, float* x) {
+  constexpr uint32_t kG = 64u * kGroupQuartets;
+  const uint32_t a0 = off & ~3u;
+  const uint32_t nq = (off + deg - a0 + 3u) >> 2;
+  const uint32_t kb = g * kG + (uint32_t)lane;
+  const bool interior = g > 0u && (g + 1u) * kG < nq;
+  uint4 raw[kGroupQuartets];
+  if (interior) {
+#pragma unroll
+    for (int j = 0; j < kGroupQuartets; ++j)
+      raw[j] = *reinterpret_cast<const uint4*>(bias + a0 + 4u * (kb + 64u * (uint32_t)j));
+  } else {
+#pragma unroll
+    for (int j = 0; j < kGroupQuartets; ++j) {
+      const uint32_t k = kb + 64u * (uint32_t)j;
+      raw[j] = make_uint4(0, 0, 0, 0);
+      if (k < nq) raw[j] = *reinterpret_cast<const uint4*>(bias + a0 + 4u * k);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kGroupQuartets; ++j) {
+    if (kApp == FW_APP_METAPATH) {
+      x[4 * j + 0] = (int32_t)raw[j].x == want ? 1.0f : 0.0f;
+      x[4 * j + 1] = (int32_t)raw[j].y == want ? 1.0f : 0.0f;
+      x[4 * j + 2] = (int32_t)raw[j].z == want ? 1.0f : 0.0f;
+      x[4 * j + 3] = (int32_t)raw[j].w == want ? 1.0f : 0.0f;
+    } else {
+      x[4 * j + 0] = __uint_as_float(raw[j].x);
+      x[4 * j + 1] = __uint_as_float(raw[j].y);
+      x[4 * j + 2] = __uint_as_float(raw[j].z);
+      x[4 * j + 3] = __uint_as_float(raw[j].w);
+    }
+  }
+  if (!interior) {
+#pragma unroll
+    for (int j = 0; j < kGroupQuartets; ++j) {
+      const uint32_t li = a0 + 4u * (kb + 64u * (uint32_t)j) - off;  // wraps below 0 for the head quartet
+      x[4 * j + 0] = li < deg ? x[4 * j + 0] : 0.0f;
+      x[4 * j + 1] = li + 1u < deg ? x[4 * j + 1] : 0.0f;
+      x[4 * j + 2] = li + 2u < deg ? x[4 * j + 2] : 0.0f;
+      x[4 * j + 3] = li + 3u < deg ? x[4 * j + 3] : 0.0f;
+    }
+  }
+}
+
+// First pass, one wave, one group: rows[0..63] = M, rows[64..127] = E, *total = T, *lastpos = last positive lane.
+template <int kApp>
+__device__ __forceinline__ void group_rows(const uint32_t* __restrict__ bias, const uint32_t off, const uint32_t deg,
+                                           const int32_t want, const uint32_t g, const int lane, float* rows,
+                                           float* total, int32_t* lastpos) {
+  constexpr int kEl = 4 * kGroupQuartets;
+  float x[kEl];
+  group_load<kApp>(bias, off, deg, want, g, lane, x);
+  float q = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kEl; ++i) q = q + x[i];
+  const float I = wave_scan(q);
+  const float T = readlane_f(I, 63);
+  const bool pos = q > 0.0f;
+  const uint64_t mpos = __ballot(pos);
+  const float M = wave_prefix_max(pos ? I : 0.0f);
+  rows[lane] = M;
+  rows[64 + lane] = I - q;
+  if (lane == 0) {
+    *total = T;
+    *lastpos = 63 - __builtin_clzll(mpos | 1ull);
+  }
+}
+
+// Second half of a two-pass step: lane and element of a walker's target `t` inside group `g` of the list, from the
+// rows group_rows left behind and the 16 biases of the lane that holds the target -- the same arithmetic on the
+// same values as batch_stream's search and pick.  Every lane works for its own walker (no cross-lane operations).
+// Returns the local index of the selected neighbour.
+template <int kApp>
+__device__ __forceinline__ int32_t resolve_pick(const uint32_t* __restrict__ bias, const uint32_t off, const uint32_t deg,
+                                                const int32_t want, const float* rows, const int32_t* lastpos,
+                                                const int32_t g, const float t) {
+  constexpr int kEl = 4 * kGroupQuartets;
+  const uint32_t a0 = off & ~3u;
+  const uint32_t nq = (off + deg - a0 + 3u) >> 2;
+  const float* M = rows + (size_t)(uint32_t)g * 128u;
+  // M never decreases: three pivots name the quarter of the lanes, its 16 entries the lane
+  const float p15 = M[15], p31 = M[31], p47 = M[47];
+  const int quarter = p15 > t ? 0 : (p31 > t ? 1 : (p47 > t ? 2 : 3));
+  const float4* Mq = reinterpret_cast<const float4*>(M + 16 * quarter);
+  const float4 m0 = Mq[0], m1 = Mq[1], m2 = Mq[2], m3 = Mq[3];
+  const float m[16] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w, m2.x, m2.y, m2.z, m2.w, m3.x, m3.y, m3.z, m3.w};
+  int below = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) below += m[i] <= t ? 1 : 0;
+  // first lane whose running maximum exceeds the target; none (rounding in the scan tree): the last positive lane
+  const int src = below < 16 ? 16 * quarter + below : lastpos[g];
+  float e = M[64 + src];
+  const uint32_t kb = (uint32_t)g * (64u * kGroupQuartets) + (uint32_t)src;
+  uint4 raw[kGroupQuartets];
+#pragma unroll
+  for (int j = 0; j < kGroupQuartets; ++j) {
+    const uint32_t k = kb + 64u * (uint32_t)j;
+    raw[j] = make_uint4(0, 0, 0, 0);
+    if (k < nq) raw[j] = *reinterpret_cast<const uint4*>(bias + a0 + 4u * k);
+  }
+  float x[kEl];
+#pragma unroll
+  for (int j = 0; j < kGroupQuartets; ++j) {
+    if (kApp == FW_APP_METAPATH) {
+      x[4 * j + 0] = (int32_t)raw[j].x == want ? 1.0f : 0.0f;
+      x[4 * j + 1] = (int32_t)raw[j].y == want ? 1.0f : 0.0f;
+      x[4 * j + 2] = (int32_t)raw[j].z == want ? 1.0f : 0.0f;
+      x[4 * j + 3] = (int32_t)raw[j].w == want ? 1.0f : 0.0f;
+    } else {
+      x[4 * j + 0] = __uint_as_float(raw[j].x);
+      x[4 * j + 1] = __uint_as_float(raw[j].y);
+      x[4 * j + 2] = __uint_as_float(raw[j].z);
+      x[4 * j + 3] = __uint_as_float(raw[j].w);
+    }
+    const uint32_t li = a0 + 4u * (kb + 64u * (uint32_t)j) - off;  // wraps below 0 for the head quartet
+    x[4 * j + 0] = li < deg ? x[4 * j + 0] : 0.0f;
+    x[4 * j + 1] = li + 1u < deg ? x[4 * j + 1] : 0.0f;
+    x[4 * j + 2] = li + 2u < deg ? x[4 * j + 2] : 0.0f;
+    x[4 * j + 3] = li + 3u < deg ? x[4 * j + 3] : 0.0f;
+  }
+  uint32_t cnt = 0u, pm = 0u;
+#pragma unroll
+  for (int i = 0; i < kEl; ++i) {
+    e = e + x[i];
+    cnt += e <= t ? 1u : 0u;
+    pm |= (x[i] > 0.0f ? 1u : 0u) << i;
+  }
+  const uint32_t cand = pm >> cnt;
+  const int pick = cand != 0u ? (int)cnt + __builtin_ctz(cand) : 31 - __builtin_clz(pm | 1u);
+  const uint32_t abs_idx = a0 + 4u * kb + 256u * (uint32_t)(pick >> 2) + (uint32_t)(pick & 3);
+  return (int32_t)(abs_idx - off);
+}
+
+// A walker's reservoir over the totals of sequence `seq` of a list (groups seq, seq + nw, ...): the group it ends
+// up in (-1: none) and its target there.  Totals past the end read as 0, which changes nothing: S stays, and a
+// test that failed on S fails again.
+__device__ __forceinline__ void table_reservoir(const fw_kargs& a, const float* totals, const uint32_t ngroups,
+                                                const uint32_t seq, const uint32_t nw, const uint32_t walker,
+                                                const uint32_t step, int32_t& gsel, float& tsel) {
+  float S = 0.0f, Sj = 0.0f, u = 1.0f;
+  LaneDraw dq;
+  gsel = -1;
+  tsel = 0.0f;
+  for (uint32_t g0 = seq; g0 < ngroups; g0 += 4u * nw) {
+    float t4[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t g = g0 + (uint32_t)j * nw;
+      t4[j] = g < ngroups ? totals[g] : 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float Snew = S + t4[j];
+      if (Snew * u > Sj) {
+        tsel = next_uniform_lane(dq, a, walker, step, seq) * t4[j];
+        gsel = (int32_t)(g0 + (uint32_t)j * nw);
+        Sj = Snew;
+        u = next_uniform_lane(dq, a, walker, step, seq);
+      }
+      S = Snew;
+    }
+  }
+}
+
+// A step of up to 64 walkers (lane i = walker i) on a hub whose rows are made: returns each walker's local index
+// (or -1).  wg: the list is sampled at workgroup granularity (kNW sequences combined by inverse transform).
+template <int kApp, int kNW>
+__device__ __forceinline__ int32_t table_sample(const fw_kargs& a, const uint32_t* __restrict__ bias, const uint32_t off,
+                                                const uint32_t deg, const int32_t want, const bool wg, const bool have,
+                                                const uint32_t walker, const uint32_t step, const int lane,
+                                                const float* totals, const float* rows, const int32_t* lastpos) {
+  constexpr uint32_t kG = 64u * kGroupQuartets;
+  const uint32_t nq = (off + deg - (off & ~3u) + 3u) >> 2;
+  const uint32_t ngroups = (nq + kG - 1u) / kG;
+  const uint32_t nw = wg ? (uint32_t)kNW : 1u;
+  int wsel = 0;
+  if (wg) {
+    // the sequences' totals, each added up in its own order by one lane, then the inverse transform over them
+    float Wl = 0.0f;
+    if ((uint32_t)lane < nw) {
+      for (uint32_t g0 = (uint32_t)lane; g0 < ngroups; g0 += 8u * nw) {
+        float t8[8];  // eight loads in flight, added in order; + 0 past the end changes nothing
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t g = g0 + (uint32_t)j * nw;
+          t8[j] = g < ngroups ? totals[g] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) Wl = Wl + t8[j];
+      }
+    }
+    const float J = row_scan(Wl);
+    const float total = readlane_f(J, kNW - 1);
+    const float target = u24(philox4x32_10(walker, step, kStreamWave, 0u, a.seed_lo, a.seed_hi).x) * total;
+    int wlast = -1;
+    wsel = -1;
+#pragma unroll
+    for (int w = 0; w < kNW; ++w) {
+      const float Ww = readlane_f(Wl, w);
+      const float Jw = readlane_f(J, w);
+      if (Ww > 0.0f) {
+        wsel = (wsel < 0 && Jw > target) ? w : wsel;
+        wlast = w;
+      }
+    }
+    wsel = wsel < 0 ? wlast : wsel;
+  }
+  // only the sequence the walker ends up in needs running: the draws of a sequence are addressed by the sequence
+  int32_t gsel = -1;
+  float tsel = 0.0f;
+  if (have && wsel >= 0) table_reservoir(a, totals, ngroups, (uint32_t)wsel, nw, walker, step, gsel, tsel);
+  int32_t pick = -1;
+  if (gsel >= 0) pick = resolve_pick<kApp>(bias, off, deg, want, rows, lastpos, gsel, tsel);
+  return pick;
+}
+
 // Step commit of a batch by one wave (lane i = walker i; include/walker.cuh:1410-1417).  Every walker's record
 // goes back to its own position of the output list, so no list counter is contended: finished walks are marked
 // (q = -1), walkers whose new vertex is parked on again are tagged and carry their position inside that vertex's
@@ -1348,6 +1575,9 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
     go_on = hidx != -2;
     park = hidx >= 0;
   }
+  const uint32_t label_slot = kApp == FW_APP_METAPATH ? (uint32_t)rec.len % (uint32_t)a.n_labels_per_hub : 0u;
+  const uint32_t bucket = (uint32_t)hidx * (uint32_t)a.n_labels_per_hub + label_slot;
+  const uint32_t rank = fw_wave_count_keys<true>(h.bucket_out, bucket, go_on && park);
   if (have) {
     fw_walker_rec out;
     out.q = go_on ? rec.q : -1;
@@ -1355,10 +1585,8 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
     out.prev = v;
     out.len = rec.len + 1;
     if (go_on && park) {
-      const uint32_t label_slot = kApp == FW_APP_METAPATH ? (uint32_t)rec.len % (uint32_t)a.n_labels_per_hub : 0u;
-      const uint32_t bucket = (uint32_t)hidx * (uint32_t)a.n_labels_per_hub + label_slot;
       out.cur = (int32_t)bucket;  // the vertex follows from the bucket
-      out.prev = (int32_t)atomicAdd(&h.bucket_out[bucket], 1u);
+      out.prev = (int32_t)rank;
       out.len |= FW_REC_PARK;
     }
     h.out[rec_base + (uint32_t)lane] = out;
@@ -1401,9 +1629,35 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
 
   __syncthreads();  // the shared initialisation above is visible
 
-  // ---- wave tasks first: lists up to hub_threshold, sampled at wave granularity, one batch per wave; the tasks are
-  //      short and many, so they are dealt out by position instead of through a contended counter ----
+  // ---- table tasks first: 64 walkers of a crowded hub whose rows the scan launch has made; one wave each,
+  //      dealt out by position like the wave tasks ----
   const uint32_t nwaves = gridDim.x * (uint32_t)kNW;
+  const uint32_t nttasks = *h.nttasks;
+  for (uint32_t t = blockIdx.x * (uint32_t)kNW + (uint32_t)wave; t < nttasks; t += nwaves) {
+    const fw_batch_task* tp = h.ttasks + t;
+    const int32_t v = __builtin_amdgcn_readfirstlane(tp->v);
+    const uint32_t off = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->off);
+    const uint32_t deg = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->deg);
+    const uint32_t rec_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->rec_base);
+    const int count = __builtin_amdgcn_readfirstlane(tp->count);
+    const uint32_t row_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->row);
+    const int32_t want = kApp == FW_APP_METAPATH ? s_schema[__builtin_amdgcn_readfirstlane(tp->slot)] : 0;
+
+    const bool have = lane < count;
+    fw_walker_rec rec;
+    rec.q = 0; rec.cur = v; rec.prev = -1; rec.len = 1;
+    if (have) rec = h.sorted[rec_base + (uint32_t)lane];
+    const uint32_t walker = a.walker_base + (uint32_t)rec.q;
+    const uint32_t step = (uint32_t)(rec.len - 1);
+
+    const int32_t sel = table_sample<kApp, kNW>(a, bias, off, deg, want, (int32_t)deg > a.hub_threshold, have, walker,
+                                               step, lane, h.totals + row_base, h.rows + (size_t)row_base * 128u,
+                                               h.lastpos + row_base);
+    batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, have, sel, walker, step, lane, n_steps, n_edges, n_out);
+  }
+
+  // ---- then wave tasks: lists up to hub_threshold, sampled at wave granularity, one batch per wave; the tasks are
+  //      short and many, so they are dealt out by position instead of through a contended counter ----
   for (uint32_t t = blockIdx.x * (uint32_t)kNW + (uint32_t)wave; t < nwtasks; t += nwaves) {
     const fw_batch_task* tp = h.wtasks + t;
     const int32_t v = __builtin_amdgcn_readfirstlane(tp->v);
@@ -1497,6 +1751,50 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
   }
 }
 
+// First pass of the two-pass steps: the rows of every crowded hub of the round.  A scan task is a run of groups
+// of one list (rec_base = first group, count = one past the last, row = the list's first row); one wave per
+// task, tasks dealt out by position.
+template <int kApp>
+__global__ __launch_bounds__(256) void fw_hub_scan(const fw_kargs a, const fw_hub_args h) {
+  __shared__ int32_t s_schema[kApp == FW_APP_METAPATH ? FW_MAX_SCHEMA : 1];
+  if (kApp == FW_APP_METAPATH) {
+    if (threadIdx.x == 0) {
+#pragma unroll
+      for (int i = 0; i < FW_MAX_SCHEMA; ++i) s_schema[i] = a.schema[i];
+    }
+    __syncthreads();
+  }
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const uint32_t nstasks = *h.nstasks;
+  const uint32_t* __restrict__ bias =
+      reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
+  const uint32_t nwaves = gridDim.x * 4u;
+  for (uint32_t t = blockIdx.x * 4u + (uint32_t)wave; t < nstasks; t += nwaves) {
+    const fw_batch_task* tp = h.stasks + t;
+    const uint32_t off = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->off);
+    const uint32_t deg = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->deg);
+    const uint32_t g0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->rec_base);
+    const uint32_t g1 = (uint32_t)__builtin_amdgcn_readfirstlane(tp->count);
+    const uint32_t row_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)tp->row);
+    const int32_t want = kApp == FW_APP_METAPATH ? s_schema[__builtin_amdgcn_readfirstlane(tp->slot)] : 0;
+    for (uint32_t g = g0; g < g1; ++g) {
+      const size_t r = (size_t)row_base + g;
+      group_rows<kApp>(bias, off, deg, want, g, lane, h.rows + r * 128u, h.totals + r, h.lastpos + r);
+    }
+  }
+}
+
+template <int kApp>
+int launch_hub_scan_app(const fw_kargs& a, const fw_hub_args& h, hipStream_t stream) {
+  int dev = 0, cus = 0;
+  FW_HIP(hipGetDevice(&dev));
+  FW_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  hipLaunchKernelGGL((fw_hub_scan<kApp>), dim3(cus * 8), dim3(256), 0, stream, a, h);
+  FW_HIP(hipGetLastError());
+  return FW_OK;
+}
+
 template <int kApp, int kWGT>
 int launch_hub_one(const fw_kargs& a, const fw_hub_args& h, hipStream_t stream) {
   int dev = 0;
@@ -1560,6 +1858,17 @@ int launch_app(const fw_kargs& a, int wg_threads, int grid, hipStream_t stream, 
 }
 
 }  // namespace
+
+int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, hipStream_t stream) {
+  switch (app) {
+    case FW_APP_DEEPWALK: return launch_hub_scan_app<FW_APP_DEEPWALK>(a, h, stream);
+    case FW_APP_PPR: return launch_hub_scan_app<FW_APP_PPR>(a, h, stream);
+    case FW_APP_METAPATH: return launch_hub_scan_app<FW_APP_METAPATH>(a, h, stream);
+    default:
+      fw_set_error("the hub scan kernel serves DeepWalk, PPR and MetaPath");
+      return FW_ERR_INVALID;
+  }
+}
 
 int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, hipStream_t stream) {
   switch (app) {

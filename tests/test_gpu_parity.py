@@ -107,6 +107,40 @@ def test_hub_parking_does_not_change_results(gpu, hub, app, wg):
         assert 0 < st.hub_steps <= st.steps
 
 
+@pytest.mark.parametrize("app", ["deepwalk", "ppr", "metapath"])
+def test_crowded_hub_is_scanned_once(gpu, hub, app):
+    """Every query starts on the same hub (the reference's --ppr start rule, src/main.cu:277-281, with many queries):
+    a bucket with hundreds of walkers on a long list is served in two passes (the list's rows once, then every
+    walker from the rows), its counters are updated once per wave, and the paths still equal the oracle's.  Both
+    sampler granularities: hub threshold below and above the hub's degree."""
+    starts = np.zeros(20000, dtype=np.int32)            # vertex 0: the 9000-degree hub
+    starts[15000:] = 1                                   # and 5000 on the 2500-degree one
+    kw = dict(deepwalk=dict(app=gpu.APP_DEEPWALK, max_depth=9),
+              ppr=dict(app=gpu.APP_PPR, max_depth=41, tp=0.2),
+              metapath=dict(app=gpu.APP_METAPATH, max_depth=6, schema=[2, 0, 4, 1, 3]))[app]
+    for hub_thr, park, wg in ((1000, 600, 512), (100000, 600, 256), (4000, 2000, 1024)):
+        _, st = _check(gpu, hub, starts, wg_threads=wg, hub_threshold=hub_thr, park_threshold=park, seed=5, **kw)
+        assert st.launches >= 3 and st.hub_steps >= 20000
+
+
+def test_walkers_that_move_together(gpu):
+    """Two centres joined to every other vertex, which are joined to the centres only: from a leaf every walker
+    moves to one of two vertices, so most lanes of a wave ask for a position in the same bucket at the same time
+    (one counter update per wave and bucket instead of one per walker).  Parked on everything (threshold 1)."""
+    leaves = 60
+    src = np.concatenate([np.zeros(leaves), np.ones(leaves), np.arange(2, leaves + 2), np.arange(2, leaves + 2)])
+    dst = np.concatenate([np.arange(2, leaves + 2), np.arange(2, leaves + 2), np.zeros(leaves), np.ones(leaves)])
+    xadj, adj = _graphs.csr_from_edges(leaves + 2, src.astype(np.int64), dst.astype(np.int64))
+    rs = np.random.RandomState(9)
+    w = rs.uniform(1.0, 9.0, size=len(adj)).astype(np.float32)
+    lab = rs.randint(0, 2, size=len(adj)).astype(np.int32)
+    starts = rs.randint(0, leaves + 2, size=30000).astype(np.int32)
+    for kw in (dict(app=gpu.APP_DEEPWALK, max_depth=12), dict(app=gpu.APP_PPR, max_depth=30, tp=0.1),
+               dict(app=gpu.APP_METAPATH, max_depth=7, schema=[0, 1, 1])):
+        _, st = _check(gpu, (xadj, adj, w, lab), starts, park_threshold=1, seed=13, **kw)
+        assert st.launches >= 3 and st.hub_steps > 0
+
+
 def test_default_parking_rule_and_its_tail(gpu, hub):
     """park_threshold = 0: the library decides (batches of at least 65,536 queries park where about four walkers
     meet), and once few walkers are left they finish in one launch without parking.  Same paths either way."""
