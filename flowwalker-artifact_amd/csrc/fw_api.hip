@@ -507,7 +507,8 @@ constexpr uint64_t kMaxRows = (2ull << 30) / 520u;  // 2 GiB of rows at most
 // two_pass_degree elements is served in two passes (scan tasks of up to kScanRun groups that make the list's rows,
 // one table task per 64 walkers) when its rows still fit; every other bucket gets one batch task per 64 walkers:
 // a workgroup task when its vertex is sampled at workgroup granularity (degree above hub_threshold), a wave task
-// otherwise.  ctrs (out): [3] workgroup tasks, [5] wave tasks, [7] table tasks, [8] scan tasks, [9] rows handed out.
+// otherwise.  ctrs (out): [3] workgroup tasks, [5] wave tasks, [7] table tasks, [8] scan tasks, [9] rows handed out,
+// [12] walkers in the fullest bucket when that is more than half of kTwoPassWalkers.
 constexpr uint32_t kScanRun = 16;
 
 struct TaskPlan {
@@ -572,6 +573,16 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
       t.slot = b % labels;
       ngroups = ((((t.off & 3u) + t.deg + 3u) >> 2) + 255u) / 256u;
     }
+    {
+      // the fullest bucket, for the host's decision about the next round
+      uint32_t cmax = c;
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) {
+        const uint32_t o = __shfl_xor(cmax, d);
+        cmax = o > cmax ? o : cmax;
+      }
+      if (lane == 0 && cmax * 2u > kTwoPassWalkers) atomicMax(&ctrs[12], cmax);  // smaller ones do not matter
+    }
     // rows first: a bucket whose rows do not fit any more falls back to batch tasks
     bool two_pass = c > plan.two_pass_walkers && t.deg >= plan.two_pass_degree;
     if (plan.two_pass_walkers != 0xFFFFFFFFu) {  // the same for every thread
@@ -632,6 +643,20 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
       }
     }
     __syncthreads();  // s_tot / s_base are reused by the next round
+  }
+}
+
+// Zeroes what a parking round starts from, in one launch: the round's counters, the next round's bucket counts, the
+// fill positions the scatter above has used, and the query dispenser.
+__global__ void fw_round_reset_kernel(uint32_t* ctrs, int n_ctrs, uint32_t* count_next, uint32_t* fill, int n_buckets,
+                                      uint32_t* dispenser) {
+  const int stride = gridDim.x * blockDim.x;
+  const int i0 = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i0 < n_ctrs) ctrs[i0] = 0u;
+  if (i0 == 0) *dispenser = 0u;
+  for (int i = i0; i < n_buckets; i += stride) {
+    count_next[i] = 0u;
+    fill[i] = 0u;
   }
 }
 
@@ -920,44 +945,58 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   h.lastpos = pb->lastpos;
   TaskPlan plan;
   plan.hub_threshold = p->hub_threshold;
-  plan.two_pass_walkers = pb->rows_cap != 0u ? kTwoPassWalkers : 0xFFFFFFFFu;
+  // Two-pass steps cost a launch per round that looks for scan tasks, so a round only gets them when the round
+  // before had a bucket at least half as full as they need (the first round always does): a bucket may then miss
+  // them for a round and is served by batches, with the same results.
+  const bool two_pass_possible = pb->rows_cap != 0u;
+  plan.two_pass_walkers = two_pass_possible ? kTwoPassWalkers : 0xFFFFFFFFu;
   plan.two_pass_degree = kTwoPassDegree;
   plan.rows_cap = pb->rows_cap;
 
-  // One walk launch and the read-back of the counters.
-  auto walk = [&](int* grid_out) -> int {
-    FW_HIP(hipMemsetAsync(a.dispenser, 0, sizeof(uint32_t), stream));  // used by the launch of fresh queries only
-    FW_HIP(hipMemsetAsync(pb->ctrs, 0, sizeof(uint32_t), stream));
-    TimedLaunch tw;
+  // Queues one walk launch (timed); the caller reads the counters back.
+  TimedLaunch tw;
+  auto queue_walk = [&](int* grid_out) -> int {
     int rc = tw.begin(stream);
     if (rc != FW_OK) return rc;
     rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, grid_out);
     if (rc != FW_OK) return rc;
     if ((rc = tw.end(stream)) != FW_OK) return rc;
     ++*launches;
-    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, kParkCtrs * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
-    FW_HIP(hipStreamSynchronize(stream));
-    tw.collect(&times->walk_ms);
     return FW_OK;
   };
+  auto read_back = [&]() -> int {
+    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, kParkCtrs * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    FW_HIP(hipStreamSynchronize(stream));
+    return FW_OK;
+  };
+  unsigned rblocks = ((unsigned)pb->n_buckets + 255u) / 256u;
+  if (rblocks > 2048u) rblocks = 2048u;
+  if (rblocks == 0u) rblocks = 1u;
 
   // first walk launch: fresh queries; the walkers it parks are counted in bucket array 0
   int cur = 0;
-  FW_HIP(hipMemsetAsync(pb->ctrs, 0, kParkCtrs * sizeof(uint32_t), stream));
-  FW_HIP(hipMemsetAsync(pb->count(0), 0, bucket_bytes, stream));
+  hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs, pb->count(0),
+                     pb->fill(), pb->n_buckets, a.dispenser);
+  FW_HIP(hipGetLastError());
   a.resume = nullptr;
+  a.n_dev = nullptr;
   a.bucket_count = pb->count(0);
-  int rc = walk(grid_used);
+  int rc = queue_walk(grid_used);
   if (rc != FW_OK) return rc;
+  if ((rc = read_back()) != FW_OK) return rc;
+  tw.collect(&times->walk_ms);
   uint32_t n_out = 0;  // records in `out` (the previous batch launch's input size)
+  uint32_t fullest = 0;  // walkers in the fullest bucket of the previous round
   for (;;) {
+    // one round: the walkers parked by the last walk launch and by the last batch launch are grouped by bucket, the
+    // batch launch moves each of them one step, and the walk launch queued right behind it takes those that are
+    // not parked again as far as their next parking.  The host looks at the counters once per round.
     const uint32_t n_walked = pb->h_ctrs[0];                 // parked by the walk launch
     const uint32_t n_again = n_out ? pb->h_ctrs[2] : 0u;     // parked again by the previous batch launch
     const uint64_t m = (uint64_t)n_walked + n_again;
     if (m == 0u) break;
     if (m > pb->cap) { fw_set_error("internal: %llu walkers parked, capacity %zu", (unsigned long long)m, pb->cap); return FW_ERR_INVALID; }
     const int nxt = cur ^ 1;
-    // group the round's walkers by bucket and cut the buckets into tasks; clear the next round's counts
     FW_HIP(rocprim::exclusive_scan(pb->tmp, pb->scan_bytes, pb->count(cur), pb->offset(), 0u, (size_t)pb->n_buckets,
                                    rocprim::plus<uint32_t>(), stream));
     auto blocks_for = [](uint32_t cnt) {
@@ -967,11 +1006,12 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     if (n_out != 0u)
       hipLaunchKernelGGL(fw_scatter_tagged_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
                          pb->offset(), pb->sorted);
-    if (n_walked != 0u) {
-      FW_HIP(hipMemsetAsync(pb->fill(), 0, bucket_bytes, stream));
+    if (n_walked != 0u)
       hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_walked)), dim3(256), 0, stream, pb->walked,
                          n_walked, pb->count(cur), pb->offset(), pb->fill(), pb->sorted);
-    }
+    FW_HIP(hipGetLastError());
+    hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs, pb->count(nxt),
+                       pb->fill(), pb->n_buckets, a.dispenser);
     FW_HIP(hipGetLastError());
     if (p->park_threshold == 0 && m < kParkTail) {
       // default rule only (an explicit threshold keeps every round in the loop): too few walkers are left to
@@ -980,12 +1020,15 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
                          pb->sorted, (uint32_t)m, g->hub_info, labels);
       FW_HIP(hipGetLastError());
       a.resume = pb->sorted;
+      a.n_dev = nullptr;
       a.n = (int32_t)m;
       a.park_threshold = INT_MAX;
-      return walk(nullptr);
+      if ((rc = queue_walk(nullptr)) != FW_OK) return rc;
+      if ((rc = read_back()) != FW_OK) return rc;
+      tw.collect(&times->walk_ms);
+      return FW_OK;
     }
-    FW_HIP(hipMemsetAsync(pb->ctrs + 1, 0, (kParkCtrs - 1) * sizeof(uint32_t), stream));
-    FW_HIP(hipMemsetAsync(pb->count(nxt), 0, bucket_bytes, stream));
+    plan.two_pass_walkers = two_pass_possible && (n_out == 0u || fullest * 2u > kTwoPassWalkers) ? kTwoPassWalkers : 0xFFFFFFFFu;
     unsigned tblocks = ((unsigned)pb->n_buckets + 1023u) / 1024u;
     if (tblocks > 1024u) tblocks = 1024u;
     hipLaunchKernelGGL(fw_bucket_tasks_kernel, dim3(tblocks), dim3(1024), 0, stream, pb->count(cur), pb->offset(),
@@ -996,7 +1039,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     TimedLaunch th;
     if ((rc = th.begin(stream)) != FW_OK) return rc;
     if (plan.two_pass_walkers != 0xFFFFFFFFu) {
-      rc = fw_launch_hub_scan(a, h, p->app, stream);  // finds its task count on the device; often none
+      rc = fw_launch_hub_scan(a, h, p->app, stream);  // finds its task count on the device
       if (rc != FW_OK) return rc;
     }
     rc = fw_launch_hub_batch(a, h, p->app, p->wg_threads, stream);
@@ -1010,25 +1053,22 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
                          pb->resume, pb->ctrs + 6);
       FW_HIP(hipGetLastError());
     }
-    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, kParkCtrs * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
-    FW_HIP(hipStreamSynchronize(stream));
+    // the walkers on vertices below the threshold continue in the walk kernel, which counts the walkers it parks in
+    // the same bucket array as the batch launch did; how many they are is only known on the device yet
+    a.resume = pb->resume;
+    a.n_dev = pb->ctrs + 6;
+    a.n = (int32_t)m;
+    a.bucket_count = pb->count(nxt);
+    if ((rc = queue_walk(nullptr)) != FW_OK) return rc;
+    if ((rc = read_back()) != FW_OK) return rc;
     th.collect(&times->hub_ms);
+    tw.collect(&times->walk_ms);
     if (getenv("FW_DEBUG_ROUNDS"))
-      fprintf(stderr, "round: parked %llu (walk %u + again %u) wg_tasks %u wave_tasks %u table_tasks %u scan_tasks %u rows %u -> resume %u again %u\n",
+      fprintf(stderr, "round: parked %llu (walk %u + again %u) wg_tasks %u wave_tasks %u table_tasks %u scan_tasks %u rows %u -> resume %u again %u, parked by the walk launch %u\n",
               (unsigned long long)m, n_walked, n_again, pb->h_ctrs[3], pb->h_ctrs[5], pb->h_ctrs[7], pb->h_ctrs[8],
-              pb->h_ctrs[9], pb->h_ctrs[1], pb->h_ctrs[2]);
+              pb->h_ctrs[9], pb->h_ctrs[6], pb->h_ctrs[2], pb->h_ctrs[0]);
     n_out = (uint32_t)m;
-    pb->h_ctrs[0] = 0u;
-    if (pb->h_ctrs[6] != 0u) {
-      // walkers on vertices below the threshold continue in the walk kernel, which counts the walkers it parks in
-      // the same bucket array as the batch launch did
-      a.resume = pb->resume;
-      a.n = (int32_t)pb->h_ctrs[6];
-      a.bucket_count = pb->count(nxt);
-      const uint32_t n_again_now = pb->h_ctrs[2];
-      if ((rc = walk(nullptr)) != FW_OK) return rc;
-      pb->h_ctrs[2] = n_again_now;  // unchanged by the walk launch; kept explicit for the next round
-    }
+    fullest = pb->h_ctrs[12];
     cur = nxt;
   }
   return FW_OK;

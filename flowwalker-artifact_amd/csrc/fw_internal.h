@@ -74,6 +74,8 @@ struct fw_kargs {
   uint32_t* parked_count;
   uint32_t* bucket_count;            // [n_hubs * n_labels_per_hub]
   const fw_walker_rec* resume;       // in: walkers to continue instead of fresh queries (NULL: use starts)
+  const uint32_t* n_dev;             // in: when not NULL, the number of entries is read here (n is an upper bound
+                                     // the grid was sized for) and slot_limit follows from it
 };
 
 // Tag in fw_walker_rec::len of a batch-kernel output record whose vertex is parked on again (stripped by readers).

@@ -860,6 +860,15 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   N2vScratch* const scr = &tt.n2v[kApp == FW_APP_NODE2VEC ? wave : 0];
   unsigned long long n_steps = 0ull, n_edges = 0ull;
+  // entries of this launch and the slots a workgroup fills: from the host, or (a launch queued before its input's
+  // size was known to the host) from the device, with the same rule: small inputs are spread over the grid
+  uint32_t n_entries = (uint32_t)a.n;
+  int32_t slot_limit = a.slot_limit;
+  if (a.n_dev != nullptr) {
+    n_entries = *a.n_dev;
+    const uint32_t per_wg = (n_entries + gridDim.x - 1u) / gridDim.x;
+    slot_limit = (int32_t)(per_wg < (uint32_t)kWGT ? (per_wg > 0u ? per_wg : 1u) : (uint32_t)kWGT);
+  }
 
   tt.len[tid] = -1;
   tt.flag[tid] = 0;
@@ -1007,7 +1016,7 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
       const int np = first ? 0 : parity;  // lists to fill for the next round
       first = false;
       int32_t len = tt.len[tid];
-      bool need = tid < a.slot_limit;  // slot wants a new walker
+      bool need = tid < slot_limit;  // slot wants a new walker
       bool park = false;               // the slot's walker has reached a hub that is served by the batch kernel
       int32_t hidx = -1;               // that vertex's index among the parked-on ones (read together with its CSR range)
       const bool parking = a.park_threshold != 0x7FFFFFFF;
@@ -1079,12 +1088,12 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
         if (want) {
           uint32_t q = base + (uint32_t)__builtin_popcountll(m & ((1ull << lane) - 1ull));
           if (by_position) {
-            const uint32_t chunk = q / (uint32_t)a.slot_limit;
-            const uint64_t pos = ((uint64_t)chunk * gridDim.x + blockIdx.x) * (uint64_t)a.slot_limit +
-                                 (q - chunk * (uint32_t)a.slot_limit);
-            q = pos < (uint64_t)(uint32_t)a.n ? (uint32_t)pos : 0xFFFFFFFFu;
+            const uint32_t chunk = q / (uint32_t)slot_limit;
+            const uint64_t pos = ((uint64_t)chunk * gridDim.x + blockIdx.x) * (uint64_t)slot_limit +
+                                 (q - chunk * (uint32_t)slot_limit);
+            q = pos < (uint64_t)n_entries ? (uint32_t)pos : 0xFFFFFFFFu;
           }
-          if (q < (uint32_t)a.n) {
+          if (q < n_entries) {
             int32_t wq, sp, pv, ln;
             if (a.resume != nullptr) {  // a walker coming back from its batch step
               const fw_walker_rec rec = a.resume[q];
