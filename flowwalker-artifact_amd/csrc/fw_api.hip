@@ -987,6 +987,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   tw.collect(&times->walk_ms);
   uint32_t n_out = 0;  // records in `out` (the previous batch launch's input size)
   uint32_t fullest = 0;  // walkers in the fullest bucket of the previous round
+  uint32_t scan_tasks = 0;  // and its scan tasks
   for (;;) {
     // one round: the walkers parked by the last walk launch and by the last batch launch are grouped by bucket, the
     // batch launch moves each of them one step, and the walk launch queued right behind it takes those that are
@@ -1039,7 +1040,8 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     TimedLaunch th;
     if ((rc = th.begin(stream)) != FW_OK) return rc;
     if (plan.two_pass_walkers != 0xFFFFFFFFu) {
-      rc = fw_launch_hub_scan(a, h, p->app, stream);  // finds its task count on the device
+      // finds its task count on the device; sized by the round before (twice that many tasks still get a wave each)
+      rc = fw_launch_hub_scan(a, h, p->app, n_out != 0u ? scan_tasks * 4u + 1u : 0u, stream);
       if (rc != FW_OK) return rc;
     }
     rc = fw_launch_hub_batch(a, h, p->app, p->wg_threads, stream);
@@ -1069,6 +1071,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
               pb->h_ctrs[9], pb->h_ctrs[6], pb->h_ctrs[2], pb->h_ctrs[0]);
     n_out = (uint32_t)m;
     fullest = pb->h_ctrs[12];
+    scan_tasks = pb->h_ctrs[8];
     cur = nxt;
   }
   return FW_OK;

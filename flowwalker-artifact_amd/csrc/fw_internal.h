@@ -176,4 +176,5 @@ int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int 
 // Launches the hub batch kernel (persistent grid, tasks taken from h.task_next).
 int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, hipStream_t stream);
 // Launches the scan kernel of the two-pass steps (it finds its task count in h.nstasks on the device).
-int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, hipStream_t stream);
+// tasks_hint: about how many scan tasks to expect, to size the grid (0 = no idea: a full resident set).
+int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, uint32_t tasks_hint, hipStream_t stream);

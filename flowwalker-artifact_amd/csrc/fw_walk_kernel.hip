@@ -1794,12 +1794,15 @@ __global__ __launch_bounds__(256) void fw_hub_scan(const fw_kargs a, const fw_hu
   }
 }
 
+// tasks_hint: about how many scan tasks to expect (the launch works through any number; 0 = no idea)
 template <int kApp>
-int launch_hub_scan_app(const fw_kargs& a, const fw_hub_args& h, hipStream_t stream) {
+int launch_hub_scan_app(const fw_kargs& a, const fw_hub_args& h, uint32_t tasks_hint, hipStream_t stream) {
   int dev = 0, cus = 0;
   FW_HIP(hipGetDevice(&dev));
   FW_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  hipLaunchKernelGGL((fw_hub_scan<kApp>), dim3(cus * 8), dim3(256), 0, stream, a, h);
+  uint32_t grid = (uint32_t)cus * 8u;  // one resident set
+  if (tasks_hint != 0u && tasks_hint / 2u + 32u < grid) grid = tasks_hint / 2u + 32u;  // 4 waves a workgroup, room to grow
+  hipLaunchKernelGGL((fw_hub_scan<kApp>), dim3(grid), dim3(256), 0, stream, a, h);
   FW_HIP(hipGetLastError());
   return FW_OK;
 }
@@ -1868,11 +1871,11 @@ int launch_app(const fw_kargs& a, int wg_threads, int grid, hipStream_t stream, 
 
 }  // namespace
 
-int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, hipStream_t stream) {
+int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, uint32_t tasks_hint, hipStream_t stream) {
   switch (app) {
-    case FW_APP_DEEPWALK: return launch_hub_scan_app<FW_APP_DEEPWALK>(a, h, stream);
-    case FW_APP_PPR: return launch_hub_scan_app<FW_APP_PPR>(a, h, stream);
-    case FW_APP_METAPATH: return launch_hub_scan_app<FW_APP_METAPATH>(a, h, stream);
+    case FW_APP_DEEPWALK: return launch_hub_scan_app<FW_APP_DEEPWALK>(a, h, tasks_hint, stream);
+    case FW_APP_PPR: return launch_hub_scan_app<FW_APP_PPR>(a, h, tasks_hint, stream);
+    case FW_APP_METAPATH: return launch_hub_scan_app<FW_APP_METAPATH>(a, h, tasks_hint, stream);
     default:
       fw_set_error("the hub scan kernel serves DeepWalk, PPR and MetaPath");
       return FW_ERR_INVALID;
