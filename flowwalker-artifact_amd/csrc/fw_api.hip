@@ -434,6 +434,15 @@ static void fill_kargs(fw_kargs* a, const fw_graph* g, const fw_walk_params* p) 
 // (counting sort on the device), the hub batch kernel serves up to 64 walkers of a hub with one pass over its
 // list, and the survivors resume in the next walk launch.  Loop until nobody is parked.
 
+// Two-pass steps: buckets with more than kTwoPassWalkers walkers on lists of at least kTwoPassDegree elements.
+// Every such list has rows of its own (520 bytes per 1024 elements and label a walker can want), set aside when
+// the lists are numbered, so that nothing has to be handed out while the walks run; kMaxHubRows bounds them
+// (lists past it are served by batches, however crowded).
+constexpr uint32_t kTwoPassWalkers = 256;
+constexpr uint32_t kTwoPassDegree = 2048;
+constexpr uint32_t kMaxHubRows = 1u << 21;             // per label: 1 GiB of rows
+constexpr uint64_t kMaxRows = (4ull << 30) / 520u;     // all labels together: 4 GiB
+
 __global__ void fw_hub_count_kernel(const uint32_t* __restrict__ xadj, int32_t V, int32_t threshold, unsigned* count) {
   const int stride = gridDim.x * blockDim.x;
   unsigned local = 0;
@@ -442,8 +451,11 @@ __global__ void fw_hub_count_kernel(const uint32_t* __restrict__ xadj, int32_t V
   if (local) atomicAdd(count, local);
 }
 
+// next[0]: the next hub number; next[1]: the next free row.  A hub of at least rows_degree elements gets rows for its
+// groups (1024 elements each, from the list's first aligned quartet on) while fewer than rows_limit are taken.
 __global__ void fw_hub_index_kernel(const uint32_t* __restrict__ xadj, int32_t V, int32_t threshold, unsigned* next,
-                                    int32_t* hub_index, fw_hub_info* hub_info) {
+                                    int32_t* hub_index, fw_hub_info* hub_info, uint32_t rows_degree,
+                                    uint32_t rows_limit) {
   const int stride = gridDim.x * blockDim.x;
   for (int v = blockIdx.x * blockDim.x + threadIdx.x; v < V; v += stride) {
     int32_t idx = -1;
@@ -453,7 +465,12 @@ __global__ void fw_hub_index_kernel(const uint32_t* __restrict__ xadj, int32_t V
       hi.v = v;
       hi.off = xadj[v];
       hi.deg = xadj[v + 1] - hi.off;
-      hi.pad = 0u;
+      hi.row = FW_NO_ROWS;
+      if (hi.deg >= rows_degree) {
+        const uint32_t ngroups = ((((hi.off & 3u) + hi.deg + 3u) >> 2) + 255u) / 256u;
+        const uint32_t row = atomicAdd(&next[1], ngroups);
+        if (row < rows_limit && ngroups <= rows_limit - row) hi.row = row;
+      }
       hub_info[idx] = hi;
     }
     // -1: not parked on; -2: no neighbours at all (a walker that arrives there is finished)
@@ -469,8 +486,8 @@ static int ensure_hub_index(fw_graph* g, int32_t threshold) {
   g->hub_index_threshold = -1;
   g->n_hubs = 0;
   unsigned* d_cnt = nullptr;
-  FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_cnt), 2 * sizeof(unsigned)));
-  FW_HIP(hipMemset(d_cnt, 0, 2 * sizeof(unsigned)));
+  FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_cnt), 3 * sizeof(unsigned)));
+  FW_HIP(hipMemset(d_cnt, 0, 3 * sizeof(unsigned)));
   hipLaunchKernelGGL(fw_hub_count_kernel, dim3(1024), dim3(256), 0, 0, g->xadj, g->V, threshold, d_cnt);
   unsigned n_hubs = 0;
   int rc = fw_check_hip(hipMemcpy(&n_hubs, d_cnt, sizeof(unsigned), hipMemcpyDeviceToHost), "hipMemcpy(hub count)", __FILE__, __LINE__);
@@ -478,12 +495,15 @@ static int ensure_hub_index(fw_graph* g, int32_t threshold) {
   if (rc == FW_OK) rc = fw_check_hip(hipMalloc(reinterpret_cast<void**>(&g->hub_info), (size_t)(n_hubs ? n_hubs : 1) * sizeof(fw_hub_info)), "hipMalloc(hub_info)", __FILE__, __LINE__);
   if (rc == FW_OK) {
     hipLaunchKernelGGL(fw_hub_index_kernel, dim3(1024), dim3(256), 0, 0, g->xadj, g->V, threshold, d_cnt + 1,
-                       g->hub_index, g->hub_info);
+                       g->hub_index, g->hub_info, kTwoPassDegree, kMaxHubRows);
     rc = fw_check_hip(hipDeviceSynchronize(), "hub index", __FILE__, __LINE__);
   }
+  unsigned rows_taken = 0;
+  if (rc == FW_OK) rc = fw_check_hip(hipMemcpy(&rows_taken, d_cnt + 2, sizeof(unsigned), hipMemcpyDeviceToHost), "hipMemcpy(hub rows)", __FILE__, __LINE__);
   (void)hipFree(d_cnt);
   if (rc != FW_OK) return rc;
   g->n_hubs = (int32_t)n_hubs;
+  g->hub_rows = rows_taken < kMaxHubRows ? rows_taken : kMaxHubRows;  // rows past the limit were not handed out
   g->hub_index_threshold = threshold;
   return FW_OK;
 }
@@ -498,24 +518,18 @@ constexpr double kParkMeet = 4.0;
 constexpr int32_t kMinDefaultPark = 64;
 constexpr int32_t kMinParkThreshold = 1;
 constexpr int kParkCtrs = 16;                    // counters of a parking round
-// Two-pass steps: buckets with more than kTwoPassWalkers walkers on lists of at least kTwoPassDegree elements
-constexpr uint32_t kTwoPassWalkers = 256;
-constexpr uint32_t kTwoPassDegree = 2048;
-constexpr uint64_t kMaxRows = (2ull << 30) / 520u;  // 2 GiB of rows at most
 
-// Cuts the round's buckets into tasks.  A bucket with more than two_pass_walkers walkers on a list of at least
-// two_pass_degree elements is served in two passes (scan tasks of up to kScanRun groups that make the list's rows,
-// one table task per 64 walkers) when its rows still fit; every other bucket gets one batch task per 64 walkers:
+// Cuts the round's buckets into tasks.  A bucket with more than two_pass_walkers walkers on a list that has rows
+// is served in two passes (scan tasks of up to kScanRun groups that make the list's rows, one table task per 64
+// walkers); every other bucket gets one batch task per 64 walkers:
 // a workgroup task when its vertex is sampled at workgroup granularity (degree above hub_threshold), a wave task
-// otherwise.  ctrs (out): [3] workgroup tasks, [5] wave tasks, [7] table tasks, [8] scan tasks, [9] rows handed out,
+// otherwise.  ctrs (out): [3] workgroup tasks, [5] wave tasks, [7] table tasks, [8] scan tasks,
 // [12] walkers in the fullest bucket when that is more than half of kTwoPassWalkers.
 constexpr uint32_t kScanRun = 16;
 
 struct TaskPlan {
   int32_t hub_threshold;
   uint32_t two_pass_walkers;  // 0xFFFFFFFF: never
-  uint32_t two_pass_degree;
-  uint32_t rows_cap;
 };
 
 __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* __restrict__ bucket_count,
@@ -528,49 +542,27 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
   constexpr int kKinds = 4;  // workgroup, wave, table, scan
   __shared__ uint32_t s_tot[kKinds][16];
   __shared__ uint32_t s_base[kKinds];
-  const int ctr_of[kKinds] = {3, 5, 7, 8};
+  __shared__ uint32_t s_cmax;
+  if (threadIdx.x == 0) s_cmax = 0u;
+  __syncthreads();
   const int stride = gridDim.x * blockDim.x;
   const int lane = (int)(threadIdx.x & 63u);
   const int wave = (int)(threadIdx.x >> 6);
   const int rounds = (n_buckets + stride - 1) / stride;  // every thread runs every round: scans and barriers
-
-  // exclusive position of x among the workgroup's threads, plus a base from the global counter `ctr`
-  auto place = [&](uint32_t x, int ctr) -> uint32_t {
-    uint32_t inc = x;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const uint32_t up = __shfl_up(inc, d);
-      if (lane >= d) inc += up;
-    }
-    if (lane == 63) s_tot[0][wave] = inc;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      uint32_t total = 0u;
-      for (int w = 0; w < 16; ++w) {
-        const uint32_t v = s_tot[0][w];
-        s_tot[0][w] = total;
-        total += v;
-      }
-      s_base[0] = total != 0u ? atomicAdd(&ctrs[ctr], total) : 0u;
-    }
-    __syncthreads();
-    const uint32_t at = s_base[0] + s_tot[0][wave] + inc - x;
-    __syncthreads();  // s_tot / s_base are reused
-    return at;
-  };
 
   for (int r = 0; r < rounds; ++r) {
     const int b = r * stride + (int)(blockIdx.x * blockDim.x + threadIdx.x);
     const uint32_t c = b < n_buckets ? bucket_count[b] : 0u;
     fw_batch_task t;
     t.v = 0; t.off = 0; t.deg = 0; t.slot = 0; t.rec_base = 0; t.count = 0; t.row = 0; t.pad = 0;
-    uint32_t ngroups = 0u;
+    uint32_t ngroups = 0u, hub_row = FW_NO_ROWS;
     if (c != 0u) {
       const fw_hub_info hi = hub_info[b / labels];
       t.v = hi.v;
       t.off = hi.off;
       t.deg = hi.deg;
       t.slot = b % labels;
+      hub_row = hi.row;
       ngroups = ((((t.off & 3u) + t.deg + 3u) >> 2) + 255u) / 256u;
     }
     {
@@ -581,15 +573,10 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
         const uint32_t o = __shfl_xor(cmax, d);
         cmax = o > cmax ? o : cmax;
       }
-      if (lane == 0 && cmax * 2u > kTwoPassWalkers) atomicMax(&ctrs[12], cmax);  // smaller ones do not matter
+      if (lane == 0 && cmax * 2u > kTwoPassWalkers) atomicMax(&s_cmax, cmax);  // smaller ones do not matter
     }
-    // rows first: a bucket whose rows do not fit any more falls back to batch tasks
-    bool two_pass = c > plan.two_pass_walkers && t.deg >= plan.two_pass_degree;
-    if (plan.two_pass_walkers != 0xFFFFFFFFu) {  // the same for every thread
-      const uint32_t row = place(two_pass ? ngroups : 0u, 9);
-      two_pass = two_pass && row <= plan.rows_cap && ngroups <= plan.rows_cap - row;
-      t.row = row;
-    }
+    const bool two_pass = c > plan.two_pass_walkers && hub_row != FW_NO_ROWS;
+    if (two_pass) t.row = hub_row * (uint32_t)labels + (uint32_t)t.slot * ngroups;
     const bool wg = (int32_t)t.deg > plan.hub_threshold;
     const uint32_t nb = (c + 63u) >> 6;
     uint32_t x[kKinds];
@@ -613,6 +600,10 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
       for (int k = 0; k < kKinds; ++k) s_tot[k][wave] = inc[k];
     }
     __syncthreads();
+    if (threadIdx.x == kKinds && s_cmax != 0u) {  // one update of the global maximum per workgroup
+      atomicMax(&ctrs[12], s_cmax);
+      s_cmax = 0u;
+    }
     if (threadIdx.x < kKinds) {
       uint32_t total = 0u;
       for (int w = 0; w < 16; ++w) {  // exclusive prefix over the waves, in place
@@ -620,15 +611,33 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
         s_tot[threadIdx.x][w] = total;
         total += v;
       }
-      s_base[threadIdx.x] = total != 0u ? atomicAdd(&ctrs[ctr_of[threadIdx.x]], total) : 0u;
+      const int ctr = threadIdx.x == 0 ? 3 : (threadIdx.x == 1 ? 5 : (threadIdx.x == 2 ? 7 : 8));
+      s_base[threadIdx.x] = total != 0u ? atomicAdd(&ctrs[ctr], total) : 0u;
     }
     __syncthreads();
+    const int kind = two_pass ? 2 : (wg ? 0 : 1);
+    // (selected, not indexed: the arrays stay in registers)
+    const uint32_t mine = two_pass ? inc[2] - x[2] : (wg ? inc[0] - x[0] : inc[1] - x[1]);
+    const uint32_t t0 = s_base[kind] + s_tot[kind][wave] + mine;
+    const uint32_t base = c != 0u ? bucket_offset[b] : 0u;
+    // a crowded bucket has thousands of tasks: those are written by the whole wave, one bucket after the other
+    constexpr uint32_t kOwnTasks = 8;
+    for (uint64_t big = __ballot(nb > kOwnTasks); big != 0ull; big &= big - 1ull) {
+      const int l = __builtin_ctzll(big);
+      fw_batch_task bt;
+      bt.v = __shfl(t.v, l); bt.off = __shfl(t.off, l); bt.deg = __shfl(t.deg, l); bt.slot = __shfl(t.slot, l);
+      bt.row = __shfl(t.row, l); bt.pad = 0;
+      const uint32_t bc = __shfl(c, l), bbase = __shfl(base, l), bt0 = __shfl(t0, l), bnb = __shfl(nb, l);
+      fw_batch_task* bout = __shfl(kind, l) == 0 ? tasks : (__shfl(kind, l) == 1 ? wtasks : ttasks);
+      for (uint32_t k = (uint32_t)lane; k < bnb; k += 64u) {
+        bt.rec_base = bbase + 64u * k;
+        bt.count = (int32_t)(bc - 64u * k < 64u ? bc - 64u * k : 64u);
+        bout[bt0 + k] = bt;
+      }
+    }
     if (c != 0u) {
-      const int kind = two_pass ? 2 : (wg ? 0 : 1);
-      const uint32_t t0 = s_base[kind] + s_tot[kind][wave] + inc[kind] - x[kind];
       fw_batch_task* out = kind == 0 ? tasks : (kind == 1 ? wtasks : ttasks);
-      const uint32_t base = bucket_offset[b];
-      for (uint32_t k = 0; k < nb; ++k) {
+      for (uint32_t k = 0; k < (nb > kOwnTasks ? 0u : nb); ++k) {
         t.rec_base = base + 64u * k;
         t.count = (int32_t)(c - 64u * k < 64u ? c - 64u * k : 64u);
         out[t0 + k] = t;
@@ -764,7 +773,7 @@ struct ParkBuffers {
   fw_batch_task* wtasks = nullptr;
   uint32_t* ctrs = nullptr;           // [0] walkers in `walked`, [1] records of `out` that resume, [2] that are parked
                                       // again, [3] workgroup tasks, [4] their dispenser, [5] wave tasks, [6] records in
-                                      // `resume`, [7] table tasks, [8] scan tasks, [9] rows handed out
+                                      // `resume`, [7] table tasks, [8] scan tasks, [12] walkers in the fullest bucket
   fw_batch_task* ttasks = nullptr;    // two-pass steps: table tasks, scan tasks and the rows between them
   fw_batch_task* stasks = nullptr;
   float* totals = nullptr;
@@ -793,7 +802,6 @@ struct ParkBuffers {
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), kParkCtrs * sizeof(uint32_t)));
     FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), kParkCtrs * sizeof(uint32_t), hipHostMallocDefault));
     // the rows are an extra: without room for them every bucket is served by batch tasks
-    if (rows_wanted > kMaxRows) rows_wanted = kMaxRows;
     if (rows_wanted != 0u) {
       // scan tasks: a list of G groups is cut into at most G / kScanRun + 1 runs, and no more lists are scanned in
       // a round than there are buckets or walkers
@@ -848,7 +856,7 @@ static void release_park_cache(fw_graph* g) {
 // NULL when the memory is not there (the caller then walks without parking).
 static ParkBuffers* cached_park_buffers(fw_graph* g, size_t n, int n_buckets, uint64_t rows_wanted) {
   ParkBuffers* c = static_cast<ParkBuffers*>(g->park_cache);
-  if (c && c->cap >= n && c->n_buckets == n_buckets) return c;
+  if (c && c->cap >= n && c->n_buckets == n_buckets && c->rows_cap >= rows_wanted) return c;
   release_park_cache(g);
   c = new (std::nothrow) ParkBuffers;
   if (!c) return nullptr;
@@ -862,15 +870,10 @@ static ParkBuffers* cached_park_buffers(fw_graph* g, size_t n, int n_buckets, ui
   return c;
 }
 
-// Rows to set aside for two-pass steps.  A list of d elements has at most d / 1024 + 2 groups, so all lists of
-// kTwoPassDegree elements or more together have at most E / 512 per label a walker can want; a quarter of that is
-// set aside, because only the lists that are crowded in the same round need rows at the same time, and a bucket
-// whose rows do not fit is served by batches like any other.
+// Rows the two-pass steps of a call need: every hub that has rows, once per label a walker can want.
 static uint64_t two_pass_rows(const fw_graph* g, int labels) {
-  int32_t max_degree = 0;
-  if (fw_graph_info(g, nullptr, nullptr, &max_degree, nullptr) != FW_OK) return 0;
-  if ((uint32_t)max_degree < kTwoPassDegree) return 0;
-  return (uint64_t)labels * (g->E / 2048u + 1024u);
+  const uint64_t rows = (uint64_t)g->hub_rows * (uint64_t)labels;
+  return rows <= kMaxRows ? rows : 0;  // too many: no two-pass steps in this call
 }
 
 // Decides whether a call parks walkers, and at which degree.  Returns INT_MAX for "no".
@@ -950,8 +953,6 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   // them for a round and is served by batches, with the same results.
   const bool two_pass_possible = pb->rows_cap != 0u;
   plan.two_pass_walkers = two_pass_possible ? kTwoPassWalkers : 0xFFFFFFFFu;
-  plan.two_pass_degree = kTwoPassDegree;
-  plan.rows_cap = pb->rows_cap;
 
   // Queues one walk launch (timed); the caller reads the counters back.
   TimedLaunch tw;
@@ -1066,9 +1067,9 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     th.collect(&times->hub_ms);
     tw.collect(&times->walk_ms);
     if (getenv("FW_DEBUG_ROUNDS"))
-      fprintf(stderr, "round: parked %llu (walk %u + again %u) wg_tasks %u wave_tasks %u table_tasks %u scan_tasks %u rows %u -> resume %u again %u, parked by the walk launch %u\n",
+      fprintf(stderr, "round: parked %llu (walk %u + again %u) wg_tasks %u wave_tasks %u table_tasks %u scan_tasks %u -> resume %u again %u, parked by the walk launch %u\n",
               (unsigned long long)m, n_walked, n_again, pb->h_ctrs[3], pb->h_ctrs[5], pb->h_ctrs[7], pb->h_ctrs[8],
-              pb->h_ctrs[9], pb->h_ctrs[6], pb->h_ctrs[2], pb->h_ctrs[0]);
+              pb->h_ctrs[6], pb->h_ctrs[2], pb->h_ctrs[0]);
     n_out = (uint32_t)m;
     fullest = pb->h_ctrs[12];
     scan_tasks = pb->h_ctrs[8];

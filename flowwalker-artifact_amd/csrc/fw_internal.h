@@ -11,8 +11,9 @@ struct fw_hub_info {
   int32_t v;
   uint32_t off;  // xadj[v]
   uint32_t deg;
-  uint32_t pad;
+  uint32_t row;  // two-pass steps: first row of this list's groups (times the labels per hub), FW_NO_ROWS: none
 };
+constexpr uint32_t FW_NO_ROWS = 0xFFFFFFFFu;
 
 // Device CSR mirror (include/gpu_graph.cuh:28-36 in the reference).  Edge arrays are allocated with
 // FW_EDGE_PAD extra elements so that aligned 16-byte loads of the last quartet stay in bounds.
@@ -31,6 +32,7 @@ struct fw_graph {
   // lazily built index of the vertices whose degree exceeds hub_index_threshold (hub parking)
   int32_t hub_index_threshold = -1;
   int32_t n_hubs = 0;
+  uint32_t hub_rows = 0;              // rows the hubs with rows need together, per label
   int32_t* hub_index = nullptr;       // int32[V]: position in hub_info, -1 (not parked on) or -2 (degree 0)
   struct fw_hub_info* hub_info = nullptr;  // [n_hubs]
   void* park_cache = nullptr;         // the parking lists of the last fw_walk_device call, kept for the next one
