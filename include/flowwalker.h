@@ -76,7 +76,7 @@ typedef struct {
   int32_t grid;           /* workgroups per launch actually used */
   /* per-kernel breakdown of kernel_ms / steps / sampled_edges (hub parking splits a pass over two kernels) */
   double walk_kernel_ms;      /* sum over fw_walk_zprs launches */
-  double hub_kernel_ms;       /* sum over fw_hub_batch launches */
+  double hub_kernel_ms;       /* sum over fw_hub_batch launches (and the fw_hub_scan launches in front of them) */
   uint64_t hub_steps;         /* steps taken in fw_hub_batch (included in steps) */
   uint64_t hub_sampled_edges; /* their source degrees (included in sampled_edges) */
 } fw_walk_stats;
