@@ -921,7 +921,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   *launches = 0;
   if (park_threshold == INT_MAX || g->n_hubs == 0 || pb == nullptr) {
     *launches = 1;
-    return fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, grid_used);
+    return fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, 0u, stream, grid_used);
   }
   const int labels = p->app == FW_APP_METAPATH ? p->schema_len : 1;
   const size_t bucket_bytes = (size_t)pb->n_buckets * sizeof(uint32_t);
@@ -956,10 +956,17 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
 
   // Queues one walk launch (timed); the caller reads the counters back.
   TimedLaunch tw;
+  uint32_t entries_hint = 0u;  // set before every queue_walk
+  // the hint counts entries of the kind the grid rule was made for, lists of up to 124 neighbours (four or two to a
+  // wave); with a higher parking threshold an entry is more work, about in proportion
+  auto hint_for = [&](uint64_t entries) -> uint32_t {
+    const uint64_t scaled = park_threshold > 124 ? entries * (uint64_t)park_threshold / 124u : entries;
+    return scaled < 0x7FFFFFFFull ? (uint32_t)scaled : 0x7FFFFFFFu;
+  };
   auto queue_walk = [&](int* grid_out) -> int {
     int rc = tw.begin(stream);
     if (rc != FW_OK) return rc;
-    rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, stream, grid_out);
+    rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, entries_hint, stream, grid_out);
     if (rc != FW_OK) return rc;
     if ((rc = tw.end(stream)) != FW_OK) return rc;
     ++*launches;
@@ -982,6 +989,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   a.resume = nullptr;
   a.n_dev = nullptr;
   a.bucket_count = pb->count(0);
+  entries_hint = hint_for((uint64_t)a.n);
   int rc = queue_walk(grid_used);
   if (rc != FW_OK) return rc;
   if ((rc = read_back()) != FW_OK) return rc;
@@ -989,6 +997,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   uint32_t n_out = 0;  // records in `out` (the previous batch launch's input size)
   uint32_t fullest = 0;  // walkers in the fullest bucket of the previous round
   uint32_t scan_tasks = 0;  // and its scan tasks
+  uint32_t resumed = 0;     // and the walkers that went on in its walk launch
   for (;;) {
     // one round: the walkers parked by the last walk launch and by the last batch launch are grouped by bucket, the
     // batch launch moves each of them one step, and the walk launch queued right behind it takes those that are
@@ -1025,6 +1034,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
       a.n_dev = nullptr;
       a.n = (int32_t)m;
       a.park_threshold = INT_MAX;
+      entries_hint = 0u;  // these walkers run to the end of their walks: every workgroup is wanted
       if ((rc = queue_walk(nullptr)) != FW_OK) return rc;
       if ((rc = read_back()) != FW_OK) return rc;
       tw.collect(&times->walk_ms);
@@ -1062,6 +1072,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     a.n_dev = pb->ctrs + 6;
     a.n = (int32_t)m;
     a.bucket_count = pb->count(nxt);
+    entries_hint = hint_for(n_out != 0u ? (uint64_t)resumed + 1u : m / 4u + 1u);  // about as many as a round ago
     if ((rc = queue_walk(nullptr)) != FW_OK) return rc;
     if ((rc = read_back()) != FW_OK) return rc;
     th.collect(&times->hub_ms);
@@ -1072,6 +1083,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
               pb->h_ctrs[6], pb->h_ctrs[2], pb->h_ctrs[0]);
     n_out = (uint32_t)m;
     fullest = pb->h_ctrs[12];
+    resumed = pb->h_ctrs[6];
     scan_tasks = pb->h_ctrs[8];
     cur = nxt;
   }

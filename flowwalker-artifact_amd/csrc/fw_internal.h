@@ -172,8 +172,10 @@ int fw_check_hip(hipError_t e, const char* what, const char* file, int line);
 
 // Launches the walk kernel for (app, sampler, wg_threads) on `stream`.  grid = 0: fill the device.
 // Returns the grid used through *grid_used.
-int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, hipStream_t stream,
-                   int* grid_used);
+// entries_hint: launches of the parking pipeline say about how many entries they will find (sizes the grid when
+// grid <= 0); 0 for a launch whose walkers run their whole walks.
+int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, uint32_t entries_hint,
+                   hipStream_t stream, int* grid_used);
 
 // Launches the hub batch kernel (persistent grid, tasks taken from h.task_next).
 int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, hipStream_t stream);

@@ -754,35 +754,61 @@ __device__ __forceinline__ void commit(const fw_kargs& a, TaskTable<kWGT, kApp>&
 // segment exactly as it joins rows 0 and 1 of a whole wave, and the steps of the whole-wave scan that are left out
 // only ever add zeros for such a list, so every slot gets the element it would get from a wave of its own.
 // `slot` is this lane's slot or -1.  Not for node2vec (its biases need the adjacency test).
+// What a packed step keeps between its two halves: the loads are started for several bundles before the first one
+// is finished, so that a wave waits for memory once per pair of bundles instead of once per bundle.
+struct PackedBundle {
+  int slot;
+  uint32_t off, deg, d0;
+  int32_t len, want;
+  bool have;
+  uint4 raw;
+  int4 adj;
+};
+
 template <int kApp, int kSeg, int kWGT>
-__device__ __forceinline__ void packed_step(const fw_kargs& a, TaskTable<kWGT, kApp>& tt, const int lane,
-                                            const int slot, unsigned long long& n_steps,
-                                            unsigned long long& n_edges) {
+__device__ __forceinline__ void packed_load(const fw_kargs& a, TaskTable<kWGT, kApp>& tt, const int lane,
+                                            const int slot, PackedBundle& b) {
   static_assert(kSeg == 16 || kSeg == 32, "a segment is one or two DPP rows");
   const bool active = slot >= 0;
   const int c = lane & (kSeg - 1);
-  const int seg_first = lane & ~(kSeg - 1);
-  uint32_t off = 0u, deg = 0u, d0 = 0u;
-  int32_t len = 1, want = 0;
+  b.slot = slot;
+  b.off = 0u; b.deg = 0u; b.d0 = 0u; b.len = 1; b.want = 0;
   if (active) {
-    off = tt.off[slot];
-    deg = (uint32_t)tt.deg[slot];
-    len = tt.len[slot];
-    d0 = tt.draw[0][slot];
-    if (kApp == FW_APP_METAPATH) want = tt.want[slot];
+    b.off = tt.off[slot];
+    b.deg = (uint32_t)tt.deg[slot];
+    b.len = tt.len[slot];
+    b.d0 = tt.draw[0][slot];
+    if (kApp == FW_APP_METAPATH) b.want = tt.want[slot];
   }
-  const uint32_t a0 = off & ~3u;
-  const uint32_t nq = (off + deg - a0 + 3u) >> 2;
-  const bool have = active && (uint32_t)c < nq;
+  const uint32_t a0 = b.off & ~3u;
+  const uint32_t nq = (b.off + b.deg - a0 + 3u) >> 2;
+  b.have = active && (uint32_t)c < nq;
   const uint32_t base = a0 + 4u * (uint32_t)c;
   const uint32_t* __restrict__ bias =
       reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
-  uint4 raw = make_uint4(0, 0, 0, 0);
-  int4 adj = make_int4(-1, -1, -1, -1);
-  if (have) {
-    raw = *reinterpret_cast<const uint4*>(bias + base);
-    adj = *reinterpret_cast<const int4*>(a.adjncy + base);
+  b.raw = make_uint4(0, 0, 0, 0);
+  b.adj = make_int4(-1, -1, -1, -1);
+  if (b.have) {
+    b.raw = *reinterpret_cast<const uint4*>(bias + base);
+    b.adj = *reinterpret_cast<const int4*>(a.adjncy + base);
   }
+}
+
+template <int kApp, int kSeg, int kWGT>
+__device__ __forceinline__ void packed_finish(const fw_kargs& a, TaskTable<kWGT, kApp>& tt, const int lane,
+                                              const PackedBundle& b, unsigned long long& n_steps,
+                                              unsigned long long& n_edges) {
+  const int slot = b.slot;
+  const bool active = slot >= 0;
+  const int c = lane & (kSeg - 1);
+  const int seg_first = lane & ~(kSeg - 1);
+  const uint32_t off = b.off, deg = b.deg, d0 = b.d0;
+  const int32_t len = b.len, want = b.want;
+  const bool have = b.have;
+  const uint4 raw = b.raw;
+  const int4 adj = b.adj;
+  const uint32_t a0 = off & ~3u;
+  const uint32_t base = a0 + 4u * (uint32_t)c;
   float x[4];
   if (kApp == FW_APP_METAPATH) {  // include/app.cuh:141-146
     x[0] = (int32_t)raw.x == want ? 1.0f : 0.0f;
@@ -848,10 +874,19 @@ __device__ __forceinline__ void packed_step(const fw_kargs& a, TaskTable<kWGT, k
   }
 }
 
+template <int kApp, int kSeg, int kWGT>
+__device__ __forceinline__ void packed_step(const fw_kargs& a, TaskTable<kWGT, kApp>& tt, const int lane,
+                                            const int slot, unsigned long long& n_steps,
+                                            unsigned long long& n_edges) {
+  PackedBundle b;
+  packed_load<kApp, kSeg, kWGT>(a, tt, lane, slot, b);
+  packed_finish<kApp, kSeg, kWGT>(a, tt, lane, b, n_steps, n_edges);
+}
+
 // ---- the kernel --------------------------------------------------------------------------------
 
 template <int kApp, int kWGT>
-__global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk_zprs(const fw_kargs a) {
+__global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 4) void fw_walk_zprs(const fw_kargs a) {
   constexpr int kNW = kWGT / 64;
   __shared__ TaskTable<kWGT, kApp> tt;
 
@@ -951,23 +986,30 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 8) void fw_walk
 
       // ---- phase A: remaining slots, claimed dynamically: four or two short lists per wave, else one ----
       if (kApp != FW_APP_NODE2VEC) {
+        // two bundles per turn: their loads are in flight together
         for (;;) {
           int idx = 0;
-          if (lane == 0) idx = atomicAdd(&tt.claim_tiny[parity], 4);
+          if (lane == 0) idx = atomicAdd(&tt.claim_tiny[parity], 8);
           idx = __builtin_amdgcn_readfirstlane(idx);
           if (idx >= nt) break;
-          const int entry = idx + (lane >> 4);
-          const int slot = entry < nt ? (int)tt.tiny_list[parity][entry] : -1;
-          packed_step<kApp, 16, kWGT>(a, tt, lane, slot, n_steps, n_edges);
+          const int e0 = idx + (lane >> 4), e1 = e0 + 4;
+          PackedBundle b0, b1;
+          packed_load<kApp, 16, kWGT>(a, tt, lane, e0 < nt ? (int)tt.tiny_list[parity][e0] : -1, b0);
+          packed_load<kApp, 16, kWGT>(a, tt, lane, e1 < nt ? (int)tt.tiny_list[parity][e1] : -1, b1);
+          packed_finish<kApp, 16, kWGT>(a, tt, lane, b0, n_steps, n_edges);
+          if (idx + 4 < nt) packed_finish<kApp, 16, kWGT>(a, tt, lane, b1, n_steps, n_edges);
         }
         for (;;) {
           int idx = 0;
-          if (lane == 0) idx = atomicAdd(&tt.claim_half[parity], 2);
+          if (lane == 0) idx = atomicAdd(&tt.claim_half[parity], 4);
           idx = __builtin_amdgcn_readfirstlane(idx);
           if (idx >= nf) break;
-          const int entry = idx + (lane >> 5);
-          const int slot = entry < nf ? (int)tt.half_list[parity][entry] : -1;
-          packed_step<kApp, 32, kWGT>(a, tt, lane, slot, n_steps, n_edges);
+          const int e0 = idx + (lane >> 5), e1 = e0 + 2;
+          PackedBundle b0, b1;
+          packed_load<kApp, 32, kWGT>(a, tt, lane, e0 < nf ? (int)tt.half_list[parity][e0] : -1, b0);
+          packed_load<kApp, 32, kWGT>(a, tt, lane, e1 < nf ? (int)tt.half_list[parity][e1] : -1, b1);
+          packed_finish<kApp, 32, kWGT>(a, tt, lane, b0, n_steps, n_edges);
+          if (idx + 2 < nf) packed_finish<kApp, 32, kWGT>(a, tt, lane, b1, n_steps, n_edges);
         }
       }
       for (;;) {
@@ -1807,16 +1849,39 @@ int launch_hub_scan_app(const fw_kargs& a, const fw_hub_args& h, uint32_t tasks_
   return FW_OK;
 }
 
+// Compute units of the current device and workgroups of `kernel` that fit one of them; asked once per kernel and
+// device (the answers do not change, and the questions are slow enough to matter in rounds of 0.3 ms).
+template <typename Kernel>
+int resident_set(Kernel kernel, int wg_threads, int* cus_out, int* per_cu_out) {
+  constexpr int kMaxDevices = 16;
+  static int s_cus[kMaxDevices] = {0};
+  static int s_per_cu[kMaxDevices] = {0};
+  int dev = 0;
+  FW_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices || s_cus[dev] == 0) {
+    int cus = 0, per_cu = 0;
+    FW_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    FW_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, wg_threads, 0));
+    if (per_cu < 1) per_cu = 1;
+    if (dev < 0 || dev >= kMaxDevices) {
+      *cus_out = cus;
+      *per_cu_out = per_cu;
+      return FW_OK;
+    }
+    s_per_cu[dev] = per_cu;
+    s_cus[dev] = cus;
+  }
+  *cus_out = s_cus[dev];
+  *per_cu_out = s_per_cu[dev];
+  return FW_OK;
+}
+
 template <int kApp, int kWGT>
 int launch_hub_one(const fw_kargs& a, const fw_hub_args& h, hipStream_t stream) {
-  int dev = 0;
-  hipDeviceProp_t prop;
-  FW_HIP(hipGetDevice(&dev));
-  FW_HIP(hipGetDeviceProperties(&prop, dev));
-  int per_cu = 0;
-  FW_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fw_hub_batch<kApp, kWGT>, kWGT, 0));
-  if (per_cu < 1) per_cu = 1;
-  const int grid = prop.multiProcessorCount * per_cu;
+  int cus = 0, per_cu = 0;
+  const int rc = resident_set(fw_hub_batch<kApp, kWGT>, kWGT, &cus, &per_cu);
+  if (rc != FW_OK) return rc;
+  const int grid = cus * per_cu;
   hipLaunchKernelGGL((fw_hub_batch<kApp, kWGT>), dim3(grid), dim3(kWGT), 0, stream, a, h);
   FW_HIP(hipGetLastError());
   return FW_OK;
@@ -1834,17 +1899,23 @@ int launch_hub_app(const fw_kargs& a, const fw_hub_args& h, int wg_threads, hipS
   }
 }
 
+// entries_hint (launches of the parking pipeline; 0 otherwise): about how many entries the launch will find.  Their
+// walkers are short-lived (a step or two until they are parked again), so a launch is a few rounds of refills plus
+// a tail of sparse rounds that every workgroup pays; fewer workgroups with kEntriesPerWorkgroup entries each
+// (but at least one per compute unit) spend less on that tail than a full resident set with a few refills each.
+constexpr int kEntriesPerWorkgroup = 4864;
+
 template <int kApp, int kWGT>
-int launch_one(fw_kargs a, int grid, hipStream_t stream, int* grid_used) {
+int launch_one(fw_kargs a, int grid, uint32_t entries_hint, hipStream_t stream, int* grid_used) {
   if (grid <= 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    FW_HIP(hipGetDevice(&dev));
-    FW_HIP(hipGetDeviceProperties(&prop, dev));
-    int per_cu = 0;
-    FW_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fw_walk_zprs<kApp, kWGT>, kWGT, 0));
-    if (per_cu < 1) per_cu = 1;
-    grid = prop.multiProcessorCount * per_cu;
+    int cus = 0, per_cu = 0;
+    const int rc = resident_set(fw_walk_zprs<kApp, kWGT>, kWGT, &cus, &per_cu);
+    if (rc != FW_OK) return rc;
+    grid = cus * per_cu;
+    if (entries_hint != 0u) {
+      const int wanted = (int)(entries_hint / (uint32_t)kEntriesPerWorkgroup);
+      if (wanted < grid) grid = wanted > cus ? wanted : cus;
+    }
   }
   // a small batch is spread over the grid (down to one query per workgroup) instead of filling the
   // task table of a few workgroups: fewer slots per workgroup, same persistent grid
@@ -1858,11 +1929,12 @@ int launch_one(fw_kargs a, int grid, hipStream_t stream, int* grid_used) {
 }
 
 template <int kApp>
-int launch_app(const fw_kargs& a, int wg_threads, int grid, hipStream_t stream, int* grid_used) {
+int launch_app(const fw_kargs& a, int wg_threads, int grid, uint32_t entries_hint, hipStream_t stream,
+               int* grid_used) {
   switch (wg_threads) {
-    case 256: return launch_one<kApp, 256>(a, grid, stream, grid_used);
-    case 512: return launch_one<kApp, 512>(a, grid, stream, grid_used);
-    case 1024: return launch_one<kApp, 1024>(a, grid, stream, grid_used);
+    case 256: return launch_one<kApp, 256>(a, grid, entries_hint, stream, grid_used);
+    case 512: return launch_one<kApp, 512>(a, grid, entries_hint, stream, grid_used);
+    case 1024: return launch_one<kApp, 1024>(a, grid, entries_hint, stream, grid_used);
     default:
       fw_set_error("wg_threads must be 256, 512 or 1024 (got %d)", wg_threads);
       return FW_ERR_INVALID;
@@ -1893,8 +1965,8 @@ int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg
   }
 }
 
-int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, hipStream_t stream,
-                   int* grid_used) {
+int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, uint32_t entries_hint,
+                   hipStream_t stream, int* grid_used) {
   // FW_SAMPLER_DPRS is an alias: the one sampler already evaluates every bias exactly once, which is
   // what the reference's DPRS kernel (include/walker.cuh:1444) exists for.
   if (sampler != FW_SAMPLER_ZPRS && sampler != FW_SAMPLER_DPRS) {
@@ -1902,10 +1974,10 @@ int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int 
     return FW_ERR_INVALID;
   }
   switch (app) {
-    case FW_APP_DEEPWALK: return launch_app<FW_APP_DEEPWALK>(a, wg_threads, grid, stream, grid_used);
-    case FW_APP_PPR: return launch_app<FW_APP_PPR>(a, wg_threads, grid, stream, grid_used);
-    case FW_APP_NODE2VEC: return launch_app<FW_APP_NODE2VEC>(a, wg_threads, grid, stream, grid_used);
-    case FW_APP_METAPATH: return launch_app<FW_APP_METAPATH>(a, wg_threads, grid, stream, grid_used);
+    case FW_APP_DEEPWALK: return launch_app<FW_APP_DEEPWALK>(a, wg_threads, grid, entries_hint, stream, grid_used);
+    case FW_APP_PPR: return launch_app<FW_APP_PPR>(a, wg_threads, grid, entries_hint, stream, grid_used);
+    case FW_APP_NODE2VEC: return launch_app<FW_APP_NODE2VEC>(a, wg_threads, grid, entries_hint, stream, grid_used);
+    case FW_APP_METAPATH: return launch_app<FW_APP_METAPATH>(a, wg_threads, grid, entries_hint, stream, grid_used);
     default:
       fw_set_error("unknown app %d", app);
       return FW_ERR_INVALID;
