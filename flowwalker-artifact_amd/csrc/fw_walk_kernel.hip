@@ -31,6 +31,7 @@
 
 namespace {
 
+constexpr int kPackedInFlight = 4;              // bundles of short lists a wave of the walk kernel loads per turn
 constexpr uint32_t kStreamWave = 0x40000000u;  // workgroup-level combine draw
 constexpr uint32_t kStreamStop = 0x80000000u;  // PPR stop draw
 constexpr int kHubChunk = 32;                  // hub tasks whose wave partials are parked in LDS at once
@@ -986,30 +987,37 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 4) void fw_walk
 
       // ---- phase A: remaining slots, claimed dynamically: four or two short lists per wave, else one ----
       if (kApp != FW_APP_NODE2VEC) {
-        // two bundles per turn: their loads are in flight together
+        // kPackedInFlight bundles per turn: their loads are in flight together, so a wave waits for memory once per
+        // turn instead of once per bundle (the registers are there: two workgroups per CU fit with up to 128)
         for (;;) {
           int idx = 0;
-          if (lane == 0) idx = atomicAdd(&tt.claim_tiny[parity], 8);
+          if (lane == 0) idx = atomicAdd(&tt.claim_tiny[parity], 4 * kPackedInFlight);
           idx = __builtin_amdgcn_readfirstlane(idx);
           if (idx >= nt) break;
-          const int e0 = idx + (lane >> 4), e1 = e0 + 4;
-          PackedBundle b0, b1;
-          packed_load<kApp, 16, kWGT>(a, tt, lane, e0 < nt ? (int)tt.tiny_list[parity][e0] : -1, b0);
-          packed_load<kApp, 16, kWGT>(a, tt, lane, e1 < nt ? (int)tt.tiny_list[parity][e1] : -1, b1);
-          packed_finish<kApp, 16, kWGT>(a, tt, lane, b0, n_steps, n_edges);
-          if (idx + 4 < nt) packed_finish<kApp, 16, kWGT>(a, tt, lane, b1, n_steps, n_edges);
+          PackedBundle b[kPackedInFlight];
+#pragma unroll
+          for (int k = 0; k < kPackedInFlight; ++k) {
+            const int e = idx + 4 * k + (lane >> 4);
+            packed_load<kApp, 16, kWGT>(a, tt, lane, e < nt ? (int)tt.tiny_list[parity][e] : -1, b[k]);
+          }
+#pragma unroll
+          for (int k = 0; k < kPackedInFlight; ++k)
+            if (idx + 4 * k < nt) packed_finish<kApp, 16, kWGT>(a, tt, lane, b[k], n_steps, n_edges);
         }
         for (;;) {
           int idx = 0;
-          if (lane == 0) idx = atomicAdd(&tt.claim_half[parity], 4);
+          if (lane == 0) idx = atomicAdd(&tt.claim_half[parity], 2 * kPackedInFlight);
           idx = __builtin_amdgcn_readfirstlane(idx);
           if (idx >= nf) break;
-          const int e0 = idx + (lane >> 5), e1 = e0 + 2;
-          PackedBundle b0, b1;
-          packed_load<kApp, 32, kWGT>(a, tt, lane, e0 < nf ? (int)tt.half_list[parity][e0] : -1, b0);
-          packed_load<kApp, 32, kWGT>(a, tt, lane, e1 < nf ? (int)tt.half_list[parity][e1] : -1, b1);
-          packed_finish<kApp, 32, kWGT>(a, tt, lane, b0, n_steps, n_edges);
-          if (idx + 2 < nf) packed_finish<kApp, 32, kWGT>(a, tt, lane, b1, n_steps, n_edges);
+          PackedBundle b[kPackedInFlight];
+#pragma unroll
+          for (int k = 0; k < kPackedInFlight; ++k) {
+            const int e = idx + 2 * k + (lane >> 5);
+            packed_load<kApp, 32, kWGT>(a, tt, lane, e < nf ? (int)tt.half_list[parity][e] : -1, b[k]);
+          }
+#pragma unroll
+          for (int k = 0; k < kPackedInFlight; ++k)
+            if (idx + 2 * k < nf) packed_finish<kApp, 32, kWGT>(a, tt, lane, b[k], n_steps, n_edges);
         }
       }
       for (;;) {
