@@ -27,6 +27,7 @@
 // Results depend only on (seed, walker id, graph, parameters): every random draw is addressed by
 // (walker, step, stream, draw index), never by which wave or workgroup happens to run the slot.
 
+#include <mutex>
 #include "fw_internal.h"
 
 namespace {
@@ -1861,26 +1862,36 @@ int launch_hub_scan_app(const fw_kargs& a, const fw_hub_args& h, uint32_t tasks_
 // device (the answers do not change, and the questions are slow enough to matter in rounds of 0.3 ms).
 template <typename Kernel>
 int resident_set(Kernel kernel, int wg_threads, int* cus_out, int* per_cu_out) {
-  constexpr int kMaxDevices = 16;
-  static int s_cus[kMaxDevices] = {0};
-  static int s_per_cu[kMaxDevices] = {0};
+  struct Entry {
+    const void* kernel;
+    int dev, cus, per_cu;
+  };
+  constexpr int kEntries = 64;
+  static Entry s_entries[kEntries];
+  static int s_count = 0;
+  static std::mutex s_lock;
   int dev = 0;
   FW_HIP(hipGetDevice(&dev));
-  if (dev < 0 || dev >= kMaxDevices || s_cus[dev] == 0) {
-    int cus = 0, per_cu = 0;
-    FW_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    FW_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, wg_threads, 0));
-    if (per_cu < 1) per_cu = 1;
-    if (dev < 0 || dev >= kMaxDevices) {
-      *cus_out = cus;
-      *per_cu_out = per_cu;
-      return FW_OK;
-    }
-    s_per_cu[dev] = per_cu;
-    s_cus[dev] = cus;
+  const void* key = reinterpret_cast<const void*>(kernel);
+  {
+    std::lock_guard<std::mutex> guard(s_lock);
+    for (int i = 0; i < s_count; ++i)
+      if (s_entries[i].kernel == key && s_entries[i].dev == dev) {
+        *cus_out = s_entries[i].cus;
+        *per_cu_out = s_entries[i].per_cu;
+        return FW_OK;
+      }
   }
-  *cus_out = s_cus[dev];
-  *per_cu_out = s_per_cu[dev];
+  int cus = 0, per_cu = 0;
+  FW_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  FW_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, wg_threads, 0));
+  if (per_cu < 1) per_cu = 1;
+  {
+    std::lock_guard<std::mutex> guard(s_lock);
+    if (s_count < kEntries) s_entries[s_count++] = Entry{key, dev, cus, per_cu};
+  }
+  *cus_out = cus;
+  *per_cu_out = per_cu;
   return FW_OK;
 }
 
