@@ -32,7 +32,7 @@
 
 namespace {
 
-constexpr int kPackedInFlight = 4;              // bundles of short lists a wave of the walk kernel loads per turn
+constexpr int kPipelineInFlight = 4;            // bundles of short lists a wave loads per turn in launches of the parking pipeline
 constexpr uint32_t kStreamWave = 0x40000000u;  // workgroup-level combine draw
 constexpr uint32_t kStreamStop = 0x80000000u;  // PPR stop draw
 constexpr int kHubChunk = 32;                  // hub tasks whose wave partials are parked in LDS at once
@@ -887,8 +887,13 @@ __device__ __forceinline__ void packed_step(const fw_kargs& a, TaskTable<kWGT, k
 
 // ---- the kernel --------------------------------------------------------------------------------
 
-template <int kApp, int kWGT>
-__global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : 4) void fw_walk_zprs(const fw_kargs a) {
+// kPackedInFlight: bundles of short lists a wave loads per turn.  1 for launches whose walkers run whole walks (80
+// VGPRs, three workgroups of 512 per CU: such launches live on streaming long lists and want every wave they can
+// get); kPipelineInFlight for the launches of the parking pipeline, which are rounds of refills and packed steps
+// on short lists and wait for one bundle's loads after the other otherwise (110 VGPRs, two workgroups per CU).
+template <int kApp, int kWGT, int kPackedInFlight>
+__global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFlight == 1 ? 8 : 4)) void fw_walk_zprs(
+    const fw_kargs a) {
   constexpr int kNW = kWGT / 64;
   __shared__ TaskTable<kWGT, kApp> tt;
 
@@ -1926,9 +1931,14 @@ constexpr int kEntriesPerWorkgroup = 4864;
 
 template <int kApp, int kWGT>
 int launch_one(fw_kargs a, int grid, uint32_t entries_hint, hipStream_t stream, int* grid_used) {
+  // launches of the parking pipeline (they park, or they continue parked walkers) take the variant with several
+  // bundles in flight
+  constexpr int kFlight = kApp == FW_APP_NODE2VEC ? 1 : kPipelineInFlight;
+  const bool pipeline = kFlight != 1 && (a.park_threshold != 0x7FFFFFFF || a.resume != nullptr);
   if (grid <= 0) {
     int cus = 0, per_cu = 0;
-    const int rc = resident_set(fw_walk_zprs<kApp, kWGT>, kWGT, &cus, &per_cu);
+    const int rc = pipeline ? resident_set(fw_walk_zprs<kApp, kWGT, kFlight>, kWGT, &cus, &per_cu)
+                            : resident_set(fw_walk_zprs<kApp, kWGT, 1>, kWGT, &cus, &per_cu);
     if (rc != FW_OK) return rc;
     grid = cus * per_cu;
     if (entries_hint != 0u) {
@@ -1941,7 +1951,10 @@ int launch_one(fw_kargs a, int grid, uint32_t entries_hint, hipStream_t stream, 
   if (grid > a.n) grid = a.n;
   const long long per_wg = ((long long)a.n + grid - 1) / grid;
   a.slot_limit = (int32_t)(per_wg < kWGT ? per_wg : kWGT);
-  hipLaunchKernelGGL((fw_walk_zprs<kApp, kWGT>), dim3(grid), dim3(kWGT), 0, stream, a);
+  if (pipeline)
+    hipLaunchKernelGGL((fw_walk_zprs<kApp, kWGT, kFlight>), dim3(grid), dim3(kWGT), 0, stream, a);
+  else
+    hipLaunchKernelGGL((fw_walk_zprs<kApp, kWGT, 1>), dim3(grid), dim3(kWGT), 0, stream, a);
   FW_HIP(hipGetLastError());
   if (grid_used) *grid_used = grid;
   return FW_OK;
