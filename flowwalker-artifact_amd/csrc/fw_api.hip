@@ -523,7 +523,7 @@ constexpr int kParkCtrs = 16;                    // counters of a parking round
 // is served in two passes (scan tasks of up to kScanRun groups that make the list's rows, one table task per 64
 // walkers); every other bucket gets one batch task per 64 walkers:
 // a workgroup task when its vertex is sampled at workgroup granularity (degree above hub_threshold), a wave task
-// otherwise.  ctrs (out): [3] workgroup tasks, [5] wave tasks, [7] table tasks, [8] scan tasks,
+// otherwise.  ctrs (out): [3] workgroup tasks, [4] their dispenser, [5] wave tasks, [7] table tasks, [8] scan tasks,
 // [12] walkers in the fullest bucket when that is more than half of kTwoPassWalkers.
 constexpr uint32_t kScanRun = 16;
 
@@ -935,6 +935,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   h.tasks = pb->tasks;
   h.ntasks = &pb->ctrs[3];
   h.task_next = &pb->ctrs[4];
+  h.dynamic_wgs = 0u;
   h.wtasks = pb->wtasks;
   h.nwtasks = &pb->ctrs[5];
   h.out = pb->out;
@@ -998,6 +999,8 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   uint32_t fullest = 0;  // walkers in the fullest bucket of the previous round
   uint32_t scan_tasks = 0;  // and its scan tasks
   uint32_t resumed = 0;     // and the walkers that went on in its walk launch
+  uint32_t batch_tasks = 0; // and its batch tasks, in waves
+  uint32_t wg_task_waves = 0;  // of which workgroup tasks
   for (;;) {
     // one round: the walkers parked by the last walk launch and by the last batch launch are grouped by bucket, the
     // batch launch moves each of them one step, and the walk launch queued right behind it takes those that are
@@ -1055,7 +1058,12 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
       rc = fw_launch_hub_scan(a, h, p->app, n_out != 0u ? scan_tasks * 4u + 1u : 0u, stream);
       if (rc != FW_OK) return rc;
     }
-    rc = fw_launch_hub_batch(a, h, p->app, p->wg_threads, stream);
+    // The grid follows the number of tasks: about as many as a round ago, scaled by the walkers (the first round
+    // has nothing to go by and takes one resident set).  Not when workgroup tasks are more than a sixteenth of the
+    // work: an oversized grid puts them behind all wave tasks, and they are better spread among those.
+    uint32_t tasks_hint = n_out != 0u ? (uint32_t)((uint64_t)batch_tasks * m / n_out) + 1u : 0u;
+    if ((uint64_t)wg_task_waves * 16u > batch_tasks) tasks_hint = 0u;
+    rc = fw_launch_hub_batch(a, h, p->app, p->wg_threads, tasks_hint, stream);
     if (rc != FW_OK) return rc;
     if ((rc = th.end(stream)) != FW_OK) return rc;
     ++*launches;
@@ -1084,6 +1092,8 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     n_out = (uint32_t)m;
     fullest = pb->h_ctrs[12];
     resumed = pb->h_ctrs[6];
+    wg_task_waves = pb->h_ctrs[3] * (uint32_t)(p->wg_threads / 64);
+    batch_tasks = pb->h_ctrs[5] + pb->h_ctrs[7] + wg_task_waves;
     scan_tasks = pb->h_ctrs[8];
     cur = nxt;
   }

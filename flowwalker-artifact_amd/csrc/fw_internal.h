@@ -99,9 +99,10 @@ struct fw_batch_task {
 // by a workgroup (degree above hub_threshold: workgroup-granularity sampling) or by a single wave.
 struct fw_hub_args {
   const fw_walker_rec* sorted;       // parked records grouped by bucket
-  const fw_batch_task* tasks;        // workgroup tasks, handed out through task_next
-  const uint32_t* ntasks;
+  const fw_batch_task* tasks;        // workgroup tasks, handed out through task_next to the last dynamic_wgs workgroups
   uint32_t* task_next;
+  uint32_t dynamic_wgs;              // set by the launch: the workgroups of one resident set
+  const uint32_t* ntasks;
   const fw_batch_task* wtasks;       // wave tasks, wave i of the grid takes i, i + waves, ...
   const uint32_t* nwtasks;
   // out[rec_base + i] = walker i of the batch after its step: q = -1 when its walk is over, len tagged with
@@ -177,8 +178,10 @@ int fw_check_hip(hipError_t e, const char* what, const char* file, int line);
 int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, uint32_t entries_hint,
                    hipStream_t stream, int* grid_used);
 
-// Launches the hub batch kernel (persistent grid, tasks taken from h.task_next).
-int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, hipStream_t stream);
+// Launches the hub batch kernel.  tasks_hint: about how many wave-sized pieces of work it will find (sizes the grid;
+// 0 = no idea: one resident set).
+int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, uint32_t tasks_hint,
+                        hipStream_t stream);
 // Launches the scan kernel of the two-pass steps (it finds its task count in h.nstasks on the device).
 // tasks_hint: about how many scan tasks to expect, to size the grid (0 = no idea: a full resident set).
 int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, uint32_t tasks_hint, hipStream_t stream);

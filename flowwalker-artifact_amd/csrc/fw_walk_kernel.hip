@@ -1745,9 +1745,13 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, have, sel, walker, step, lane, n_steps, n_edges, n_out);
   }
 
-  // ---- then workgroup tasks: lists above hub_threshold, sampled at workgroup granularity.  They are handed out
-  //      dynamically, which evens out what the fixed deal of the wave tasks left uneven ----
+  // ---- then workgroup tasks: lists above hub_threshold, sampled at workgroup granularity.  They are few, long and
+  //      uneven, so they are handed out through a counter -- to the last resident set of workgroups only: the
+  //      rest of an oversized grid exists to even out the wave tasks (one counter update per workgroup of it
+  //      would cost more than these tasks), and the workgroups that start last hold nobody up while they work
+  //      through long lists ----
   for (;;) {
+    if (blockIdx.x + h.dynamic_wgs < gridDim.x) break;
     if (tid == 0) s_task = atomicAdd(h.task_next, 1u);
     __syncthreads();
     const uint32_t t = s_task;
@@ -1900,23 +1904,36 @@ int resident_set(Kernel kernel, int wg_threads, int* cus_out, int* per_cu_out) {
   return FW_OK;
 }
 
+// tasks_hint: about how many wave-sized pieces of work the launch will find (wave tasks + table tasks + waves of
+// workgroup tasks; 0 = no idea).  All tasks are dealt out by position, so the grid may be larger than what is
+// resident: the hardware then starts a workgroup wherever one has finished, which evens out the uneven shares
+// without any counter.  About kTasksPerWave tasks per wave, between one and eight resident sets.
+constexpr uint32_t kTasksPerWave = 8;
+
 template <int kApp, int kWGT>
-int launch_hub_one(const fw_kargs& a, const fw_hub_args& h, hipStream_t stream) {
+int launch_hub_one(const fw_kargs& a, const fw_hub_args& h, uint32_t tasks_hint, hipStream_t stream) {
   int cus = 0, per_cu = 0;
   const int rc = resident_set(fw_hub_batch<kApp, kWGT>, kWGT, &cus, &per_cu);
   if (rc != FW_OK) return rc;
-  const int grid = cus * per_cu;
-  hipLaunchKernelGGL((fw_hub_batch<kApp, kWGT>), dim3(grid), dim3(kWGT), 0, stream, a, h);
+  const int resident = cus * per_cu;
+  fw_hub_args hh = h;
+  hh.dynamic_wgs = (uint32_t)resident;
+  int grid = resident;
+  if (tasks_hint != 0u) {
+    const uint32_t wanted = tasks_hint / ((uint32_t)(kWGT / 64) * kTasksPerWave);
+    if (wanted > (uint32_t)grid) grid = wanted < 8u * (uint32_t)resident ? (int)wanted : 8 * resident;
+  }
+  hipLaunchKernelGGL((fw_hub_batch<kApp, kWGT>), dim3(grid), dim3(kWGT), 0, stream, a, hh);
   FW_HIP(hipGetLastError());
   return FW_OK;
 }
 
 template <int kApp>
-int launch_hub_app(const fw_kargs& a, const fw_hub_args& h, int wg_threads, hipStream_t stream) {
+int launch_hub_app(const fw_kargs& a, const fw_hub_args& h, int wg_threads, uint32_t tasks_hint, hipStream_t stream) {
   switch (wg_threads) {
-    case 256: return launch_hub_one<kApp, 256>(a, h, stream);
-    case 512: return launch_hub_one<kApp, 512>(a, h, stream);
-    case 1024: return launch_hub_one<kApp, 1024>(a, h, stream);
+    case 256: return launch_hub_one<kApp, 256>(a, h, tasks_hint, stream);
+    case 512: return launch_hub_one<kApp, 512>(a, h, tasks_hint, stream);
+    case 1024: return launch_hub_one<kApp, 1024>(a, h, tasks_hint, stream);
     default:
       fw_set_error("wg_threads must be 256, 512 or 1024 (got %d)", wg_threads);
       return FW_ERR_INVALID;
@@ -1986,11 +2003,12 @@ int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, uint32_
   }
 }
 
-int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, hipStream_t stream) {
+int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, uint32_t tasks_hint,
+                        hipStream_t stream) {
   switch (app) {
-    case FW_APP_DEEPWALK: return launch_hub_app<FW_APP_DEEPWALK>(a, h, wg_threads, stream);
-    case FW_APP_PPR: return launch_hub_app<FW_APP_PPR>(a, h, wg_threads, stream);
-    case FW_APP_METAPATH: return launch_hub_app<FW_APP_METAPATH>(a, h, wg_threads, stream);
+    case FW_APP_DEEPWALK: return launch_hub_app<FW_APP_DEEPWALK>(a, h, wg_threads, tasks_hint, stream);
+    case FW_APP_PPR: return launch_hub_app<FW_APP_PPR>(a, h, wg_threads, tasks_hint, stream);
+    case FW_APP_METAPATH: return launch_hub_app<FW_APP_METAPATH>(a, h, wg_threads, tasks_hint, stream);
     default:
       fw_set_error("the hub batch kernel serves DeepWalk, PPR and MetaPath (node2vec biases depend on the walker)");
       return FW_ERR_INVALID;
