@@ -41,7 +41,7 @@ HEADLINE = "deepwalk_rmat24_sym"
 # HBM-side bytes of one pass (all launches of the walk pipeline) from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs, each scaled by what the same counter reads for the 1 GiB copy kernel (profiles/).
 # None for workloads that have not been measured.
-MEASURED_TRAFFIC_BYTES = {"deepwalk_rmat24_sym": 5.89e11}
+MEASURED_TRAFFIC_BYTES = {"deepwalk_rmat24_sym": 5.73e11}
 
 
 def algorithmic_bytes(app, steps, sampled_edges, queries, probe_terms=0):
