@@ -4,14 +4,21 @@
 //   flowwalker --input PREFIX (--deepwalk | --ppr | --node2vec | --metapath)
 //              [--n N | --all] [--seq] [--d D] [--batch] [--batchsize B] [--autobatch] [--headroom MB] [--syn]
 //              [--tp T] [--p P] [--q Q] [--schema 0,1,2] [--dprs] [--printresult] [--printworkload]
-//              [--seed S] [--pprstart maxdeg|seq] [--hub_threshold T] [--wg_threads W] [--savepaths FILE]
+//              [--seed S] [--pprstart maxdeg|seq] [--hub_threshold T] [--wg_threads W] [--park_threshold P]
+//              [--walkmode M] [--savepaths FILE]
 //
 // Flags follow gflags syntax: --flag, --flag=value, --flag value, --noflag.  Differences from the
 // reference, on purpose: random start vertices come from --seed instead of time(NULL) (src/main.cu:284),
 // the first min(100, n) walkers are printed (the reference always prints 100 and reads out of bounds for
 // smaller n: src/main.cu:165), errors return a non-zero status with a message instead of exit() inside a
-// macro, --lognorm draws its weights from a seeded host generator, and --walkmode / --umgraph (ablation and
-// out-of-core switches) are accepted and ignored with a note.
+// macro, --lognorm draws its weights from a seeded host generator, --umgraph (out-of-core graphs) is accepted
+// and ignored with a note, and --walkmode selects the ablation levels of THIS engine (the reference's levels,
+// README.md:152-163, name optimisations of its CUDA kernels that have no counterpart here):
+//   --walkmode=9 / 10  the walk kernel alone, every list sampled by one wave (no workgroup sampler, no parking;
+//                      the counter-based RNG has one form, so 9 and 10 are the same)
+//   --walkmode=1       + the workgroup sampler for lists above --hub_threshold
+//   --walkmode=6       + parking: walkers waiting on the same vertex share one scan of its list (the default)
+// --park_threshold passes fw_walk_params.park_threshold through (0 library rule, < 0 off, > 0 explicit degree).
 
 #include <stdint.h>
 #include <stdio.h>
@@ -52,6 +59,7 @@ struct Flags {
   std::string pprstart = "maxdeg";
   int hub_threshold = -1;
   int wg_threads = 0;
+  int park_threshold = 0;
   std::string savepaths;
 };
 
@@ -81,6 +89,7 @@ bool parse_flags(int argc, char** argv, Flags* f) {
       {"lognorm", {kBool, &f->lognorm}},     {"seed", {kLong, &f->seed}},
       {"pprstart", {kString, &f->pprstart}}, {"hub_threshold", {kInt, &f->hub_threshold}},
       {"wg_threads", {kInt, &f->wg_threads}}, {"savepaths", {kString, &f->savepaths}},
+      {"park_threshold", {kInt, &f->park_threshold}},
   };
   for (int i = 1; i < argc; ++i) {
     std::string arg = argv[i];
@@ -195,9 +204,10 @@ int main(int argc, char** argv) {
          "------------------------------------\n");
   Flags F;
   if (!parse_flags(argc, argv, &F)) return 2;
-  for (const char* ignored : {"walkmode", "umgraph"}) {
-    const bool set = (!strcmp(ignored, "walkmode") && F.walkmode >= 0) || (!strcmp(ignored, "umgraph") && F.umgraph);
-    if (set) fprintf(stderr, "flowwalker: --%s selects an ablation / debug mode that this build does not have; ignored\n", ignored);
+  if (F.umgraph) fprintf(stderr, "flowwalker: --umgraph (out-of-core graphs) is not part of this build; ignored\n");
+  if (F.walkmode >= 0 && F.walkmode != 1 && F.walkmode != 6 && F.walkmode != 9 && F.walkmode != 10) {
+    fprintf(stderr, "flowwalker: --walkmode must be 9, 10, 1 or 6 (ablation levels); %d ignored\n", F.walkmode);
+    F.walkmode = -1;
   }
   if (!(F.deepwalk || F.ppr || F.node2vec || F.metapath)) {  // src/walk.cu:565-568
     printf("Please choose a walk mode\n");
@@ -303,6 +313,14 @@ int main(int argc, char** argv) {
   P.seed = (uint64_t)F.seed;
   if (F.hub_threshold >= 0) P.hub_threshold = F.hub_threshold;
   if (F.wg_threads > 0) P.wg_threads = F.wg_threads;
+  P.park_threshold = F.park_threshold;
+  if (F.walkmode >= 0) {  // ablation levels, lowest first
+    if (F.walkmode == 9 || F.walkmode == 10) P.hub_threshold = 0x7FFFFFFF;
+    if (F.walkmode != 6) P.park_threshold = -1;
+    printf("ablation level %d: %s\n", F.walkmode,
+           F.walkmode == 6 ? "workgroup sampler and parking (the full engine)"
+                           : F.walkmode == 1 ? "workgroup sampler, no parking" : "wave sampler only, no parking");
+  }
 
   // ---- walk (src/main.cu:346-357) ----
   int32_t* paths = nullptr;

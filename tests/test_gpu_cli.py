@@ -136,3 +136,27 @@ def test_save_degree_and_lognorm(gpu, graph_files, tmp_path):
             if row[j] < 0:
                 break
             assert row[j] in adj[xadj[row[j - 1]]:xadj[row[j - 1] + 1]]
+
+
+def test_ablation_levels_and_park_threshold(gpu, graph_files, tmp_path):
+    """--walkmode selects this engine's ablation levels (README.md:152-163 of the reference names its own): 9 / 10
+    the wave sampler alone, 1 adds the workgroup sampler, 6 adds parking.  Parking never changes a path, the
+    sampler's granularity is part of the sampling definition; every level equals the oracle run with its settings."""
+    prefix, csr = graph_files
+    V = len(csr[0]) - 1
+    starts = np.arange(V, dtype=np.int32)
+    og = orc.Graph(*csr)
+    ref_wg, _, _ = orc.walk(og, orc.make_params(max_depth=11, seed=3, hub_threshold=1000), starts)
+    ref_wave, _, _ = orc.walk(og, orc.make_params(max_depth=11, seed=3, hub_threshold=0x7FFFFFFF), starts)
+    for mode, ref, note in ((9, ref_wave, "wave sampler only"), (10, ref_wave, "wave sampler only"),
+                            (1, ref_wg, "no parking"), (6, ref_wg, "full engine")):
+        out = str(tmp_path / ("m%d.bin" % mode))
+        text = _run("--input", prefix, "--deepwalk", "--all", "--d=10", "--seed=3", "--hub_threshold=1000",
+                    "--walkmode=%d" % mode, "--savepaths", out)
+        assert "ablation level %d" % mode in text and note in text
+        assert (np.fromfile(out, dtype=np.int32).reshape(V, 11) == ref).all(), mode
+    for park in (-1, 50):
+        out = str(tmp_path / ("k%d.bin" % park))
+        _run("--input", prefix, "--deepwalk", "--all", "--d=10", "--seed=3", "--hub_threshold=1000",
+             "--park_threshold=%d" % park, "--savepaths", out)
+        assert (np.fromfile(out, dtype=np.int32).reshape(V, 11) == ref_wg).all(), park
