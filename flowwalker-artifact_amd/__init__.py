@@ -20,6 +20,7 @@ FW_MAX_SCHEMA = 64
 APP_DEEPWALK, APP_PPR, APP_NODE2VEC, APP_METAPATH = 0, 1, 2, 3
 SAMPLER_ZPRS, SAMPLER_DPRS = 0, 1
 FW_OK = 0
+GRAPH_DEVICE, GRAPH_HOST_PINNED = 0, 1
 
 # every symbol include/flowwalker.h declares
 EXPORTED = [
@@ -28,6 +29,7 @@ EXPORTED = [
     "fw_graph_create", "fw_graph_adopt_device", "fw_graph_destroy", "fw_graph_info", "fw_graph_is_sorted",
     "fw_graph_download", "fw_walk_device", "fw_walk_batch", "fw_host_alloc_pinned", "fw_host_free_pinned",
     "fw_gen_rmat", "fw_csr_read_header", "fw_csr_load", "fw_csr_write", "fw_graph_load",
+    "fw_graph_create_placed", "fw_graph_load_placed",
 ]
 
 
@@ -88,6 +90,8 @@ def lib():
         L.fw_dev_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         L.fw_graph_create.argtypes = [C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.POINTER(C.c_void_p)]
+        L.fw_graph_create_placed.argtypes = [C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                             C.c_int, C.POINTER(C.c_void_p)]
         L.fw_graph_adopt_device.argtypes = [C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                             C.c_int, C.POINTER(C.c_void_p)]
         L.fw_graph_destroy.argtypes = [C.c_void_p]
@@ -106,6 +110,7 @@ def lib():
         L.fw_csr_load.argtypes = [C.c_char_p, C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.fw_csr_write.argtypes = [C.c_char_p, C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.fw_graph_load.argtypes = [C.c_char_p, C.c_int, C.c_int, C.POINTER(C.c_void_p)]
+        L.fw_graph_load_placed.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p)]
         _lib = L
     return _lib
 
@@ -215,20 +220,20 @@ class Graph:
         self.V, self.E = V.value, E.value
 
     @classmethod
-    def from_csr(cls, xadj, adjncy, weight=None, label=None):
+    def from_csr(cls, xadj, adjncy, weight=None, label=None, placement=GRAPH_DEVICE):
         xadj = np.ascontiguousarray(xadj, dtype=np.uint32)
         adjncy = np.ascontiguousarray(adjncy, dtype=np.int32)
         weight = None if weight is None else np.ascontiguousarray(weight, dtype=np.float32)
         label = None if label is None else np.ascontiguousarray(label, dtype=np.int32)
         h = C.c_void_p()
-        check(lib().fw_graph_create(len(xadj) - 1, len(adjncy), _ptr(xadj), _ptr(adjncy), _ptr(weight), _ptr(label),
-                                    C.byref(h)))
+        check(lib().fw_graph_create_placed(len(xadj) - 1, len(adjncy), _ptr(xadj), _ptr(adjncy), _ptr(weight),
+                                           _ptr(label), placement, C.byref(h)))
         return cls(h)
 
     @classmethod
-    def load(cls, prefix, weights=True, labels=False):
+    def load(cls, prefix, weights=True, labels=False, placement=GRAPH_DEVICE):
         h = C.c_void_p()
-        check(lib().fw_graph_load(prefix.encode(), int(weights), int(labels), C.byref(h)))
+        check(lib().fw_graph_load_placed(prefix.encode(), int(weights), int(labels), placement, C.byref(h)))
         return cls(h)
 
     @classmethod

@@ -205,11 +205,20 @@ static int validate_csr_host(int32_t V, uint64_t E, const uint32_t* xadj, const 
   return FW_OK;
 }
 
+// One edge array with FW_EDGE_PAD zeroed elements behind it, filled from the host copy.  In pinned host memory the
+// array is mapped into the device's address space: the kernels use the same pointer and every read crosses the bus.
 template <typename T>
-static int alloc_edge_array(T** out, uint64_t E) {
+static int alloc_edge_array(T** out, uint64_t E, const T* h_src, int host_pinned) {
   const size_t bytes = (size_t)(E + FW_EDGE_PAD) * sizeof(T);
+  if (host_pinned) {
+    FW_HIP(hipHostMalloc(reinterpret_cast<void**>(out), bytes, hipHostMallocDefault));
+    memcpy(*out, h_src, (size_t)E * sizeof(T));
+    memset(reinterpret_cast<char*>(*out) + (size_t)E * sizeof(T), 0, FW_EDGE_PAD * sizeof(T));
+    return FW_OK;
+  }
   FW_HIP(hipMalloc(reinterpret_cast<void**>(out), bytes));
   FW_HIP(hipMemset(reinterpret_cast<char*>(*out) + (size_t)E * sizeof(T), 0, FW_EDGE_PAD * sizeof(T)));
+  FW_HIP(hipMemcpy(*out, h_src, (size_t)E * sizeof(T), hipMemcpyHostToDevice));
   return FW_OK;
 }
 
@@ -219,9 +228,10 @@ extern "C" int fw_graph_destroy(fw_graph* g) {
   if (!g) return FW_OK;
   int rc = FW_OK;
   if (g->owns) {
-    void* ptrs[4] = {g->xadj, g->adjncy, g->weight, g->label};
+    if (g->xadj && hipFree(g->xadj) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
+    void* ptrs[3] = {g->adjncy, g->weight, g->label};
     for (void* p : ptrs) {
-      if (p && hipFree(p) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
+      if (p && (g->host_edges ? hipHostFree(p) : hipFree(p)) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
     }
   }
   release_park_cache(g);
@@ -233,10 +243,14 @@ extern "C" int fw_graph_destroy(fw_graph* g) {
   return rc;
 }
 
-extern "C" int fw_graph_create(int32_t V, uint64_t E, const uint32_t* h_xadj, const int32_t* h_adjncy,
-                               const float* h_weight, const int32_t* h_label, fw_graph** out) {
+extern "C" int fw_graph_create_placed(int32_t V, uint64_t E, const uint32_t* h_xadj, const int32_t* h_adjncy,
+                                      const float* h_weight, const int32_t* h_label, int placement, fw_graph** out) {
   if (!out) { fw_set_error("fw_graph_create: out is NULL"); return FW_ERR_INVALID; }
   *out = nullptr;
+  if (placement != FW_GRAPH_DEVICE && placement != FW_GRAPH_HOST_PINNED) {
+    fw_set_error("fw_graph_create_placed: unknown placement %d", placement);
+    return FW_ERR_INVALID;
+  }
   int rc = validate_csr_host(V, E, h_xadj, h_adjncy, h_weight);
   if (rc != FW_OK) return rc;
   rc = require_device();
@@ -246,23 +260,22 @@ extern "C" int fw_graph_create(int32_t V, uint64_t E, const uint32_t* h_xadj, co
   g->V = V;
   g->E = E;
   g->owns = 1;
+  g->host_edges = placement == FW_GRAPH_HOST_PINNED;
   auto fail = [&](int code) { fw_graph_destroy(g); return code; };
   if (hipGetDevice(&g->device) != hipSuccess) return fail(FW_ERR_HIP);
   const size_t xbytes = (size_t)(V + 1) * sizeof(uint32_t);
   if ((rc = fw_check_hip(hipMalloc(reinterpret_cast<void**>(&g->xadj), xbytes), "hipMalloc(xadj)", __FILE__, __LINE__))) return fail(rc);
   if ((rc = fw_check_hip(hipMemcpy(g->xadj, h_xadj, xbytes, hipMemcpyHostToDevice), "hipMemcpy(xadj)", __FILE__, __LINE__))) return fail(rc);
-  if ((rc = alloc_edge_array(&g->adjncy, E))) return fail(rc);
-  if ((rc = fw_check_hip(hipMemcpy(g->adjncy, h_adjncy, (size_t)E * 4, hipMemcpyHostToDevice), "hipMemcpy(adjncy)", __FILE__, __LINE__))) return fail(rc);
-  if (h_weight) {
-    if ((rc = alloc_edge_array(&g->weight, E))) return fail(rc);
-    if ((rc = fw_check_hip(hipMemcpy(g->weight, h_weight, (size_t)E * 4, hipMemcpyHostToDevice), "hipMemcpy(weight)", __FILE__, __LINE__))) return fail(rc);
-  }
-  if (h_label) {
-    if ((rc = alloc_edge_array(&g->label, E))) return fail(rc);
-    if ((rc = fw_check_hip(hipMemcpy(g->label, h_label, (size_t)E * 4, hipMemcpyHostToDevice), "hipMemcpy(label)", __FILE__, __LINE__))) return fail(rc);
-  }
+  if ((rc = alloc_edge_array(&g->adjncy, E, h_adjncy, g->host_edges))) return fail(rc);
+  if (h_weight && (rc = alloc_edge_array(&g->weight, E, h_weight, g->host_edges))) return fail(rc);
+  if (h_label && (rc = alloc_edge_array(&g->label, E, h_label, g->host_edges))) return fail(rc);
   *out = g;
   return FW_OK;
+}
+
+extern "C" int fw_graph_create(int32_t V, uint64_t E, const uint32_t* h_xadj, const int32_t* h_adjncy,
+                               const float* h_weight, const int32_t* h_label, fw_graph** out) {
+  return fw_graph_create_placed(V, E, h_xadj, h_adjncy, h_weight, h_label, FW_GRAPH_DEVICE, out);
 }
 
 extern "C" int fw_graph_adopt_device(int32_t V, uint64_t E, uint32_t* d_xadj, int32_t* d_adjncy, float* d_weight,
@@ -357,14 +370,15 @@ extern "C" int fw_graph_download(const fw_graph* g, uint32_t* h_xadj, int32_t* h
                                  int32_t* h_label) {
   if (!g) { fw_set_error("fw_graph_download: graph is NULL"); return FW_ERR_INVALID; }
   if (h_xadj) FW_HIP(hipMemcpy(h_xadj, g->xadj, (size_t)(g->V + 1) * 4, hipMemcpyDeviceToHost));
-  if (h_adjncy) FW_HIP(hipMemcpy(h_adjncy, g->adjncy, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+  const hipMemcpyKind edge_kind = g->host_edges ? hipMemcpyHostToHost : hipMemcpyDeviceToHost;
+  if (h_adjncy) FW_HIP(hipMemcpy(h_adjncy, g->adjncy, (size_t)g->E * 4, edge_kind));
   if (h_weight) {
     if (!g->weight) { fw_set_error("graph has no weights"); return FW_ERR_INVALID; }
-    FW_HIP(hipMemcpy(h_weight, g->weight, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+    FW_HIP(hipMemcpy(h_weight, g->weight, (size_t)g->E * 4, edge_kind));
   }
   if (h_label) {
     if (!g->label) { fw_set_error("graph has no labels"); return FW_ERR_INVALID; }
-    FW_HIP(hipMemcpy(h_label, g->label, (size_t)g->E * 4, hipMemcpyDeviceToHost));
+    FW_HIP(hipMemcpy(h_label, g->label, (size_t)g->E * 4, edge_kind));
   }
   return FW_OK;
 }
@@ -511,11 +525,13 @@ static int ensure_hub_index(fw_graph* g, int32_t threshold) {
 // Default parking rule (batches of at least kMinParkBatch queries): park on vertices where about kParkMeet or more
 // walkers of the batch stand at the same time.  With n walkers spread in proportion to degree over E adjacency
 // entries, a vertex of degree d holds about n * d / E of them, so the threshold is kParkMeet * E / n, not below
-// kMinDefaultPark (shorter lists cost less to read than a record costs to move).
+// kMinDefaultPark (shorter lists cost less to read than a record costs to move).  Edge arrays in host memory are
+// read over the bus, where every shared read counts: vertices where one walker is expected, not below kMinHostPark.
 constexpr int32_t kMinParkBatch = 65536;
 constexpr uint32_t kParkTail = 32768;  // fewer walkers than this finish in one walk launch without parking
 constexpr double kParkMeet = 4.0;
 constexpr int32_t kMinDefaultPark = 64;
+constexpr int32_t kMinHostPark = 16;
 constexpr int32_t kMinParkThreshold = 1;
 constexpr int kParkCtrs = 16;                    // counters of a parking round
 
@@ -882,9 +898,10 @@ static int32_t resolve_park_threshold(const fw_graph* g, const fw_walk_params* p
   if (p->park_threshold < 0) return INT_MAX;
   if (p->park_threshold == 0) {
     if (n < kMinParkBatch) return INT_MAX;  // too few walkers to meet
-    const double t = kParkMeet * (double)g->E / (double)n;
+    const double t = (g->host_edges ? 1.0 : kParkMeet) * (double)g->E / (double)n;
     if (t >= 2.0e9) return INT_MAX;
-    return t < (double)kMinDefaultPark ? kMinDefaultPark : (int32_t)t;
+    const int32_t floor_deg = g->host_edges ? kMinHostPark : kMinDefaultPark;
+    return t < (double)floor_deg ? floor_deg : (int32_t)t;
   }
   return p->park_threshold < kMinParkThreshold ? kMinParkThreshold : p->park_threshold;
 }

@@ -115,6 +115,11 @@ extern "C" int fw_csr_write(const char* prefix, int32_t V, uint64_t E, const uin
 }
 
 extern "C" int fw_graph_load(const char* prefix, int want_weight, int want_label, fw_graph** out) {
+  return fw_graph_load_placed(prefix, want_weight, want_label, FW_GRAPH_DEVICE, out);
+}
+
+extern "C" int fw_graph_load_placed(const char* prefix, int want_weight, int want_label, int placement,
+                                    fw_graph** out) {
   if (!out) { fw_set_error("fw_graph_load: out is NULL"); return FW_ERR_INVALID; }
   *out = nullptr;
   int32_t V = 0;
@@ -128,6 +133,6 @@ extern "C" int fw_graph_load(const char* prefix, int want_weight, int want_label
   rc = fw_csr_load(prefix, V, E, xadj.data(), adj.data(), want_weight ? w.data() : nullptr,
                    want_label ? lab.data() : nullptr);
   if (rc != FW_OK) return rc;
-  return fw_graph_create(V, E, xadj.data(), adj.data(), want_weight ? w.data() : nullptr,
-                         want_label ? lab.data() : nullptr, out);
+  return fw_graph_create_placed(V, E, xadj.data(), adj.data(), want_weight ? w.data() : nullptr,
+                                want_label ? lab.data() : nullptr, placement, out);
 }

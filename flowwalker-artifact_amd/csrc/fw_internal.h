@@ -25,6 +25,7 @@ struct fw_graph {
   float* weight = nullptr;
   int32_t* label = nullptr;
   int owns = 1;
+  int host_edges = 0;  // edge arrays live in pinned host memory (FW_GRAPH_HOST_PINNED) and are read over the bus
   int device = 0;
   int32_t max_degree = -1;  // lazily computed
   int32_t max_degree_vertex = -1;

@@ -11,8 +11,9 @@
 // reference, on purpose: random start vertices come from --seed instead of time(NULL) (src/main.cu:284),
 // the first min(100, n) walkers are printed (the reference always prints 100 and reads out of bounds for
 // smaller n: src/main.cu:165), errors return a non-zero status with a message instead of exit() inside a
-// macro, --lognorm draws its weights from a seeded host generator, --umgraph (out-of-core graphs) is accepted
-// and ignored with a note, and --walkmode selects the ablation levels of THIS engine (the reference's levels,
+// macro, --lognorm draws its weights from a seeded host generator, --umgraph keeps the edge arrays in pinned host
+// memory that the kernels read over the bus (the reference uses managed memory that migrates by page,
+// include/gpu_graph.cuh:46-54), and --walkmode selects the ablation levels of THIS engine (the reference's levels,
 // README.md:152-163, name optimisations of its CUDA kernels that have no counterpart here):
 //   --walkmode=9 / 10  the walk kernel alone, every list sampled by one wave (no workgroup sampler, no parking;
 //                      the counter-based RNG has one form, so 9 and 10 are the same)
@@ -204,7 +205,7 @@ int main(int argc, char** argv) {
          "------------------------------------\n");
   Flags F;
   if (!parse_flags(argc, argv, &F)) return 2;
-  if (F.umgraph) fprintf(stderr, "flowwalker: --umgraph (out-of-core graphs) is not part of this build; ignored\n");
+  if (F.umgraph) printf("umgraph: edge arrays stay in pinned host memory and are read over the bus\n");
   if (F.walkmode >= 0 && F.walkmode != 1 && F.walkmode != 6 && F.walkmode != 9 && F.walkmode != 10) {
     fprintf(stderr, "flowwalker: --walkmode must be 9, 10, 1 or 6 (ablation levels); %d ignored\n", F.walkmode);
     F.walkmode = -1;
@@ -247,8 +248,9 @@ int main(int argc, char** argv) {
   }
   printf("Max degree: %d, idx: %d\n", max_deg, max_idx);
   fw_graph* g = nullptr;
-  if (fw_graph_create(V, E, xadj.data(), adjncy.data(), F.metapath ? nullptr : weight.data(),
-                      F.metapath ? label.data() : nullptr, &g) != FW_OK)
+  if (fw_graph_create_placed(V, E, xadj.data(), adjncy.data(), F.metapath ? nullptr : weight.data(),
+                             F.metapath ? label.data() : nullptr, F.umgraph ? FW_GRAPH_HOST_PINNED : FW_GRAPH_DEVICE,
+                             &g) != FW_OK)
     return fail("uploading the graph");
   if (F.node2vec) {  // the adjacency test binary-searches neighbour lists (include/gpu_graph.cuh:97-118)
     int sorted = 0;

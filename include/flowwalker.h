@@ -128,6 +128,19 @@ int fw_graph_create(int32_t V, uint64_t E, const uint32_t* h_xadj, const int32_t
                     const float* h_weight, const int32_t* h_label, fw_graph** out);
 
 /*
+ * Where the edge arrays (adjncy, weight, label) of a graph live.  Replaces FLAGS_umgraph
+ * (src/main.cu:48, include/gpu_graph.cuh:46-54: cudaMallocManaged instead of cudaMalloc, for graphs
+ * that do not fit the device).  FW_GRAPH_HOST_PINNED keeps them in pinned host memory mapped into the
+ * device's address space: the kernels read them over the bus, 64 bytes per request, nothing migrates
+ * and nothing has to fit the device except xadj, the parking index (4 bytes per vertex) and the walk
+ * buffers.  Results are identical to FW_GRAPH_DEVICE; throughput is bounded by the bus, which hub
+ * parking (one read of a hub's list per 64 walkers) relieves.
+ */
+enum { FW_GRAPH_DEVICE = 0, FW_GRAPH_HOST_PINNED = 1 };
+int fw_graph_create_placed(int32_t V, uint64_t E, const uint32_t* h_xadj, const int32_t* h_adjncy,
+                           const float* h_weight, const int32_t* h_label, int placement, fw_graph** out);
+
+/*
  * Adopts device arrays that already hold a CSR (e.g. produced by fw_gen_rmat).  The arrays must
  * stay valid until fw_graph_destroy and must be readable 12 bytes past their last element
  * (the kernels use aligned 16-byte loads).  take_ownership != 0: destroy frees them with hipFree.
@@ -163,6 +176,8 @@ int fw_csr_write(const char* prefix, int32_t V, uint64_t E, const uint32_t* h_xa
                  const float* h_weight, const int32_t* h_label);
 /* load + fw_graph_create: graph::graph(...) followed by gpu_graph::gpu_graph(graph*) (src/main.cu:312-325). */
 int fw_graph_load(const char* prefix, int want_weight, int want_label, fw_graph** out);
+/* The same with the edge arrays placed as fw_graph_create_placed does (--umgraph, src/main.cu:48). */
+int fw_graph_load_placed(const char* prefix, int want_weight, int want_label, int placement, fw_graph** out);
 
 /* ---- walks ------------------------------------------------------------------------------------ */
 

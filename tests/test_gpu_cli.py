@@ -160,3 +160,14 @@ def test_ablation_levels_and_park_threshold(gpu, graph_files, tmp_path):
         _run("--input", prefix, "--deepwalk", "--all", "--d=10", "--seed=3", "--hub_threshold=1000",
              "--park_threshold=%d" % park, "--savepaths", out)
         assert (np.fromfile(out, dtype=np.int32).reshape(V, 11) == ref_wg).all(), park
+
+
+def test_umgraph_keeps_edges_on_the_host(gpu, graph_files, tmp_path):
+    """--umgraph (src/main.cu:48): the graph's edge arrays are not copied to the device; same walks."""
+    prefix, csr = graph_files
+    V = len(csr[0]) - 1
+    ref, _, _ = orc.walk(orc.Graph(*csr), orc.make_params(max_depth=11, seed=9), np.arange(V, dtype=np.int32))
+    out = str(tmp_path / "um.bin")
+    text = _run("--input", prefix, "--deepwalk", "--all", "--d=10", "--seed=9", "--umgraph", "--savepaths", out)
+    assert "umgraph: edge arrays stay in pinned host memory" in text
+    assert (np.fromfile(out, dtype=np.int32).reshape(V, 11) == ref).all()

@@ -12,10 +12,10 @@ import fw_oracle_binding as _oracle
 pytestmark = pytest.mark.gpu
 
 
-def _check(fw, csr, starts, **kw):
+def _check(fw, csr, starts, placement=0, **kw):
     xadj, adj, w, lab = csr
     og = _oracle.Graph(xadj, adj, w, lab)
-    g = fw.Graph.from_csr(xadj, adj, w, lab)
+    g = fw.Graph.from_csr(xadj, adj, w, lab, placement=placement)
     try:
         p = fw.default_params(**kw)
         paths, st = g.walk(p, starts)
@@ -255,3 +255,30 @@ def test_walk_on_generated_rmat(gpu):
         ref, steps, edges = _oracle.walk(og, _oracle.from_walk_params(p), starts)
         assert (paths == ref).all()
         assert (st.steps, st.sampled_edges) == (steps, edges)
+
+
+def test_edges_in_pinned_host_memory(gpu, hub):
+    """FW_GRAPH_HOST_PINNED (the reference's --umgraph, include/gpu_graph.cuh:46-54): the edge arrays stay in host
+    memory and the kernels read them over the bus.  Where the arrays live changes no draw and no path: all four
+    applications, the walk kernel alone and the parking pipeline, equal the oracle; downloading the graph returns
+    the arrays that went in."""
+    xadj, adj, w, lab = hub
+    g = gpu.Graph.from_csr(xadj, adj, w, lab, placement=gpu.GRAPH_HOST_PINNED)
+    try:
+        back = g.download(weights=True, labels=True)
+        assert g.is_sorted()
+    finally:
+        g.destroy()
+    for a, b in zip(back, hub):
+        assert (a == b).all()
+    starts = np.random.RandomState(8).randint(0, 12000, size=6000).astype(np.int32)
+    starts[:500] = 0
+    for park in (-1, 50):
+        _check(gpu, hub, starts, placement=gpu.GRAPH_HOST_PINNED, app=gpu.APP_DEEPWALK, max_depth=21,
+               hub_threshold=1000, park_threshold=park, seed=41)
+        _check(gpu, hub, starts, placement=gpu.GRAPH_HOST_PINNED, app=gpu.APP_PPR, max_depth=81, tp=0.2,
+               hub_threshold=1000, park_threshold=park, seed=42)
+        _check(gpu, hub, starts, placement=gpu.GRAPH_HOST_PINNED, app=gpu.APP_METAPATH, max_depth=6,
+               schema=[0, 1, 2, 3, 4], hub_threshold=1000, park_threshold=park, seed=43)
+    _check(gpu, hub, starts[:2000], placement=gpu.GRAPH_HOST_PINNED, app=gpu.APP_NODE2VEC, max_depth=11, p=2.0, q=0.5,
+           hub_threshold=1000, seed=44)
