@@ -113,6 +113,11 @@ def test_graph_create_validates_before_touching_the_device(fw):
         with pytest.raises(fw.FlowWalkerError, match=msg) as e:
             fw.Graph.from_csr(bad_x, bad_a, bad_w)
         assert e.value.status == 1
+        with pytest.raises(fw.FlowWalkerError, match=msg):  # the same checks whichever memory the edges go to
+            fw.Graph.from_csr(bad_x, bad_a, bad_w, placement=fw.GRAPH_HOST_PINNED)
+    with pytest.raises(fw.FlowWalkerError, match="unknown placement 7") as e:
+        fw.Graph.from_csr(x, a, w, placement=7)
+    assert e.value.status == 1
 
 
 def test_no_cpu_fallback(fw):
@@ -125,6 +130,8 @@ def test_no_cpu_fallback(fw):
     with pytest.raises(fw.FlowWalkerError, match="no HIP device") as e:
         fw.Graph.from_csr(x, a, w)
     assert e.value.status == 3
+    with pytest.raises(fw.FlowWalkerError, match="no HIP device"):
+        fw.Graph.from_csr(x, a, w, placement=fw.GRAPH_HOST_PINNED)
     with pytest.raises(fw.FlowWalkerError, match="no HIP device"):
         fw.Graph.rmat(8)
     with pytest.raises(fw.FlowWalkerError):
