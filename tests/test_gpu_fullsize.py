@@ -100,3 +100,51 @@ def test_config5_metapath_rmat26(gpu):
         _check_paths(xadj, adj, paths, starts, st, 6, sample=500000, label=lab, schema=schema)
     finally:
         g.destroy()
+
+
+def test_csr_offsets_above_two_to_the_31(gpu):
+    """A CSR with more than 2^31 entries (the format's offsets are uint32, include/graph.cuh:93-136): the walkers
+    live on the vertices whose lists start above 2^31, among them eight lists of 200,000 neighbours (workgroup
+    sampler, crowded buckets) and 32,760 of 520 (wave sampler, parked or not).  Bit-exact against the oracle."""
+    import fw_oracle_binding as orc
+
+    V, d, n_hubs, d_hub, C = 1 << 22, 520, 8, 200_000, 1 << 15
+    deg = np.full(V, d, dtype=np.int64)
+    deg[-n_hubs:] = d_hub
+    xadj64 = np.concatenate(([0], np.cumsum(deg)))
+    E = int(xadj64[-1])
+    assert (1 << 31) < E < (1 << 32) - 16
+    xadj = xadj64.astype(np.uint32)
+    first = V - C                                  # the community the walkers stay in; its lists start above 2^31
+    assert xadj64[first] > (1 << 31)
+    rng = np.random.default_rng(5)
+    # below the community: any valid graph will do, nobody walks there (every edge leads to vertex 0, weight 1)
+    adj = np.zeros(E, dtype=np.int32)
+    w = np.ones(E, dtype=np.float32)
+    lo = int(xadj64[first])
+    m = E - lo
+    inside = rng.integers(first, V, size=m, dtype=np.int32)
+    to_hub = rng.random(m) < 0.2                   # a fifth of the steps lands on one of the eight long lists
+    inside[to_hub] = (V - n_hubs + rng.integers(0, n_hubs, size=int(to_hub.sum()))).astype(np.int32)
+    adj[lo:] = inside
+    w[lo:] = (1.0 + 99.0 * rng.random(m, dtype=np.float32)).astype(np.float32)
+    w[lo:][rng.random(m) < 0.05] = 0.0
+    print("graph made: E = %d" % E, flush=True)
+
+    g = gpu.Graph.from_csr(xadj, adj, w, None)
+    og = orc.Graph(xadj, adj, w, None)
+    starts = rng.integers(first, V, size=20_000).astype(np.int32)
+    starts[:1000] = V - 1
+    try:
+        for kw in (dict(app=gpu.APP_DEEPWALK, max_depth=11, park_threshold=100, seed=71),
+                   dict(app=gpu.APP_DEEPWALK, max_depth=11, park_threshold=-1, seed=72),
+                   dict(app=gpu.APP_PPR, max_depth=21, tp=0.15, park_threshold=100, hub_threshold=1000, seed=73)):
+            p = gpu.default_params(**kw)
+            print("walk", kw, flush=True)
+            paths, st = g.walk(p, starts)
+            ref, steps, edges = orc.walk(og, orc.from_walk_params(p), starts)
+            assert (paths == ref).all(), kw
+            assert (st.steps, st.sampled_edges) == (steps, edges)
+            assert (paths[:, 1] >= first).all()
+    finally:
+        g.destroy()
