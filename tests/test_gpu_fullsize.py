@@ -148,3 +148,33 @@ def test_csr_offsets_above_two_to_the_31(gpu):
             assert (paths[:, 1] >= first).all()
     finally:
         g.destroy()
+
+
+def test_path_matrix_of_more_than_two_to_the_32_entries(gpu):
+    """54 million walks of length 80: the path matrix has 4.4e9 entries, so a walker's row starts beyond what 32 bits
+    index for every query past 53 million.  The first and the last rows equal the oracle's walks with the same
+    walker ids (draws are addressed by walker id), with parking (crowded buckets of millions) and without."""
+    import _graphs
+    import fw_oracle_binding as orc
+
+    xadj, adj, w, lab = _graphs.hub_graph(V=12000, hub_degrees=(9000, 2500, 700), base_degree=5, seed=11)
+    n, depth, k = 54_000_000, 81, 4000
+    assert n * depth > (1 << 32)
+    starts = (np.arange(n, dtype=np.int64) * 7919 % 12000).astype(np.int32)
+    g = gpu.Graph.from_csr(xadj, adj, w, lab)
+    og = orc.Graph(xadj, adj, w, lab)
+    try:
+        for park in (0, -1):
+            p = gpu.default_params(app=gpu.APP_DEEPWALK, max_depth=depth, hub_threshold=1000, park_threshold=park, seed=91)
+            print("walk park", park, flush=True)
+            paths, st = g.walk(p, starts)
+            assert (paths[:, 0] == starts).all()
+            assert st.steps == int((paths[:, 1:] >= 0).sum(dtype=np.int64))
+            head, _, _ = orc.walk(og, orc.from_walk_params(p), starts[:k])
+            assert (paths[:k] == head).all()
+            p.walker_base = n - k
+            tail, _, _ = orc.walk(og, orc.from_walk_params(p), starts[n - k:])
+            assert (paths[n - k:] == tail).all()
+            del paths
+    finally:
+        g.destroy()
