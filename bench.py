@@ -168,6 +168,12 @@ def main():
             "algorithmic_bytes": int(alg_bytes),
         },
     }
+    if out["roofline"]["traffic"] is not None:
+        # what the memory actually moved per pass, as a rate over the same device time: with hub parking a list is
+        # read once per batch of walkers, so `achieved` (bytes every walker would read alone) exceeds the peak and
+        # measures reuse; this pair is the pipeline's real HBM rate
+        out["roofline"]["traffic_achieved"] = out["roofline"]["traffic"] / (avg_kernel_ms * 1e-3) / 1e9
+        out["roofline"]["traffic_frac"] = out["roofline"]["traffic_achieved"] / HBM_PEAK_GBS
     if last.launches > 1:
         # per-kernel view of the last pass: each kernel's own HIP-event time and the algorithmic bytes of the steps
         # it took (what every walker would have to read on its own; fw_hub_batch reads a hub list once per batch
