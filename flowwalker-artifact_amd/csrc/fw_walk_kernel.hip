@@ -185,10 +185,11 @@ __device__ __forceinline__ uint32_t coop_upper_bound(const int32_t* __restrict__
   return lo + (uint32_t)__builtin_popcountll(__ballot(le));
 }
 
-// first index in [lo, hi) with arr[index] >= x (hi if none), galloping from lo
+// first index in [lo, hi) with arr[index] >= x (hi if none), galloping from lo; step0 (a power of two) is the first
+// stride: 1 when x is expected right behind lo, more when the caller knows that it has jumped ahead in its own list
 __device__ __forceinline__ uint32_t gallop_lower_bound(const int32_t* __restrict__ arr, uint32_t lo, uint32_t hi,
-                                                       int32_t x) {
-  uint32_t a = lo, b = lo, step = 1u;
+                                                       int32_t x, uint32_t step0 = 1u) {
+  uint32_t a = lo, b = lo + step0 - 1u, step = step0;
   while (b < hi && arr[b] < x) {
     a = b + 1u;
     b = a + step - 1u;
@@ -227,6 +228,19 @@ __device__ __forceinline__ uint32_t coop_lower_bound(const int32_t* __restrict__
 constexpr int kN2vChunk = 256;    // entries of N(prev) resolved per refill: 4 per lane
 constexpr int kN2vWindow = 1024;  // entries of N(prev) staged per group
 constexpr int kN2vMaxWindows = 16;   // longer stretches of N(prev) per group are searched in place
+// First strides of the forward test's gallops (powers of two; the answers do not depend on them).  A lane's
+// neighbours ascend, so the search for one starts where the search for the one before ended, but the first
+// neighbour of a quartet lies 252 neighbours of cur behind the lane's last one, a lane's first search in a streamed
+// window can end anywhere in it, and a stretch that is streamed or searched in place holds many entries of N(prev)
+// per neighbour of the group.  Measured on symmetrised R-MAT graphs, the doubling phase of a gallop that starts
+// with stride 1 costs more than it saves in all of these places: the strides below make such a search nearly a
+// binary search over what is left, and only the neighbours inside a quartet keep stride 1 when the stretch fits
+// one window.
+constexpr uint32_t kN2vQuartetStride = 256;
+constexpr uint32_t kN2vWindowStride = 512;
+constexpr uint32_t kN2vStreamedStride = 32;
+constexpr uint32_t kN2vInPlaceQuartetStride = 8192;
+constexpr uint32_t kN2vInPlaceStride = 128;
 constexpr uint64_t kN2vReverseRatio = 8;  // reversed test when N(prev) is at least this many times shorter than N(cur)
 struct N2vScratch {
   union {
@@ -495,7 +509,7 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
           if (post[e] == c.prev) {  // the return edge, or an entry outside the list (bias 0 already)
             x[4 * j + e] = x[4 * j + e] * a.inv_p;
           } else {
-            lane_pos = gallop_lower_bound(win, lane_pos, st_hi, post[e]);
+            lane_pos = gallop_lower_bound(win, lane_pos, st_hi, post[e], e == 0 ? kN2vQuartetStride : 1u);
             const bool common = lane_pos < st_hi && win[lane_pos] == post[e];
             x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
           }
@@ -545,7 +559,7 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
             if (post[e] == c.prev) {
               x[4 * j + e] = x[4 * j + e] * a.inv_p;
             } else {
-              pos = gallop_lower_bound(win, pos, hi_w, post[e]);
+              pos = gallop_lower_bound(win, pos, hi_w, post[e], e == 0 ? kN2vQuartetStride : 1u);
               const bool common = pos < hi_w && win[pos] == post[e];
               x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
             }
@@ -566,22 +580,38 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
             }
           }
         }
+        // the next window's entries are fetched into registers while the current window is searched
+        int4 ahead[kN2vWindow / 256];
+#pragma unroll
+        for (int k = 0; k < kN2vWindow / 256; ++k) {
+          const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
+          ahead[k] = make_int4(0, 0, 0, 0);
+          if (wa + wi < p_hi) ahead[k] = *reinterpret_cast<const int4*>(a.adjncy + wa + wi);
+        }
         for (uint32_t ws = wa; ws < p_hi; ws += (uint32_t)kN2vWindow) {
           __builtin_amdgcn_wave_barrier();  // the previous window's searches are done
 #pragma unroll
           for (int k = 0; k < kN2vWindow / 256; ++k) {
             const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
-            if (ws + wi < p_hi)
-              *reinterpret_cast<int4*>(&scr->window[wi]) = *reinterpret_cast<const int4*>(a.adjncy + ws + wi);
+            if (ws + wi < p_hi) *reinterpret_cast<int4*>(&scr->window[wi]) = ahead[k];
           }
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
           __builtin_amdgcn_wave_barrier();
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          {
+            const uint32_t wn = ws + (uint32_t)kN2vWindow;
+#pragma unroll
+            for (int k = 0; k < kN2vWindow / 256; ++k) {
+              const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
+              if (wn + wi < p_hi) ahead[k] = *reinterpret_cast<const int4*>(a.adjncy + wn + wi);
+            }
+          }
           const int32_t* win = scr->window;
           const uint32_t hi_w = (p_hi - ws) < (uint32_t)kN2vWindow ? (p_hi - ws) : (uint32_t)kN2vWindow;
           const bool last = ws + (uint32_t)kN2vWindow >= p_hi;
           const int32_t wmax = win[hi_w - 1u];
           uint32_t pos = ws == wa ? p_lo - wa : 0u;
+          uint32_t stride = kN2vWindowStride;  // a lane's first search in a window starts anywhere in it
 #pragma unroll
           for (int j = 0; j < kJ; ++j) {
             const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
@@ -589,7 +619,8 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
             for (int e = 0; e < 4; ++e) {
               const int i = 4 * j + e;
               if (((done >> i) & 1u) == 0u && (post[e] <= wmax || last)) {
-                pos = gallop_lower_bound(win, pos, hi_w, post[e]);
+                pos = gallop_lower_bound(win, pos, hi_w, post[e], stride);
+                stride = kN2vStreamedStride;
                 const bool common = pos < hi_w && win[pos] == post[e];
                 x[i] = common ? x[i] : x[i] * a.inv_q;
                 done |= 1u << i;
@@ -607,7 +638,7 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
             if (post[e] == c.prev) {
               x[4 * j + e] = x[4 * j + e] * a.inv_p;
             } else {
-              pos = gallop_lower_bound(plist, pos, seg_hi, post[e]);
+              pos = gallop_lower_bound(plist, pos, seg_hi, post[e], e == 0 ? kN2vInPlaceQuartetStride : kN2vInPlaceStride);
               const bool common = pos < seg_hi && plist[pos] == post[e];
               x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
             }
