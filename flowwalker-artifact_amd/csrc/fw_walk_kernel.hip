@@ -225,7 +225,8 @@ __device__ __forceinline__ uint32_t coop_lower_bound(const int32_t* __restrict__
 // Per-wave LDS scratch of the adjacency test.  Forward test (neighbours of cur looked up in N(prev)): `window`
 // holds the part of N(prev) that can contain the current group's vertices, so the per-lane searches run in LDS.
 // Reversed test (entries of N(prev) looked up in N(cur)): `match` and `mask` share the same memory.
-constexpr int kN2vChunk = 256;    // entries of N(prev) resolved per refill: 4 per lane
+constexpr int kN2vPerLane = 2;    // entries of N(prev) a lane resolves per refill
+constexpr int kN2vChunk = 64 * kN2vPerLane;  // entries of N(prev) resolved per refill
 constexpr int kN2vWindow = 1024;  // entries of N(prev) staged per group
 constexpr int kN2vMaxWindows = 16;   // longer stretches of N(prev) per group are searched in place
 // First strides of the forward test's gallops (powers of two; the answers do not depend on them).  A lane's
@@ -260,60 +261,57 @@ struct N2vCursor {
   uint32_t mpos = 0;    // matches already applied
 };
 
-// Resolves the next kN2vChunk entries of N(prev): each lane looks its 4 consecutive entries up in N(cur)
-// (galloping from the resolved prefix) and the hits are written to scr.match in ascending order.
+// Resolves the next kN2vChunk entries of N(prev) (fewer at the end of the list): entry i of them is looked up in
+// N(cur), over the part of it that is not resolved yet, by lane i % 64 in its chain i / 64, and the hits are written
+// to scr.match in ascending order.  The chains of a lane do not depend on each other and the entries of a short
+// N(prev) lie far apart in N(cur): plain binary searches advancing together, one memory latency per round for all
+// of them.  A chain that no lane needs (fewer than 64 * chain entries left) costs nothing.
 __device__ __forceinline__ void n2v_refill(const int32_t* __restrict__ clist, uint32_t dc,
                                            const int32_t* __restrict__ plist, uint32_t dp, N2vScratch& scr,
                                            N2vCursor& k, int lane) {
+  constexpr int kP = kN2vPerLane;
   const uint32_t cnt = (dp - k.pc) < (uint32_t)kN2vChunk ? (dp - k.pc) : (uint32_t)kN2vChunk;
-  const uint32_t base = k.pc + 4u * (uint32_t)lane;
-  // The four look-ups of a lane do not depend on each other, and the entries of a short N(prev) lie far apart in
-  // N(cur): plain binary searches over the unresolved part, advancing together (one memory latency per round
-  // for all four, instead of galloping from hit to hit).
-  uint32_t hit_pos[4];
-  bool hit[4];
-  int32_t y[4];
-  bool valid[4];
-  uint32_t lo[4], hi[4];
+  int32_t y[kP];
+  uint32_t lo[kP], hi[kP];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    valid[e] = base + (uint32_t)e < k.pc + cnt;
-    y[e] = valid[e] ? plist[base + (uint32_t)e] : 0;
+  for (int e = 0; e < kP; ++e) {
+    const uint32_t i = 64u * (uint32_t)e + (uint32_t)lane;
+    const bool valid = i < cnt;
+    y[e] = valid ? plist[k.pc + i] : 0;
     lo[e] = k.cov;
-    hi[e] = valid[e] ? dc : k.cov;
+    hi[e] = valid ? dc : k.cov;
   }
   for (uint32_t span = dc - k.cov; span != 0u; span >>= 1) {  // ceil(log2(span + 1)) rounds close every search
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const bool open = lo[e] < hi[e];
-      const uint32_t mid = (lo[e] + hi[e]) >> 1;
-      const int32_t val = open ? clist[mid] : 0;
-      const bool less = open && val < y[e];
-      lo[e] = less ? mid + 1u : lo[e];
-      hi[e] = (open && !less) ? mid : hi[e];
+    for (int e = 0; e < kP; ++e) {
+      if (64u * (uint32_t)e < cnt) {  // uniform in the wave
+        const bool open = lo[e] < hi[e];
+        const uint32_t mid = (lo[e] + hi[e]) >> 1;
+        const int32_t val = open ? clist[mid] : 0;
+        const bool less = open && val < y[e];
+        lo[e] = less ? mid + 1u : lo[e];
+        hi[e] = (open && !less) ? mid : hi[e];
+      }
     }
   }
-  uint32_t resolved = k.cov;  // after this lane's last entry: indices below are resolved
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    hit_pos[e] = lo[e];
-    hit[e] = valid[e] && lo[e] < dc && clist[lo[e]] == y[e];
-    if (valid[e]) resolved = lo[e] + (hit[e] ? 1u : 0u);
-  }
-  const uint64_t m0 = __ballot(hit[0]), m1 = __ballot(hit[1]), m2 = __ballot(hit[2]), m3 = __ballot(hit[3]);
   const uint64_t below = (1ull << lane) - 1ull;
-  uint32_t at = (uint32_t)(__builtin_popcountll(m0 & below) + __builtin_popcountll(m1 & below) +
-                           __builtin_popcountll(m2 & below) + __builtin_popcountll(m3 & below));
+  const uint32_t last = cnt - 1u;  // the list's entries ascend: after this one, every index below its place is resolved
+  uint32_t total = 0u, cov = k.cov;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    if (hit[e]) scr.match[at++] = (int32_t)hit_pos[e];
+  for (int e = 0; e < kP; ++e) {
+    if (64u * (uint32_t)e < cnt) {
+      const bool valid = 64u * (uint32_t)e + (uint32_t)lane < cnt;
+      const bool hit = valid && lo[e] < dc && clist[lo[e]] == y[e];
+      const uint64_t m = __ballot(hit);
+      if (hit) scr.match[total + (uint32_t)__builtin_popcountll(m & below)] = (int32_t)lo[e];
+      total += (uint32_t)__builtin_popcountll(m);
+      if ((last >> 6) == (uint32_t)e)
+        cov = (uint32_t)__builtin_amdgcn_readlane((int)(lo[e] + (hit ? 1u : 0u)), (int)(last & 63u));
+    }
   }
-  k.mcount = (uint32_t)(__builtin_popcountll(m0) + __builtin_popcountll(m1) + __builtin_popcountll(m2) +
-                        __builtin_popcountll(m3));
+  k.mcount = total;
   k.mpos = 0u;
   k.pc += cnt;
-  const uint32_t last_lane = (cnt - 1u) >> 2;
-  const uint32_t cov = (uint32_t)__builtin_amdgcn_readlane((int)resolved, (int)last_lane);
   k.cov = k.pc >= dp ? dc : cov;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
