@@ -24,7 +24,7 @@ GRAPH_DEVICE, GRAPH_HOST_PINNED = 0, 1
 
 # every symbol include/flowwalker.h declares
 EXPORTED = [
-    "fw_last_error", "fw_device_count", "fw_device_mem_info", "fw_walk_params_default", "fw_autobatch_size",
+    "fw_last_error", "fw_device_count", "fw_device_mem_info", "fw_walk_params_default", "fw_walk_params_default_for", "fw_autobatch_size",
     "fw_dev_alloc", "fw_dev_free", "fw_dev_upload", "fw_dev_download", "fw_dev_fill_i32", "fw_dev_copy", "fw_dev_sync",
     "fw_graph_create", "fw_graph_adopt_device", "fw_graph_destroy", "fw_graph_info", "fw_graph_is_sorted",
     "fw_graph_download", "fw_walk_device", "fw_walk_batch", "fw_host_alloc_pinned", "fw_host_free_pinned",
@@ -82,6 +82,8 @@ def lib():
         L.fw_device_mem_info.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
         L.fw_walk_params_default.argtypes = [C.POINTER(WalkParams)]
         L.fw_walk_params_default.restype = None
+        L.fw_walk_params_default_for.argtypes = [C.POINTER(WalkParams), C.c_int]
+        L.fw_walk_params_default_for.restype = None
         L.fw_dev_alloc.argtypes = [C.c_size_t, C.POINTER(C.c_void_p)]
         L.fw_dev_free.argtypes = [C.c_void_p]
         L.fw_dev_upload.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
@@ -132,7 +134,10 @@ def mem_info():
 
 def default_params(**overrides):
     p = WalkParams()
-    lib().fw_walk_params_default(C.byref(p))
+    if "app" in overrides:  # the library's choices for that application (node2vec: wave granularity)
+        lib().fw_walk_params_default_for(C.byref(p), int(overrides["app"]))
+    else:
+        lib().fw_walk_params_default(C.byref(p))
     set_params(p, **overrides)
     return p
 

@@ -84,6 +84,13 @@ extern "C" void fw_walk_params_default(fw_walk_params* p) {
   p->grid = 0;
 }
 
+extern "C" void fw_walk_params_default_for(fw_walk_params* p, int app) {
+  if (!p) return;
+  fw_walk_params_default(p);
+  p->app = app;
+  if (app == FW_APP_NODE2VEC) p->hub_threshold = INT_MAX;
+}
+
 extern "C" uint32_t fw_autobatch_size(size_t free_bytes, int32_t headroom_mb, int32_t max_depth, int sync,
                                       uint32_t n_queries) {
   const size_t headroom = (size_t)(headroom_mb > 0 ? headroom_mb : 0) * 1024u * 1024u;

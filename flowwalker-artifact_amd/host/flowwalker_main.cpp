@@ -262,7 +262,7 @@ int main(int argc, char** argv) {
   }
 
   fw_walk_params P;
-  fw_walk_params_default(&P);
+  fw_walk_params_default_for(&P, F.deepwalk ? FW_APP_DEEPWALK : F.ppr ? FW_APP_PPR : F.node2vec ? FW_APP_NODE2VEC : FW_APP_METAPATH);
   std::vector<int> schema;
   if (F.metapath) {
     if (!parse_schema(F.schema, &schema) || schema.size() > FW_MAX_SCHEMA) {

@@ -97,6 +97,12 @@ int fw_device_mem_info(size_t* free_bytes, size_t* total_bytes);
 /* Fills defaults: app DeepWalk, d = 80, tp 0.2, p 2.0, q 0.5, schema 0,1,2,3,4, seed 1337 (src/main.cu:40-80). */
 void fw_walk_params_default(fw_walk_params* p);
 
+/* The same defaults with `app` set and what the library would choose for that application: node2vec samples every
+ * list at wave granularity (hub_threshold INT32_MAX), because only a single wave can look a short N(prev) up in
+ * N(cur) instead of testing every neighbour of cur.  The reference also picks node2vec's kernel by application
+ * (the one-pass sampler, src/walk.cu:403). */
+void fw_walk_params_default_for(fw_walk_params* p, int app);
+
 /*
  * Autobatch rule of adjust_flags (src/main.cu:259-271):
  *   bs = min((free - headroom_mb * 2^20) / (4 * (d + 2)), INT_MAX); halved unless sync; min(bs, n_queries).

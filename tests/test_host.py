@@ -40,6 +40,19 @@ def test_default_params_follow_the_reference_flags(fw):
     assert p.wg_threads in (256, 512, 1024) and p.hub_threshold > 0
 
 
+def test_default_params_per_application(fw):
+    """Per-application defaults differ from the plain ones only where the library chooses differently: node2vec
+    samples every list at wave granularity."""
+    base = fw.default_params()
+    for app in (fw.APP_DEEPWALK, fw.APP_PPR, fw.APP_METAPATH):
+        p = fw.default_params(app=app)
+        assert p.app == app and p.hub_threshold == base.hub_threshold
+    p = fw.default_params(app=fw.APP_NODE2VEC)
+    assert p.app == fw.APP_NODE2VEC and p.hub_threshold == 2 ** 31 - 1
+    assert (p.max_depth, p.wg_threads, p.seed) == (base.max_depth, base.wg_threads, base.seed)
+    assert fw.default_params(app=fw.APP_NODE2VEC, hub_threshold=4096).hub_threshold == 4096
+
+
 def test_autobatch_rule(fw):
     """bs = min((free - headroom MB) / (4 (d + 2)), INT_MAX); halved unless sync; capped at the query count
     (src/main.cu:259-271)."""
