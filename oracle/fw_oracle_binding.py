@@ -52,6 +52,13 @@ def lib():
         L.fw_oracle_num_threads.restype = C.c_int
         L.fw_oracle_sequential_reservoir.argtypes = [C.c_void_p, C.c_void_p, C.c_int32]
         L.fw_oracle_sequential_reservoir.restype = C.c_int32
+        for name in ("fw_ref_sampler_thread", "fw_ref_sampler_zprs", "fw_ref_sampler_dprs"):
+            getattr(L, name).restype = C.c_int32
+        L.fw_ref_sampler_thread.argtypes = [C.c_void_p, C.c_int32, C.c_void_p]
+        L.fw_ref_sampler_zprs.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]
+        L.fw_ref_sampler_dprs.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]
+        L.fw_ref_sample_many.argtypes = [C.c_int, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p]
+        L.fw_ref_sample_many.restype = C.c_int
         _lib = L
     return _lib
 
@@ -134,3 +141,18 @@ def sequential_reservoir(w, u):
     w = np.ascontiguousarray(w, dtype=np.float32)
     u = np.ascontiguousarray(u, dtype=np.float32)
     return int(lib().fw_oracle_sequential_reservoir(w.ctypes.data_as(C.c_void_p), u.ctypes.data_as(C.c_void_p), len(w)))
+
+
+REF_THREAD, REF_ZPRS, REF_DPRS = 0, 1, 2
+
+
+def ref_sample_many(kind, w, u, width=32):
+    """The reference's own samplers restated (fw_ref_samplers.c): row r of `u` (one uniform per bias) drives step r."""
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    u = np.ascontiguousarray(u, dtype=np.float32)
+    assert u.ndim == 2 and u.shape[1] == len(w)
+    out = np.empty(u.shape[0], dtype=np.int32)
+    rc = lib().fw_ref_sample_many(kind, w.ctypes.data, len(w), width, u.ctypes.data, u.shape[0], out.ctypes.data)
+    if rc != 0:
+        raise ValueError("fw_ref_sample_many: bad arguments")
+    return out

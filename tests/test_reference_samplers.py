@@ -1,0 +1,103 @@
+"""The reference's own samplers (include/sampler.cuh), restated thread by thread in oracle/fw_ref_samplers.c, against
+their sequential ground truth and against this build's sampler.
+
+The walk engine here samples with a different algorithm than the reference, so what the two must share is the law of
+one sampling step, P(i) = w_i / sum w, and the special cases.  These tests pin that on the reference's algorithm
+itself: (1) its parallel samplers are the sequential weighted reservoir over a permutation of the list (exact
+equality on integer-valued biases, where f32 sums do not depend on the order of the additions), and (2) all of them
+and this build's sampler follow the same distribution on the same list (chi-square).
+"""
+import numpy as np
+import pytest
+from scipy.stats import chisquare
+
+import fw_oracle_binding as orc
+
+
+def _uniforms(rng, shape):
+    """(0, 1] like cuRAND's (include/myrand.cuh:213-215): x * 2^-32 + 2^-33 on 32 random bits."""
+    bits = rng.randint(0, 2 ** 32, size=shape, dtype=np.uint64)
+    return (bits.astype(np.float64) * 2.0 ** -32 + 2.0 ** -33).astype(np.float32)
+
+
+def _int_biases(rng, n, zero_fraction):
+    w = rng.randint(1, 50, size=n).astype(np.float32)
+    w[rng.random_sample(n) < zero_fraction] = 0.0
+    return w
+
+
+@pytest.mark.parametrize("width", [32, 512])
+@pytest.mark.parametrize("n", [1, 2, 31, 32, 33, 100, 511, 512, 513, 2000])
+def test_zprs_is_the_sequential_reservoir_over_the_lane_major_order(n, width):
+    """include/sampler.cuh:46-127: lane l owns elements l, l + W, ...; the key i + size * lane makes the highest lane's
+    latest acceptance win, which is sequential reservoir sampling over (lane 0's elements, lane 1's, ...)."""
+    rng = np.random.RandomState(1000 * width + n)
+    for zero_fraction in (0.0, 0.3, 1.0):
+        w = _int_biases(rng, n, zero_fraction)
+        u = _uniforms(rng, (200, n))
+        order = np.concatenate([np.arange(l, n, width) for l in range(min(width, n))])
+        assert sorted(order) == list(range(n))
+        got = orc.ref_sample_many(orc.REF_ZPRS, w, u, width)
+        seq = orc.ref_sample_many(orc.REF_THREAD, w[order], u[:, order], width)
+        # positions in the permuted list map back through the order; the fallback "index 0" of :37 / :75 is
+        # position 0 there and element 0 here, and order[0] == 0
+        want = np.where(seq < 0, -1, order[np.maximum(seq, 0)])
+        assert (got == want).all()
+        if zero_fraction == 1.0:
+            assert (got == -1).all()
+
+
+@pytest.mark.parametrize("width", [32, 512])
+@pytest.mark.parametrize("n", [1, 2, 31, 32, 33, 64, 100, 512, 513, 2000])
+def test_dprs_is_the_sequential_reservoir_in_list_order(n, width):
+    """include/sampler.cuh:129-200: chunks of W in list order with a carried prefix; the running maximum of the accepted
+    indices is the last acceptance of sequential reservoir sampling."""
+    rng = np.random.RandomState(7000 * width + n)
+    for zero_fraction in (0.0, 0.3, 1.0):
+        w = _int_biases(rng, n, zero_fraction)
+        u = _uniforms(rng, (200, n))
+        got = orc.ref_sample_many(orc.REF_DPRS, w, u, width)
+        seq = orc.ref_sample_many(orc.REF_THREAD, w, u, width)
+        assert (got == seq).all()
+
+
+def test_sequential_reservoir_matches_this_builds_ground_truth():
+    """fw_oracle_sequential_reservoir (accept iff u * S < w) and the reference's form (u < w / S) agree."""
+    rng = np.random.RandomState(5)
+    w = _int_biases(rng, 300, 0.2)
+    u = _uniforms(rng, (2000, 300))
+    ref = orc.ref_sample_many(orc.REF_THREAD, w, u)
+    ours = np.array([orc.lib().fw_oracle_sequential_reservoir(w.ctypes.data, u[r].ctypes.data, len(w))
+                     for r in range(len(u))])
+    assert (ref == ours).mean() > 0.999  # the two forms can round differently when u is within an ulp of w / S
+    assert ((ref >= 0) == (ours >= 0)).all()
+
+
+def test_all_samplers_follow_the_same_law():
+    """Reference thread / ZPRS / DPRS samplers and this build's group-reservoir sampler on one list of 1500 biases
+    (f32 U[1, 100), a tenth of them zero): chi-square against w / sum w, p > 0.01 each; zero biases never taken."""
+    rng = np.random.RandomState(99)
+    n, m = 1500, 90000
+    w = (1.0 + 99.0 * rng.random_sample(n)).astype(np.float32)
+    w[rng.random_sample(n) < 0.1] = 0.0
+    pos = w > 0
+    expect = w[pos].astype(np.float64) / w.astype(np.float64).sum() * m
+    for kind, width in ((orc.REF_THREAD, 32), (orc.REF_ZPRS, 32), (orc.REF_ZPRS, 512), (orc.REF_DPRS, 32),
+                        (orc.REF_DPRS, 512)):
+        cnt = np.zeros(n)
+        for _ in range(3):  # three slabs of uniforms keep the memory small
+            u = _uniforms(rng, (m // 3, n))
+            cnt += np.bincount(orc.ref_sample_many(kind, w, u, width), minlength=n)
+        assert cnt[~pos].sum() == 0
+        assert chisquare(cnt[pos], expect).pvalue > 0.01, (kind, width)
+    # this build's sampler: vertex 1 of a small graph owns the same list (neighbour i is vertex i % V)
+    V = n + 2
+    xadj = np.zeros(V + 1, dtype=np.uint32)
+    xadj[2:] = n
+    g = orc.Graph(xadj, (np.arange(n) % V).astype(np.int32), w)
+    for thr in (1 << 30, 1000):
+        p = orc.make_params(max_depth=2, hub_threshold=thr, seed=77)
+        paths, _, _ = orc.walk(g, p, np.full(m, 1, dtype=np.int32))
+        cnt = np.bincount(paths[:, 1], minlength=V)[:n].astype(np.float64)
+        assert cnt.sum() == m and cnt[~pos].sum() == 0
+        assert chisquare(cnt[pos], expect).pvalue > 0.01, thr
