@@ -282,3 +282,52 @@ def test_edges_in_pinned_host_memory(gpu, hub):
                schema=[0, 1, 2, 3, 4], hub_threshold=1000, park_threshold=park, seed=43)
     _check(gpu, hub, starts[:2000], placement=gpu.GRAPH_HOST_PINNED, app=gpu.APP_NODE2VEC, max_depth=11, p=2.0, q=0.5,
            hub_threshold=1000, seed=44)
+
+
+def test_randomized_configurations(gpu):
+    """Seeded random graphs (planted hubs up to degree 33,000, directed or undirected, zero weights), applications,
+    depths, workgroup sizes, granularity and parking thresholds, start sets (spread, all on one vertex, a handful of
+    vertices): every case bit-exact against the oracle."""
+    rng = np.random.RandomState(20240)
+    apps = [gpu.APP_DEEPWALK, gpu.APP_PPR, gpu.APP_NODE2VEC, gpu.APP_METAPATH]
+    for _ in range(24):
+        V = int(rng.choice([300, 2000, 9000, 40000]))
+        nh = int(rng.randint(0, 5))
+        hubs = tuple(int(min(V - 1, rng.choice([70, 130, 300, 1100, 2500, 5000, 17000, 33000]))) for _ in range(nh))
+        csr = _graphs.hub_graph(V=V, hub_degrees=hubs, base_degree=int(rng.choice([1, 3, 8, 20])),
+                                seed=int(rng.randint(1, 1 << 30)), symmetric=bool(rng.randint(0, 2)),
+                                zero_weight_fraction=float(rng.choice([0.0, 0.0, 0.05, 0.5])))
+        xadj, adj, w, lab = csr
+        og = _oracle.Graph(xadj, adj, w, lab)
+        g = gpu.Graph.from_csr(xadj, adj, w, lab)
+        try:
+            for _ in range(6):
+                app = int(rng.choice(apps))
+                depth = int(rng.choice([2, 4, 6])) if app == gpu.APP_METAPATH else int(rng.choice([2, 3, 11, 41, 81]))
+                n = int(rng.choice([1, 63, 1000, 20000]))
+                mode = rng.randint(0, 3)
+                if mode == 0:
+                    starts = rng.randint(0, V, size=n)
+                elif mode == 1:
+                    starts = np.full(n, rng.randint(0, nh if nh else V))
+                else:
+                    starts = rng.randint(0, min(V, 8), size=n)
+                kw = dict(app=app, max_depth=depth, wg_threads=int(rng.choice([256, 512, 1024])),
+                          hub_threshold=int(rng.choice([0, 64, 500, 1024, 16384, 1 << 30])),
+                          park_threshold=int(rng.choice([-1, 0])) if app == gpu.APP_NODE2VEC
+                          else int(rng.choice([-1, 0, 1, 4, 16, 64, 200, 3000])), seed=int(rng.randint(0, 1 << 31)))
+                if app == gpu.APP_NODE2VEC:
+                    kw["p"], kw["q"] = float(rng.choice([0.25, 1.0, 2.0])), float(rng.choice([0.5, 1.0, 4.0]))
+                if app == gpu.APP_PPR:
+                    kw["tp"] = float(rng.choice([0.05, 0.2, 0.9]))
+                if app == gpu.APP_METAPATH:
+                    kw["schema"] = [int(x) for x in rng.randint(0, 5, size=depth - 1)]
+                p = gpu.default_params(**kw)
+                paths, st = g.walk(p, starts.astype(np.int32))
+                ref, steps, edges = _oracle.walk(og, _oracle.from_walk_params(p), starts.astype(np.int32))
+                bad = np.nonzero((paths != ref).any(axis=1))[0]
+                assert len(bad) == 0, "hubs %s, %s: first differing walk %d:\n gpu %s\n ref %s" % (
+                    hubs, kw, bad[0], paths[bad[0]], ref[bad[0]])
+                assert (st.steps, st.sampled_edges) == (steps, edges), (hubs, kw)
+        finally:
+            g.destroy()
