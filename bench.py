@@ -41,7 +41,7 @@ HEADLINE = "deepwalk_rmat24_sym"
 # HBM-side bytes of one pass (all launches of the walk pipeline) from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs, each scaled by what the same counter reads for the 1 GiB copy kernel (profiles/).
 # None for workloads that have not been measured.
-MEASURED_TRAFFIC_BYTES = {"deepwalk_rmat24_sym": 5.73e11}
+MEASURED_TRAFFIC_BYTES = {"deepwalk_rmat24_sym": 5.73e11, "node2vec_rmat24_sym": 5.24e13}
 
 
 def algorithmic_bytes(app, steps, sampled_edges, queries, probe_terms=0):
@@ -161,8 +161,10 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
+            # measured with the library defaults only: any override makes it another run
             "traffic": MEASURED_TRAFFIC_BYTES.get(
-                args.workload if not args.scale and args.park_threshold == 0 and last.launches > 1 else None),
+                args.workload if not args.scale and args.park_threshold == 0 and args.hub_threshold < 0
+                and args.wg_threads == 0 and (last.launches > 1 or wl["app"] == "node2vec") else None),
             "kernel": "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_batch pipeline",
             "kernel_ms": avg_kernel_ms,
             "algorithmic_bytes": int(alg_bytes),
