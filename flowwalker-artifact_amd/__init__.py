@@ -29,7 +29,7 @@ EXPORTED = [
     "fw_graph_create", "fw_graph_adopt_device", "fw_graph_destroy", "fw_graph_info", "fw_graph_is_sorted",
     "fw_graph_download", "fw_walk_device", "fw_walk_batch", "fw_host_alloc_pinned", "fw_host_free_pinned",
     "fw_gen_rmat", "fw_csr_read_header", "fw_csr_load", "fw_csr_write", "fw_graph_load",
-    "fw_graph_create_placed", "fw_graph_load_placed",
+    "fw_graph_create_placed", "fw_graph_load_placed", "fw_walk_device_noalloc",
 ]
 
 
@@ -103,6 +103,7 @@ def lib():
         L.fw_graph_download.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.fw_walk_device.argtypes = [C.c_void_p, C.POINTER(WalkParams), C.c_void_p, C.c_int32, C.c_void_p,
                                      C.c_void_p, C.POINTER(WalkStats)]
+        L.fw_walk_device_noalloc.argtypes = L.fw_walk_device.argtypes
         L.fw_walk_batch.argtypes = [C.c_void_p, C.POINTER(WalkParams), C.c_void_p, C.c_int32, C.c_uint32, C.c_int,
                                     C.c_void_p, C.POINTER(WalkStats)]
         L.fw_host_alloc_pinned.argtypes = [C.c_size_t, C.POINTER(C.c_void_p)]
@@ -276,6 +277,13 @@ class Graph:
         """One launch over device-resident starts / paths (DeviceBuffer objects).  Returns WalkStats."""
         st = WalkStats()
         check(lib().fw_walk_device(self.handle, C.byref(params), d_starts.ptr, int(n), d_paths.ptr, None, C.byref(st)))
+        return st
+
+    def walk_device_noalloc(self, params, d_starts, n, d_paths):
+        """fw_walk_device_noalloc: one launch, scratch in the library's static device array.  Returns WalkStats."""
+        st = WalkStats()
+        check(lib().fw_walk_device_noalloc(self.handle, C.byref(params), d_starts.ptr, int(n), d_paths.ptr, None,
+                                           C.byref(st)))
         return st
 
     def walk(self, params, starts):

@@ -12,6 +12,7 @@
 #include <cstring>
 
 #include <chrono>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -1207,6 +1208,114 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
     stats->hub_kernel_ms = times.hub_ms;
     stats->hub_steps = h.counters[2];
     stats->hub_sampled_edges = h.counters[3];
+  }
+  return FW_OK;
+}
+
+// ---- fw_walk_device_noalloc: the single-launch walk for callers that cannot allocate -----------------------
+//
+// fw_walk_device allocates its launch scratch (query dispenser word + workload counters) and two events per call.
+// This variant keeps that scratch in a file-scope device array and creates its events once per device, so a call
+// makes no hipMalloc / hipFree / hipEventCreate.  Every device holds its own copy of the array at its own address;
+// the address is looked up once per device (the array's name is only a host-side handle, never a kernel argument).
+// All calls on a device share the array: calls that overlap on one device race on it.
+
+static __device__ __align__(256) unsigned char scratch[256];
+static_assert(sizeof(Scratch) <= sizeof(scratch), "the launch scratch record must fit the static array");
+
+namespace {
+constexpr int kNoAllocMaxDevices = 64;
+struct NoAllocDevice {
+  Scratch* ptr = nullptr;  // device address of `scratch` on this device
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+};
+NoAllocDevice g_noalloc[kNoAllocMaxDevices];
+std::mutex g_noalloc_lock;
+
+// Set-up of the current device, once: the array's address on this device and the two timing events.
+int noalloc_device(NoAllocDevice** out) {
+  int dev = 0;
+  FW_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kNoAllocMaxDevices) {
+    fw_set_error("fw_walk_device_noalloc: device %d is beyond the %d devices it keeps state for", dev, kNoAllocMaxDevices);
+    return FW_ERR_INVALID;
+  }
+  std::lock_guard<std::mutex> guard(g_noalloc_lock);
+  NoAllocDevice& d = g_noalloc[dev];
+  if (d.ptr == nullptr) {
+    void* p = nullptr;
+    FW_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (p == nullptr) { fw_set_error("fw_walk_device_noalloc: the scratch array has no address on device %d", dev); return FW_ERR_HIP; }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    FW_HIP(hipEventCreate(&e0));
+    if (fw_check_hip(hipEventCreate(&e1), "hipEventCreate", __FILE__, __LINE__) != FW_OK) {
+      (void)hipEventDestroy(e0);
+      return FW_ERR_HIP;
+    }
+    d.ev0 = e0;
+    d.ev1 = e1;
+    d.ptr = static_cast<Scratch*>(p);
+  }
+  *out = &d;
+  return FW_OK;
+}
+}  // namespace
+
+extern "C" int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p, const int32_t* d_starts, int32_t n,
+                                      int32_t* d_paths, void* stream_v, fw_walk_stats* stats) {
+  int rc = check_walk_args(g, p, d_starts, n, d_paths);
+  if (rc != FW_OK) return rc;
+  if (n > FW_WALK_NOALLOC_MAX_QUERIES) {
+    fw_set_error("fw_walk_device_noalloc: n = %d exceeds FW_WALK_NOALLOC_MAX_QUERIES = %d (split the batch and advance "
+                 "walker_base, or use fw_walk_device)", n, FW_WALK_NOALLOC_MAX_QUERIES);
+    return FW_ERR_INVALID;
+  }
+  hipStream_t stream = reinterpret_cast<hipStream_t>(stream_v);
+  const double t0 = now_ms();
+  NoAllocDevice* d = nullptr;
+  if ((rc = noalloc_device(&d)) != FW_OK) return rc;
+  Scratch* const scr = d->ptr;  // the device address; never the array's name
+
+  // the array keeps the last call's contents: the dispenser word and the counters start at zero (fill kernels, not
+  // memset nodes, so that a caller may capture the call's launches)
+  hipLaunchKernelGGL(fw_fill_i32_kernel, dim3(1), dim3(64), 0, stream, reinterpret_cast<int32_t*>(scr), 0,
+                     sizeof(Scratch) / sizeof(int32_t));
+  FW_HIP(hipGetLastError());
+  {
+    const size_t count = (size_t)n * (size_t)p->max_depth;  // -1 fill of the path matrix: src/walk.cu:398, :536
+    size_t blocks = (count + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(fw_fill_i32_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, d_paths, -1, count);
+    FW_HIP(hipGetLastError());
+  }
+  fw_kargs a;
+  fill_kargs(&a, g, p);  // park_threshold stays INT_MAX: one launch, walkers run whole walks
+  a.starts = d_starts;
+  a.paths = d_paths;
+  a.n = n;
+  a.dispenser = &scr->dispenser;
+  a.counters = scr->counters;
+  int grid_used = 0;
+  FW_HIP(hipEventRecord(d->ev0, stream));
+  rc = fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, 0u, stream, &grid_used);
+  if (rc != FW_OK) return rc;
+  FW_HIP(hipEventRecord(d->ev1, stream));
+  FW_HIP(hipStreamSynchronize(stream));
+  float ms = 0.0f;
+  FW_HIP(hipEventElapsedTime(&ms, d->ev0, d->ev1));
+  Scratch h;
+  FW_HIP(hipMemcpy(&h, scr, sizeof(h), hipMemcpyDeviceToHost));
+  if (stats) {
+    stats->kernel_ms = ms;
+    stats->total_ms = now_ms() - t0;
+    stats->steps = h.counters[0];
+    stats->sampled_edges = h.counters[1];
+    stats->launches = 1;
+    stats->grid = grid_used;
+    stats->walk_kernel_ms = ms;
+    stats->hub_kernel_ms = 0.0;
+    stats->hub_steps = 0;
+    stats->hub_sampled_edges = 0;
   }
   return FW_OK;
 }

@@ -199,6 +199,23 @@ int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const int32_t* d_
                    int32_t* d_paths, void* stream, fw_walk_stats* stats);
 
 /*
+ * fw_walk_device for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (walk_test allocates on every
+ * call, src/walk.cu:535-536).  Same arguments, same walks and same counters as fw_walk_device with
+ * park_threshold < 0 (one launch, walkers run their whole walks; parking never changes results, so the paths also
+ * equal fw_walk_device's under any park_threshold).  The launch scratch (query dispenser word and workload
+ * counters, 48 bytes) lives in a 256-byte array inside the library's device image, one copy per device, held
+ * until the process ends; the call makes no hipMalloc / hipFree / event creation after its first call on a
+ * device.  n is limited to FW_WALK_NOALLOC_MAX_QUERIES, the largest batch fw_walk_device itself serves with a
+ * single launch under its default rule (larger batches are what its parking pipeline and the lists it allocates
+ * are for): FW_ERR_INVALID beyond it.  All calls on one device share the array, so calls that overlap on one
+ * device (two host threads, two streams) race; calls one after the other are independent.
+ */
+#define FW_WALK_NOALLOC_MAX_QUERIES 65535
+int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p, const int32_t* d_starts, int32_t n,
+                           int32_t* d_paths, void* stream, fw_walk_stats* stats);
+
+/*
  * Batched walk over host queries: replaces walk_batch (src/walk.cu:576-649) with
  * timing_batch_async (two streams, double-buffered H2D / kernel / D2H, :373-466) or, when
  * sync != 0, timing_batch_sync (:468-523).  h_starts: int32[n]; h_paths: int32[n][max_depth],
