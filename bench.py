@@ -6,13 +6,15 @@ symmetrised R-MAT scale-24 graph (edge factor 16, a/b/c/d = .57/.19/.19/.05, wei
 Inputs (CSR, start vertices, path matrix) are resident in HBM before the timed region starts.
 
 Prints ONE JSON line with the walk-steps/s of the whole job, the HBM roofline of the walk path
-(algorithmic bytes of one pass / device time of that pass, measured with HIP events on the launch
-stream) and the CPU oracle timed on the host cores of the same box over a bounded prefix of the same
-queries.  With hub parking (the default for large batches) one pass is a short pipeline of launches --
+(bytes the kernels of one pass requested from memory, counted by the library in the run / device time
+of that pass, measured with HIP events on the launch stream; the algorithmic bytes every walker would
+read alone are reported beside it), one line per benchmark configuration measured after the timed
+region (`configs`) and the CPU oracle timed on the host cores of the same box over a bounded prefix
+of the same queries.  With hub parking (the default for large batches) one pass is a short pipeline of launches --
 fw_walk_zprs, then per round fw_hub_scan + fw_hub_batch + fw_walk_zprs -- and the HIP events bracket the whole
 pipeline, host-side round trips included.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-configs]
 """
 import argparse
 import importlib
@@ -37,22 +39,126 @@ WORKLOADS = {
     "metapath_rmat26": dict(scale=26, sym=False, app="metapath", depth=5, queries=10_000_000, labels=5),
 }
 HEADLINE = "deepwalk_rmat24_sym"
+CONFIG_OF = {"deepwalk_rmat22": "C2", "ppr_rmat22": "C3", "node2vec_rmat24_sym": "C4", "metapath_rmat26": "C5",
+             "deepwalk_rmat24_sym": "C4 graph, DeepWalk (headline)"}
 
-# HBM-side bytes of one pass (all launches of the walk pipeline) from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs, each scaled by what the same counter reads for the 1 GiB copy kernel (profiles/).
-# None for workloads that have not been measured.
-MEASURED_TRAFFIC_BYTES = {"deepwalk_rmat24_sym": 5.73e11, "node2vec_rmat24_sym": 5.24e13}
+# HBM-side bytes of one pass (all launches of the walk pipeline) as rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE saw them
+# on an earlier run of the same workload with the library defaults, each counter scaled by what it reads for the
+# 1 GiB copy kernel; the file under profiles/ holds the command and the per-kernel figures.  Reported beside the
+# bytes this run counts itself (roofline.requested_bytes), never instead of them.
+PROFILED_TRAFFIC = {
+    "deepwalk_rmat24_sym": (5.73e11, "profiles/walk_pipeline_deepwalk_rmat24sym_pmc.txt"),
+    "node2vec_rmat24_sym": (5.24e13, "profiles/fw_walk_zprs_node2vec_rmat24sym_pmc.txt"),
+}
 
 
-def algorithmic_bytes(app, steps, sampled_edges, queries, probe_terms=0):
-    """Bytes the algorithm has to touch: bias array once per visited neighbour + per-step and per-query words.
-
-    DeepWalk / PPR / MetaPath: 4*D + 16*S + 16*Q; node2vec: 8*D + 24*S + 16*Q (binary-search probes are
-    reported separately and not included).
-    """
+def algorithmic_bytes(app, steps, sampled_edges, queries):
+    """Bytes every walker would have to touch on its own: the bias array once per visited neighbour + per-step and
+    per-query words.  DeepWalk / PPR / MetaPath: 4*D + 16*S + 16*Q; node2vec: 8*D + 24*S + 16*Q (binary-search
+    probes not included)."""
     if app == "node2vec":
         return 8 * sampled_edges + 24 * steps + 16 * queries
     return 4 * sampled_edges + 16 * steps + 16 * queries
+
+
+def roofline_of(app, st, n, kernel_ms):
+    """HBM roofline of one pass from the run's own counters.  `achieved` is the rate of the bytes the kernels
+    requested from the memory system (lists as often as they were actually streamed + 64 bytes per scattered access,
+    counted by the library: fw_walk_stats.requested_bytes) over the device time of the pass, so `frac` is a fraction
+    of what the memory can deliver.  `algorithmic_rate` divides the bytes every walker would read alone
+    (4*D + 16*S + 16*Q) by the same time: with hub parking a list is read once per batch of walkers, so this figure
+    exceeds the peak and `reuse_factor` = algorithmic / requested says by how much lists were shared.  node2vec never
+    parks and its requested bytes leave out the probes of the adjacency test, so its algorithmic bytes are used."""
+    alg = algorithmic_bytes(app, st.steps, st.sampled_edges, n)
+    req = int(st.requested_bytes)
+    hbm = alg if app == "node2vec" or req == 0 else req
+    sec = kernel_ms * 1e-3
+    return {
+        "bound": "hbm", "achieved": hbm / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": hbm / sec / 1e9 / HBM_PEAK_GBS, "kernel_ms": kernel_ms,
+        "bytes_basis": "algorithmic" if hbm == alg else "requested (counted by the library in this run)",
+        "requested_bytes": req, "algorithmic_bytes": int(alg), "algorithmic_rate": alg / sec / 1e9,
+        "reuse_factor": alg / hbm,
+    }
+
+
+def make_graph(fw, wl):
+    return fw.Graph.rmat(wl["scale"], 16, 0.57, 0.19, 0.19, symmetrise=wl["sym"], w_lo=1.0, w_hi=100.0,
+                         n_labels=wl["labels"], make_weights=wl["app"] != "metapath", seed=1)
+
+
+def starts_of(g, wl):
+    if wl["queries"] == "all":
+        return np.arange(g.V, dtype=np.int32)
+    return np.random.RandomState(12345).randint(0, g.V, size=int(wl["queries"])).astype(np.int32)
+
+
+def app_id_of(fw, name):
+    return {"deepwalk": fw.APP_DEEPWALK, "ppr": fw.APP_PPR, "node2vec": fw.APP_NODE2VEC,
+            "metapath": fw.APP_METAPATH}[name]
+
+
+def one_config(fw, g, name, wl, passes, warmup, **overrides):
+    """`passes` passes of one configuration with the library defaults, device-resident inputs; a line of configs[]."""
+    starts = starts_of(g, wl)
+    n = len(starts)
+    params = fw.default_params(app=app_id_of(fw, wl["app"]), max_depth=wl["depth"] + 1, seed=1, **overrides)
+    d_starts = fw.DeviceBuffer.from_numpy(starts)
+    d_paths = fw.DeviceBuffer(n * params.max_depth * 4)
+    try:
+        for _ in range(warmup):
+            g.walk_device(params, d_starts, n, d_paths)
+        ms, st = [], None
+        for _ in range(passes):
+            st = g.walk_device(params, d_starts, n, d_paths)
+            ms.append(st.kernel_ms)
+    finally:
+        d_starts.free()
+        d_paths.free()
+    kernel_ms = float(np.mean(ms))
+    r = roofline_of(wl["app"], st, n, kernel_ms)
+    return {
+        "config": CONFIG_OF.get(name, name), "workload": name, "app": wl["app"], "vertices": g.V, "csr_entries": g.E,
+        "queries": n, "walk_steps_per_pass": int(st.steps), "passes": passes, "device_ms_per_pass": kernel_ms,
+        "steps_per_s": st.steps / (kernel_ms * 1e-3), "launches_per_pass": st.launches,
+        "frac": r["frac"], "achieved_GBs": r["achieved"], "bytes_basis": r["bytes_basis"],
+        "algorithmic_rate_GBs": r["algorithmic_rate"], "reuse_factor": r["reuse_factor"],
+    }
+
+
+def config1(fw):
+    """C1: directed uniform-random graph, 7,115 vertices, 103,689 distinct edges (no self-loops), weights U[1,5),
+    seed 1; 100 seeded uniform starts, length 80."""
+    rng = np.random.RandomState(1)
+    V, E = 7115, 103689
+    keys = np.empty(0, dtype=np.int64)
+    while len(keys) < E:
+        s = rng.randint(0, V, size=2 * E).astype(np.int64)
+        d = rng.randint(0, V, size=2 * E).astype(np.int64)
+        keys = np.unique(np.concatenate([keys, (s * V + d)[s != d]]))
+    keys = np.sort(rng.choice(keys, size=E, replace=False))
+    xadj = np.zeros(V + 1, dtype=np.uint32)
+    np.cumsum(np.bincount(keys // V, minlength=V), out=xadj[1:])
+    g = fw.Graph.from_csr(xadj, (keys % V).astype(np.int32), (1.0 + 4.0 * rng.random_sample(E)).astype(np.float32))
+    try:
+        wl = dict(app="deepwalk", depth=80, queries=100)
+        starts = rng.randint(0, V, size=100).astype(np.int32)
+        params = fw.default_params(app=fw.APP_DEEPWALK, max_depth=81, seed=1)
+        g.walk(params, starts)
+        ms, st = [], None
+        for _ in range(5):
+            _, st = g.walk(params, starts)
+            ms.append(st.kernel_ms)
+        kernel_ms = float(np.mean(ms))
+        r = roofline_of("deepwalk", st, 100, kernel_ms)
+        return {"config": "C1", "workload": "deepwalk_uniform_7115", "app": "deepwalk", "vertices": V, "csr_entries": E,
+                "queries": 100, "walk_steps_per_pass": int(st.steps), "passes": 5, "device_ms_per_pass": kernel_ms,
+                "steps_per_s": st.steps / (kernel_ms * 1e-3), "launches_per_pass": st.launches, "frac": r["frac"],
+                "achieved_GBs": r["achieved"], "bytes_basis": r["bytes_basis"],
+                "algorithmic_rate_GBs": r["algorithmic_rate"], "reuse_factor": r["reuse_factor"],
+                "note": "100 walks of 80 dependent steps: a latency measurement, not a bandwidth one"}
+    finally:
+        g.destroy()
 
 
 def main():
@@ -63,6 +169,8 @@ def main():
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
     ap.add_argument("--scale", type=int, default=0, help="override the R-MAT scale (smaller boxes / quick checks)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the one-pass report of the other configurations after the timed region")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
     ap.add_argument("--hub-threshold", type=int, default=-1)
     ap.add_argument("--wg-threads", type=int, default=0)
@@ -83,21 +191,16 @@ def main():
     wl = dict(WORKLOADS[args.workload])
     if args.scale:
         wl["scale"] = args.scale
-    app_id = {"deepwalk": fw.APP_DEEPWALK, "ppr": fw.APP_PPR, "node2vec": fw.APP_NODE2VEC,
-              "metapath": fw.APP_METAPATH}[wl["app"]]
+    defaults = not args.scale and args.park_threshold == 0 and args.hub_threshold < 0 and args.wg_threads == 0
 
     t0 = time.time()
-    g = fw.Graph.rmat(wl["scale"], 16, 0.57, 0.19, 0.19, symmetrise=wl["sym"], w_lo=1.0, w_hi=100.0,
-                      n_labels=wl["labels"], make_weights=wl["app"] != "metapath", seed=1)
+    g = make_graph(fw, wl)
     fw.check(fw.lib().fw_dev_sync())
     gen_s = time.time() - t0
 
-    if wl["queries"] == "all":
-        starts = np.arange(g.V, dtype=np.int32)
-    else:
-        starts = np.random.RandomState(12345).randint(0, g.V, size=int(wl["queries"])).astype(np.int32)
+    starts = starts_of(g, wl)
     n = len(starts)
-    params = fw.default_params(app=app_id, max_depth=wl["depth"] + 1, seed=1)
+    params = fw.default_params(app=app_id_of(fw, wl["app"]), max_depth=wl["depth"] + 1, seed=1)
     if args.hub_threshold >= 0:
         params.hub_threshold = args.hub_threshold
     if args.wg_threads:
@@ -125,13 +228,27 @@ def main():
         kernel_ms.append(last.kernel_ms)
     fw.check(fw.lib().fw_dev_sync())
     wall = time.perf_counter() - t0
+    d_starts.free()
+    d_paths.free()
 
     steps_per_pass = last.steps
     ms_per_step = wall * 1e3 / args.steps
     value = steps_per_pass * args.steps / wall
     avg_kernel_ms = float(np.mean(kernel_ms))
-    alg_bytes = algorithmic_bytes(wl["app"], last.steps, last.sampled_edges, n)
-    achieved = alg_bytes / (avg_kernel_ms * 1e-3) / 1e9
+    roofline = roofline_of(wl["app"], last, n, avg_kernel_ms)
+    roofline["kernel"] = "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_scan + fw_hub_batch pipeline"
+    # the profiler's view of the same workload (library defaults only: any override makes it another run)
+    prof = PROFILED_TRAFFIC.get(args.workload) if defaults and (last.launches > 1 or wl["app"] == "node2vec") else None
+    roofline["traffic"] = prof[0] if prof else None
+    if prof:
+        roofline["traffic_source"] = prof[1]
+        roofline["traffic_frac"] = prof[0] / (avg_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+    if last.launches > 1:
+        # per-kernel view of the last pass: each kernel's own HIP-event time and the steps it took
+        roofline["kernels"] = [
+            {"kernel": "fw_walk_zprs", "total_ms": last.walk_kernel_ms, "steps": int(last.steps - last.hub_steps)},
+            {"kernel": "fw_hub_scan + fw_hub_batch", "total_ms": last.hub_kernel_ms, "steps": int(last.hub_steps)},
+        ]
 
     out = {
         "metric": "walk steps/sec (1 GPU) + % of HBM roofline; R-MAT s24 DeepWalk len 80",
@@ -155,44 +272,42 @@ def main():
             "park_threshold": params.park_threshold, "launches_per_pass": last.launches, "grid": last.grid,
             "graph_gen_s": round(gen_s, 2),
         },
-        "roofline": {
-            "bound": "hbm",
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            # measured with the library defaults only: any override makes it another run
-            "traffic": MEASURED_TRAFFIC_BYTES.get(
-                args.workload if not args.scale and args.park_threshold == 0 and args.hub_threshold < 0
-                and args.wg_threads == 0 and (last.launches > 1 or wl["app"] == "node2vec") else None),
-            "kernel": "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_batch pipeline",
-            "kernel_ms": avg_kernel_ms,
-            "algorithmic_bytes": int(alg_bytes),
-        },
+        "roofline": roofline,
     }
-    if out["roofline"]["traffic"] is not None:
-        # what the memory actually moved per pass, as a rate over the same device time: with hub parking a list is
-        # read once per batch of walkers, so `achieved` (bytes every walker would read alone) exceeds the peak and
-        # measures reuse; this pair is the pipeline's real HBM rate
-        out["roofline"]["traffic_achieved"] = out["roofline"]["traffic"] / (avg_kernel_ms * 1e-3) / 1e9
-        out["roofline"]["traffic_frac"] = out["roofline"]["traffic_achieved"] / HBM_PEAK_GBS
-    if last.launches > 1:
-        # per-kernel view of the last pass: each kernel's own HIP-event time and the algorithmic bytes of the steps
-        # it took (what every walker would have to read on its own; fw_hub_batch reads a hub list once per batch
-        # of up to 64 walkers, so its figure measures reuse, not DRAM speed)
-        walk_b = algorithmic_bytes(wl["app"], last.steps - last.hub_steps, last.sampled_edges - last.hub_sampled_edges, n)
-        hub_b = algorithmic_bytes(wl["app"], last.hub_steps, last.hub_sampled_edges, 0)
-        out["roofline"]["kernels"] = [
-            {"kernel": "fw_walk_zprs", "total_ms": last.walk_kernel_ms, "algorithmic_bytes": int(walk_b),
-             "achieved": walk_b / (last.walk_kernel_ms * 1e-3) / 1e9, "steps": int(last.steps - last.hub_steps)},
-            {"kernel": "fw_hub_scan + fw_hub_batch", "total_ms": last.hub_kernel_ms, "algorithmic_bytes": int(hub_b),
-             "achieved": hub_b / (last.hub_kernel_ms * 1e-3) / 1e9, "steps": int(last.hub_steps)},
-        ]
 
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(fw, g, params, starts, args.cpu_seconds)
-
-    g.destroy()
+    if not args.no_configs and defaults and args.workload == HEADLINE:
+        # after the timed region: the headline without hub parking (every walker reads its lists itself, one launch:
+        # the walk kernel against the roofline on the bytes it touches) and one line per benchmark configuration
+        out["roofline"]["no_parking"] = one_config(fw, g, HEADLINE, wl, passes=1, warmup=0, park_threshold=-1)
+        configs = [config1(fw)]
+        configs.append(one_config(fw, g, "node2vec_rmat24_sym", WORKLOADS["node2vec_rmat24_sym"], passes=1, warmup=0))
+        cpu = None if args.no_cpu else cpu_baseline(fw, g, params, starts, args.cpu_seconds)
+        g.destroy()
+        g22 = make_graph(fw, WORKLOADS["deepwalk_rmat22"])
+        try:
+            configs.insert(1, one_config(fw, g22, "deepwalk_rmat22", WORKLOADS["deepwalk_rmat22"], passes=3, warmup=1))
+            configs.insert(2, one_config(fw, g22, "ppr_rmat22", WORKLOADS["ppr_rmat22"], passes=3, warmup=1))
+        finally:
+            g22.destroy()
+        g26 = make_graph(fw, WORKLOADS["metapath_rmat26"])
+        try:
+            configs.append(one_config(fw, g26, "metapath_rmat26", WORKLOADS["metapath_rmat26"], passes=3, warmup=1))
+        finally:
+            g26.destroy()
+        configs.append({
+            "config": CONFIG_OF[HEADLINE], "workload": HEADLINE, "app": wl["app"], "vertices": out["config"]["vertices"],
+            "csr_entries": out["config"]["csr_entries"], "queries": n, "walk_steps_per_pass": int(last.steps),
+            "passes": args.steps, "device_ms_per_pass": avg_kernel_ms, "steps_per_s": last.steps / (avg_kernel_ms * 1e-3),
+            "launches_per_pass": last.launches, "frac": roofline["frac"], "achieved_GBs": roofline["achieved"],
+            "bytes_basis": roofline["bytes_basis"], "algorithmic_rate_GBs": roofline["algorithmic_rate"],
+            "reuse_factor": roofline["reuse_factor"]})
+        out["configs"] = configs
+        if cpu is not None:
+            out["cpu_baseline"] = cpu
+    else:
+        if not args.no_cpu:
+            out["cpu_baseline"] = cpu_baseline(fw, g, params, starts, args.cpu_seconds)
+        g.destroy()
     print(json.dumps(out))
 
 

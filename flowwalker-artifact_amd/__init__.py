@@ -29,7 +29,7 @@ EXPORTED = [
     "fw_graph_create", "fw_graph_adopt_device", "fw_graph_destroy", "fw_graph_info", "fw_graph_is_sorted",
     "fw_graph_download", "fw_walk_device", "fw_walk_batch", "fw_host_alloc_pinned", "fw_host_free_pinned",
     "fw_gen_rmat", "fw_csr_read_header", "fw_csr_load", "fw_csr_write", "fw_graph_load",
-    "fw_graph_create_placed", "fw_graph_load_placed", "fw_walk_device_noalloc",
+    "fw_graph_create_placed", "fw_graph_load_placed", "fw_walk_device_noalloc", "fw_csr_sort_neighbours",
 ]
 
 
@@ -47,7 +47,7 @@ class WalkStats(C.Structure):
         ("kernel_ms", C.c_double), ("total_ms", C.c_double), ("steps", C.c_uint64),
         ("sampled_edges", C.c_uint64), ("launches", C.c_int32), ("grid", C.c_int32),
         ("walk_kernel_ms", C.c_double), ("hub_kernel_ms", C.c_double), ("hub_steps", C.c_uint64),
-        ("hub_sampled_edges", C.c_uint64),
+        ("hub_sampled_edges", C.c_uint64), ("requested_bytes", C.c_uint64),
     ]
 
 
@@ -112,6 +112,8 @@ def lib():
         L.fw_csr_read_header.argtypes = [C.c_char_p, C.POINTER(C.c_int32), C.POINTER(C.c_uint64)]
         L.fw_csr_load.argtypes = [C.c_char_p, C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.fw_csr_write.argtypes = [C.c_char_p, C.c_int32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.fw_csr_sort_neighbours.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                             C.POINTER(C.c_int64)]
         L.fw_graph_load.argtypes = [C.c_char_p, C.c_int, C.c_int, C.POINTER(C.c_void_p)]
         L.fw_graph_load_placed.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p)]
         _lib = L
@@ -180,6 +182,13 @@ def csr_write(prefix, xadj, adjncy, weight=None, label=None):
     label = None if label is None else np.ascontiguousarray(label, dtype=np.int32)
     check(lib().fw_csr_write(prefix.encode(), len(xadj) - 1, len(adjncy), _ptr(xadj), _ptr(adjncy), _ptr(weight),
                              _ptr(label)))
+
+
+def csr_sort_neighbours(xadj, adjncy, weight=None, label=None):
+    """Sorts the neighbour lists in place (weight / label follow their edges).  Returns the number of lists changed."""
+    n = C.c_int64()
+    check(lib().fw_csr_sort_neighbours(len(xadj) - 1, _ptr(xadj), _ptr(adjncy), _ptr(weight), _ptr(label), C.byref(n)))
+    return n.value
 
 
 class DeviceBuffer:

@@ -243,7 +243,8 @@ extern "C" int fw_graph_destroy(fw_graph* g) {
     }
   }
   release_park_cache(g);
-  void* index_ptrs[2] = {g->hub_index, g->hub_info};
+  for (hipEvent_t e : g->call_ev) if (e) (void)hipEventDestroy(e);
+  void* index_ptrs[3] = {g->hub_index, g->hub_info, g->call_scratch};
   for (void* p : index_ptrs) {
     if (p && hipFree(p) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
   }
@@ -357,21 +358,29 @@ extern "C" int fw_graph_info(const fw_graph* g, int32_t* V, uint64_t* E, int32_t
   return FW_OK;
 }
 
-extern "C" int fw_graph_is_sorted(const fw_graph* g, int* sorted) {
-  if (!g || !sorted) { fw_set_error("fw_graph_is_sorted: NULL argument"); return FW_ERR_INVALID; }
+// d_flag: one int of device memory to use (the caller's), or NULL: allocated and freed here.
+static int graph_sorted(const fw_graph* g, int* sorted, int* d_flag_in) {
   fw_graph* mg = const_cast<fw_graph*>(g);
   if (mg->sorted < 0) {
-    int* d_flag = nullptr;
-    FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_flag), sizeof(int)));
-    FW_HIP(hipMemset(d_flag, 0, sizeof(int)));
-    hipLaunchKernelGGL(fw_sorted_kernel, dim3(2048), dim3(256), 0, 0, g->xadj, g->adjncy, g->V, d_flag);
+    int* d_flag = d_flag_in;
+    if (!d_flag) FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_flag), sizeof(int)));
     int flag = 0;
-    FW_HIP(hipMemcpy(&flag, d_flag, sizeof(flag), hipMemcpyDeviceToHost));
-    FW_HIP(hipFree(d_flag));
+    int rc = fw_check_hip(hipMemset(d_flag, 0, sizeof(int)), "hipMemset(sorted flag)", __FILE__, __LINE__);
+    if (rc == FW_OK) {
+      hipLaunchKernelGGL(fw_sorted_kernel, dim3(2048), dim3(256), 0, 0, g->xadj, g->adjncy, g->V, d_flag);
+      rc = fw_check_hip(hipMemcpy(&flag, d_flag, sizeof(flag), hipMemcpyDeviceToHost), "hipMemcpy(sorted flag)", __FILE__, __LINE__);
+    }
+    if (!d_flag_in) (void)hipFree(d_flag);
+    if (rc != FW_OK) return rc;
     mg->sorted = flag ? 0 : 1;
   }
   *sorted = mg->sorted;
   return FW_OK;
+}
+
+extern "C" int fw_graph_is_sorted(const fw_graph* g, int* sorted) {
+  if (!g || !sorted) { fw_set_error("fw_graph_is_sorted: NULL argument"); return FW_ERR_INVALID; }
+  return graph_sorted(g, sorted, nullptr);
 }
 
 extern "C" int fw_graph_download(const fw_graph* g, uint32_t* h_xadj, int32_t* h_adjncy, float* h_weight,
@@ -393,8 +402,9 @@ extern "C" int fw_graph_download(const fw_graph* g, uint32_t* h_xadj, int32_t* h
 
 // ---- walks ---------------------------------------------------------------------------------------
 
+// d_flag: one int of device memory for the neighbour-order check of node2vec (NULL: allocated when needed).
 static int check_walk_args(const fw_graph* g, const fw_walk_params* p, const void* starts, int32_t n,
-                           const void* paths) {
+                           const void* paths, int* d_flag = nullptr) {
   if (!g || !p || !starts || !paths) { fw_set_error("walk: NULL argument"); return FW_ERR_INVALID; }
   if (n <= 0) { fw_set_error("walk: n must be positive (got %d)", n); return FW_ERR_INVALID; }
   if (p->max_depth < 1) { fw_set_error("walk: max_depth must be >= 1 (got %d)", p->max_depth); return FW_ERR_INVALID; }
@@ -423,6 +433,16 @@ static int check_walk_args(const fw_graph* g, const fw_walk_params* p, const voi
   if (p->app == FW_APP_NODE2VEC && !(p->p > 0.0f && p->q > 0.0f)) {
     fw_set_error("walk: p and q must be positive");
     return FW_ERR_INVALID;
+  }
+  if (p->app == FW_APP_NODE2VEC) {  // the adjacency test searches ascending lists (include/gpu_graph.cuh:97-118)
+    int sorted = 0;
+    const int rc = graph_sorted(g, &sorted, d_flag);  // one pass over the adjacency the first time, then cached
+    if (rc != FW_OK) return rc;
+    if (!sorted) {
+      fw_set_error("walk: node2vec needs strictly ascending neighbour lists and this graph has others "
+                   "(fw_csr_sort_neighbours sorts a host CSR before the upload)");
+      return FW_ERR_INVALID;
+    }
   }
   return FW_OK;
 }
@@ -548,7 +568,8 @@ constexpr int kParkCtrs = 16;                    // counters of a parking round
 // walkers); every other bucket gets one batch task per 64 walkers:
 // a workgroup task when its vertex is sampled at workgroup granularity (degree above hub_threshold), a wave task
 // otherwise.  ctrs (out): [3] workgroup tasks, [4] their dispenser, [5] wave tasks, [7] table tasks, [8] scan tasks,
-// [12] walkers in the fullest bucket when that is more than half of kTwoPassWalkers.
+// [12] walkers in the fullest bucket when that is more than half of kTwoPassWalkers, [13] walkers served by table
+// tasks, [14..15] (one 64-bit word) 16-byte quartets the round's batch and scan tasks stream.
 constexpr uint32_t kScanRun = 16;
 
 struct TaskPlan {
@@ -603,6 +624,21 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
     if (two_pass) t.row = hub_row * (uint32_t)labels + (uint32_t)t.slot * ngroups;
     const bool wg = (int32_t)t.deg > plan.hub_threshold;
     const uint32_t nb = (c + 63u) >> 6;
+    {
+      // what the round's hub launches will stream: a list once per batch task, or once by the scan tasks
+      const unsigned long long nq = c != 0u ? (((t.off & 3u) + t.deg + 3u) >> 2) : 0u;
+      unsigned long long quartets = two_pass ? nq : nq * nb;
+      uint32_t table_walkers = two_pass ? c : 0u;
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) {
+        quartets += __shfl_xor(quartets, d);
+        table_walkers += __shfl_xor(table_walkers, d);
+      }
+      if (lane == 0 && quartets != 0ull) {
+        atomicAdd(reinterpret_cast<unsigned long long*>(ctrs + 14), quartets);
+        if (table_walkers != 0u) atomicAdd(&ctrs[13], table_walkers);
+      }
+    }
     uint32_t x[kKinds];
     x[0] = !two_pass && wg ? nb : 0u;
     x[1] = !two_pass && !wg ? nb : 0u;
@@ -807,6 +843,7 @@ struct ParkBuffers {
   uint32_t* h_ctrs = nullptr;         // pinned mirror
   void* tmp = nullptr;                // scan temporary storage
   size_t scan_bytes = 0;
+  hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};  // timing events of the walk and the hub launches
 
   uint32_t* count(int parity) const { return buckets + (size_t)parity * n_buckets; }
   uint32_t* offset() const { return buckets + (size_t)2 * n_buckets; }
@@ -825,6 +862,7 @@ struct ParkBuffers {
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&wtasks), ntask * sizeof(fw_batch_task)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), kParkCtrs * sizeof(uint32_t)));
     FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), kParkCtrs * sizeof(uint32_t), hipHostMallocDefault));
+    for (hipEvent_t& e : ev) FW_HIP(hipEventCreate(&e));
     // the rows are an extra: without room for them every bucket is served by batch tasks
     if (rows_wanted != 0u) {
       // scan tasks: a list of G groups is cut into at most G / kScanRun + 1 runs, and no more lists are scanned in
@@ -859,6 +897,10 @@ struct ParkBuffers {
     void* dev[9] = {walked, sorted, out, resume, buckets, tasks, wtasks, ctrs, tmp};
     for (void* p : dev) if (p) (void)hipFree(p);
     if (h_ctrs) (void)hipHostFree(h_ctrs);
+    for (hipEvent_t& e : ev) {
+      if (e) (void)hipEventDestroy(e);
+      e = nullptr;
+    }
     walked = sorted = out = resume = nullptr;
     buckets = ctrs = h_ctrs = nullptr;
     tasks = wtasks = nullptr;
@@ -919,24 +961,31 @@ static int32_t resolve_park_threshold(const fw_graph* g, const fw_walk_params* p
 struct KernelTimes {
   double walk_ms = 0.0;
   double hub_ms = 0.0;
+  // what the parking pipeline asked of the memory system beyond the walk launches' own steps (see requested_bytes)
+  uint64_t hub_quartets = 0;     // 16-byte quartets streamed by batch and scan tasks
+  uint64_t table_walkers = 0;    // walkers served from a crowded hub's rows
+  uint64_t parked_records = 0;   // records parked by walk launches
+  uint64_t resume_entries = 0;   // records read back by walk launches
+  uint64_t sorted_records = 0;   // records moved by the counting sort (one per walker and round)
+  uint64_t bucket_passes = 0;    // buckets x rounds (scan, reset, task list)
 };
 
-// Records one event pair around a launch and adds its duration to *acc after the next stream sync.
+// Records one event pair around a launch and adds its duration to *acc after the next stream sync.  The events belong
+// to the parking buffers (created once with them, not per launch).
 struct TimedLaunch {
   hipEvent_t e0 = nullptr, e1 = nullptr;
+  bool open = false;
   int begin(hipStream_t s) {
-    FW_HIP(hipEventCreate(&e0));
-    FW_HIP(hipEventCreate(&e1));
     FW_HIP(hipEventRecord(e0, s));
+    open = true;
     return FW_OK;
   }
   int end(hipStream_t s) { FW_HIP(hipEventRecord(e1, s)); return FW_OK; }
   void collect(double* acc) {  // call after the stream has been synchronised
     float ms = 0.0f;
-    if (e0 && e1 && hipEventElapsedTime(&ms, e0, e1) == hipSuccess) *acc += ms;
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    e0 = e1 = nullptr;
+    if (open && hipEventElapsedTime(&ms, e0, e1) == hipSuccess) *acc += ms;
+    else (void)hipGetLastError();
+    open = false;
   }
 };
 
@@ -949,7 +998,6 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     return fw_launch_walk(a, p->app, p->sampler, p->wg_threads, p->grid, 0u, stream, grid_used);
   }
   const int labels = p->app == FW_APP_METAPATH ? p->schema_len : 1;
-  const size_t bucket_bytes = (size_t)pb->n_buckets * sizeof(uint32_t);
   a.park_threshold = park_threshold;
   a.n_labels_per_hub = labels;
   a.hub_index = g->hub_index;
@@ -982,6 +1030,8 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
 
   // Queues one walk launch (timed); the caller reads the counters back.
   TimedLaunch tw;
+  tw.e0 = pb->ev[0];
+  tw.e1 = pb->ev[1];
   uint32_t entries_hint = 0u;  // set before every queue_walk
   // the hint counts entries of the kind the grid rule was made for, lists of up to 124 neighbours (four or two to a
   // wave); with a higher parking threshold an entry is more work, about in proportion
@@ -1020,6 +1070,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   if (rc != FW_OK) return rc;
   if ((rc = read_back()) != FW_OK) return rc;
   tw.collect(&times->walk_ms);
+  times->parked_records += pb->h_ctrs[0];
   uint32_t n_out = 0;  // records in `out` (the previous batch launch's input size)
   uint32_t fullest = 0;  // walkers in the fullest bucket of the previous round
   uint32_t scan_tasks = 0;  // and its scan tasks
@@ -1066,6 +1117,9 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
       if ((rc = queue_walk(nullptr)) != FW_OK) return rc;
       if ((rc = read_back()) != FW_OK) return rc;
       tw.collect(&times->walk_ms);
+      times->resume_entries += m;
+      times->sorted_records += m;
+      times->bucket_passes += (uint64_t)pb->n_buckets;
       return FW_OK;
     }
     plan.two_pass_walkers = two_pass_possible && (n_out == 0u || fullest * 2u > kTwoPassWalkers) ? kTwoPassWalkers : 0xFFFFFFFFu;
@@ -1077,6 +1131,8 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     FW_HIP(hipGetLastError());
     h.bucket_out = pb->count(nxt);
     TimedLaunch th;
+    th.e0 = pb->ev[2];
+    th.e1 = pb->ev[3];
     if ((rc = th.begin(stream)) != FW_OK) return rc;
     if (plan.two_pass_walkers != 0xFFFFFFFFu) {
       // finds its task count on the device; sized by the round before (twice that many tasks still get a wave each)
@@ -1110,10 +1166,12 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     if ((rc = read_back()) != FW_OK) return rc;
     th.collect(&times->hub_ms);
     tw.collect(&times->walk_ms);
-    if (getenv("FW_DEBUG_ROUNDS"))
-      fprintf(stderr, "round: parked %llu (walk %u + again %u) wg_tasks %u wave_tasks %u table_tasks %u scan_tasks %u -> resume %u again %u, parked by the walk launch %u\n",
-              (unsigned long long)m, n_walked, n_again, pb->h_ctrs[3], pb->h_ctrs[5], pb->h_ctrs[7], pb->h_ctrs[8],
-              pb->h_ctrs[6], pb->h_ctrs[2], pb->h_ctrs[0]);
+    times->hub_quartets += *reinterpret_cast<const uint64_t*>(pb->h_ctrs + 14);
+    times->table_walkers += pb->h_ctrs[13];
+    times->parked_records += pb->h_ctrs[0];
+    times->resume_entries += pb->h_ctrs[6];
+    times->sorted_records += m;
+    times->bucket_passes += (uint64_t)pb->n_buckets;
     n_out = (uint32_t)m;
     fullest = pb->h_ctrs[12];
     resumed = pb->h_ctrs[6];
@@ -1125,11 +1183,58 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   return FW_OK;
 }
 
+// Bytes a call's kernels request from the memory system, from the counters of the run: lists are streamed in
+// 16-byte quartets, every scattered access (a path entry, a CSR offset pair, a parking index, a counter, the selected
+// neighbour) is one 64-byte line, records are 16 bytes.  See fw_walk_stats::requested_bytes.
+static uint64_t requested_bytes_model(const fw_walk_params* p, int32_t n, bool parked, int32_t park_threshold,
+                                      uint64_t walk_steps, uint64_t walk_edges, uint64_t hub_steps,
+                                      const KernelTimes& t) {
+  constexpr uint64_t kLine = 64, kRec = 16;
+  const bool n2v = p->app == FW_APP_NODE2VEC;
+  uint64_t b = 0;
+  // walk launches.  A list is read from its first aligned quartet on (about 12 bytes of padding per step); lists of
+  // up to 64 quartets bring their neighbours along with the biases, longer ones fetch the selected neighbour alone.
+  const bool short_lists = parked && park_threshold <= 252;
+  const uint64_t per_entry_array = (n2v || short_lists) ? 2 : 1;
+  b += per_entry_array * (4 * walk_edges + 12 * walk_steps);
+  if (!short_lists) b += kLine * walk_steps;                      // adjncy[off + sel]
+  b += (kLine + kLine + (parked ? kLine : 0)) * walk_steps;       // path entry, xadj pair, parking index
+  b += (4 + kLine + kLine + (parked ? kLine : 0)) * (uint64_t)n;  // start vertex, path[0], xadj pair, parking index
+  if (parked) {
+    b += (kRec + kLine) * t.parked_records;                       // record out, bucket counter
+    b += (kRec + kLine + kLine) * t.resume_entries;               // record in, xadj pair, parking index
+    // hub launches: the lists, and per walker its record in and out, the selected neighbour, the path entry, the
+    // parking index of the new vertex and that vertex's bucket counter
+    b += 16 * t.hub_quartets;
+    b += (2 * kRec + 4 * kLine) * hub_steps;
+    b += 8 * kLine * t.table_walkers;                             // pivots, lane row, prefix, four quartets of one lane
+    // counting sort, compaction, task list, reset, bucket scan
+    b += (kRec + kLine + kLine) * t.sorted_records + 2 * kRec * t.sorted_records;
+    b += (12 + 8 + 8) * t.bucket_passes;
+  }
+  return b;
+}
+
 struct Scratch {  // dispenser word + workload counters of the two kernels, 48 bytes per launch slot
   uint32_t dispenser;
   uint32_t pad;
   unsigned long long counters[4];
   unsigned long long pad2;
+};
+
+// One walk call at a time per graph: the parking index, the parking lists and the launch record are cached in the
+// graph, so a second call that started while one is running would rebuild or overwrite them under it.
+struct BusyGuard {
+  fw_graph* g;
+  bool held;
+  explicit BusyGuard(const fw_graph* graph) : g(const_cast<fw_graph*>(graph)), held(false) {
+    int expected = 0;
+    held = g->busy.compare_exchange_strong(expected, 1);
+    if (!held) fw_set_error("walk: another walk call is running on this fw_graph (one call at a time per graph; "
+                            "make a second fw_graph, or use fw_walk_device_noalloc, to walk concurrently)");
+  }
+  bool ok() const { return held; }
+  ~BusyGuard() { if (held) g->busy.store(0); }
 };
 
 static double now_ms() {
@@ -1141,6 +1246,8 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
                               int32_t* d_paths, void* stream_v, fw_walk_stats* stats) {
   int rc = check_walk_args(g, p, d_starts, n, d_paths);
   if (rc != FW_OK) return rc;
+  BusyGuard busy(g);
+  if (!busy.ok()) return FW_ERR_INVALID;
   hipStream_t stream = reinterpret_cast<hipStream_t>(stream_v);
   const double t0 = now_ms();
 
@@ -1159,21 +1266,18 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
     pb = cached_park_buffers(const_cast<fw_graph*>(g), (size_t)n, g->n_hubs * labels, two_pass_rows(g, labels));
     use_pb = pb != nullptr;  // no room for the parking lists: walk without parking (same results, one launch)
   }
-  Scratch* d_scr = nullptr;
-  FW_HIP(hipMalloc(reinterpret_cast<void**>(&d_scr), sizeof(Scratch)));
-  hipEvent_t ev0 = nullptr, ev1 = nullptr;
-  auto cleanup = [&]() {
-    if (ev0) (void)hipEventDestroy(ev0);
-    if (ev1) (void)hipEventDestroy(ev1);
-    if (d_scr) (void)hipFree(d_scr);
-  };
+  // the launch record and the two timing events are the graph's, made once
+  fw_graph* mg = const_cast<fw_graph*>(g);
+  if (!mg->call_scratch) FW_HIP(hipMalloc(&mg->call_scratch, sizeof(Scratch)));
+  for (hipEvent_t& e : mg->call_ev) if (!e) FW_HIP(hipEventCreate(&e));
+  Scratch* const d_scr = static_cast<Scratch*>(mg->call_scratch);
+  const hipEvent_t ev0 = mg->call_ev[0], ev1 = mg->call_ev[1];
+  auto cleanup = [&]() {};
 #define FW_TRY(call)                                                 \
   do {                                                               \
     int rc_ = fw_check_hip((call), #call, __FILE__, __LINE__);       \
     if (rc_ != FW_OK) { cleanup(); return rc_; }                     \
   } while (0)
-  FW_TRY(hipEventCreate(&ev0));
-  FW_TRY(hipEventCreate(&ev1));
   FW_TRY(hipMemsetAsync(d_scr, 0, sizeof(Scratch), stream));
   // -1 fill of the path matrix: src/walk.cu:398, :536
   FW_TRY(hipMemsetAsync(d_paths, 0xFF, (size_t)n * (size_t)p->max_depth * sizeof(int32_t), stream));
@@ -1208,6 +1312,8 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
     stats->hub_kernel_ms = times.hub_ms;
     stats->hub_steps = h.counters[2];
     stats->hub_sampled_edges = h.counters[3];
+    stats->requested_bytes = requested_bytes_model(p, n, launches > 1, park_threshold, h.counters[0], h.counters[1],
+                                                   h.counters[2], times);
   }
   return FW_OK;
 }
@@ -1221,7 +1327,7 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
 // All calls on a device share the array: calls that overlap on one device race on it.
 
 static __device__ __align__(256) unsigned char scratch[256];
-static_assert(sizeof(Scratch) <= sizeof(scratch), "the launch scratch record must fit the static array");
+static_assert(sizeof(Scratch) <= 128 && sizeof(scratch) >= 128 + sizeof(int), "launch record in the first half, flag behind it");
 
 namespace {
 constexpr int kNoAllocMaxDevices = 64;
@@ -1263,7 +1369,11 @@ int noalloc_device(NoAllocDevice** out) {
 
 extern "C" int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p, const int32_t* d_starts, int32_t n,
                                       int32_t* d_paths, void* stream_v, fw_walk_stats* stats) {
-  int rc = check_walk_args(g, p, d_starts, n, d_paths);
+  NoAllocDevice* d = nullptr;
+  int rc = noalloc_device(&d);
+  if (rc != FW_OK) return rc;
+  // (the neighbour-order check of a graph's first node2vec call keeps its flag behind the launch record)
+  rc = check_walk_args(g, p, d_starts, n, d_paths, reinterpret_cast<int*>(reinterpret_cast<unsigned char*>(d->ptr) + 128));
   if (rc != FW_OK) return rc;
   if (n > FW_WALK_NOALLOC_MAX_QUERIES) {
     fw_set_error("fw_walk_device_noalloc: n = %d exceeds FW_WALK_NOALLOC_MAX_QUERIES = %d (split the batch and advance "
@@ -1272,8 +1382,6 @@ extern "C" int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p
   }
   hipStream_t stream = reinterpret_cast<hipStream_t>(stream_v);
   const double t0 = now_ms();
-  NoAllocDevice* d = nullptr;
-  if ((rc = noalloc_device(&d)) != FW_OK) return rc;
   Scratch* const scr = d->ptr;  // the device address; never the array's name
 
   // the array keeps the last call's contents: the dispenser word and the counters start at zero (fill kernels, not
@@ -1316,6 +1424,7 @@ extern "C" int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p
     stats->hub_kernel_ms = 0.0;
     stats->hub_steps = 0;
     stats->hub_sampled_edges = 0;
+    stats->requested_bytes = requested_bytes_model(p, n, false, INT_MAX, h.counters[0], h.counters[1], 0, KernelTimes());
   }
   return FW_OK;
 }
@@ -1324,6 +1433,8 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
                              uint32_t batch_size, int sync, int32_t* h_paths, fw_walk_stats* stats) {
   int rc = check_walk_args(g, p, h_starts, n, h_paths);
   if (rc != FW_OK) return rc;
+  BusyGuard busy(g);
+  if (!busy.ok()) return FW_ERR_INVALID;
   if (batch_size == 0) {  // autobatch, src/main.cu:259-271 with the default 512 MB headroom
     size_t free_b = 0, total_b = 0;
     rc = fw_device_mem_info(&free_b, &total_b);
@@ -1445,6 +1556,9 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     stats->grid = grid_used;
     stats->walk_kernel_ms = times.hub_ms == 0.0 && times.walk_ms == 0.0 ? kernel_ms : times.walk_ms;
     stats->hub_kernel_ms = times.hub_ms;
+    stats->requested_bytes = requested_bytes_model(p, n, times.hub_ms != 0.0, park_threshold,
+                                                   stats->steps - stats->hub_steps,
+                                                   stats->sampled_edges - stats->hub_sampled_edges, stats->hub_steps, times);
   }
   return FW_OK;
 }

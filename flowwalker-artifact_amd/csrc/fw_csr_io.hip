@@ -10,6 +10,7 @@
 #include <string.h>
 #include <sys/stat.h>
 
+#include <algorithm>
 #include <string>
 #include <vector>
 
@@ -111,6 +112,44 @@ extern "C" int fw_csr_write(const char* prefix, int32_t V, uint64_t E, const uin
   if ((rc = write_all(p + "_edge.bin", h_adjncy, (size_t)E * 4, nullptr, 0)) != FW_OK) return rc;
   if (h_weight && (rc = write_all(p + "_weight.bin", h_weight, (size_t)E * 4, nullptr, 0)) != FW_OK) return rc;
   if (h_label && (rc = write_all(p + "_label.bin", h_label, (size_t)E * 4, nullptr, 0)) != FW_OK) return rc;
+  return FW_OK;
+}
+
+// Sorts every neighbour list that is not ascending, carrying weight and label with their edges.  The reference's
+// converter writes lists in insertion order (data/EdgeListToCSR.cpp:182-191) while node2vec's adjacency test
+// binary-searches them (include/gpu_graph.cuh:97-118); the sampling law does not depend on the order of a list.
+extern "C" int fw_csr_sort_neighbours(int32_t V, const uint32_t* h_xadj, int32_t* h_adjncy, float* h_weight,
+                                      int32_t* h_label, int64_t* lists_sorted) {
+  if (V <= 0 || !h_xadj || !h_adjncy) { fw_set_error("fw_csr_sort_neighbours: bad argument"); return FW_ERR_INVALID; }
+  int64_t touched = 0;
+  std::vector<uint32_t> perm;
+  std::vector<int32_t> ta, tl;
+  std::vector<float> tw;
+  for (int32_t v = 0; v < V; ++v) {
+    const uint32_t b = h_xadj[v], e = h_xadj[v + 1];
+    bool ascending = true;
+    for (uint32_t i = b + 1; i < e && ascending; ++i) ascending = h_adjncy[i - 1] <= h_adjncy[i];
+    if (ascending) continue;
+    ++touched;
+    const uint32_t d = e - b;
+    perm.resize(d);
+    for (uint32_t i = 0; i < d; ++i) perm[i] = i;
+    std::stable_sort(perm.begin(), perm.end(), [&](uint32_t x, uint32_t y) { return h_adjncy[b + x] < h_adjncy[b + y]; });
+    ta.resize(d);
+    for (uint32_t i = 0; i < d; ++i) ta[i] = h_adjncy[b + perm[i]];
+    std::copy(ta.begin(), ta.end(), h_adjncy + b);
+    if (h_weight) {
+      tw.resize(d);
+      for (uint32_t i = 0; i < d; ++i) tw[i] = h_weight[b + perm[i]];
+      std::copy(tw.begin(), tw.end(), h_weight + b);
+    }
+    if (h_label) {
+      tl.resize(d);
+      for (uint32_t i = 0; i < d; ++i) tl[i] = h_label[b + perm[i]];
+      std::copy(tl.begin(), tl.end(), h_label + b);
+    }
+  }
+  if (lists_sorted) *lists_sorted = touched;
   return FW_OK;
 }
 

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "flowwalker.h"
 
 // A vertex that walkers are parked on: its CSR range, so that building batch tasks is a streaming pass.
@@ -37,6 +39,9 @@ struct fw_graph {
   int32_t* hub_index = nullptr;       // int32[V]: position in hub_info, -1 (not parked on) or -2 (degree 0)
   struct fw_hub_info* hub_info = nullptr;  // [n_hubs]
   void* park_cache = nullptr;         // the parking lists of the last fw_walk_device call, kept for the next one
+  void* call_scratch = nullptr;       // launch record (dispenser word + counters) of fw_walk_device, allocated once
+  hipEvent_t call_ev[2] = {nullptr, nullptr};  // and its two timing events
+  std::atomic<int> busy{0};           // a walk call is running on this graph (the caches above are per graph)
 };
 
 constexpr int FW_EDGE_PAD = 4;

@@ -239,6 +239,15 @@ int main(int argc, char** argv) {
     std::lognormal_distribution<float> dist(0.0f, 3.0f);
     for (size_t i = 0; i < weight.size(); ++i) weight[i] = dist(gen);
   }
+  if (F.node2vec) {
+    // the adjacency test binary-searches neighbour lists (include/gpu_graph.cuh:97-118), but the reference's own
+    // converter writes them in insertion order (data/EdgeListToCSR.cpp:182-191, its shipped wiki-Vote files
+    // included): lists that do not ascend are sorted here, weights moving with their edges (same sampling law)
+    int64_t changed = 0;
+    if (fw_csr_sort_neighbours(V, xadj.data(), adjncy.data(), weight.data(), nullptr, &changed) != FW_OK)
+      return fail("sorting neighbour lists");
+    if (changed) printf("node2vec: %lld neighbour lists were not ascending and have been sorted\n", (long long)changed);
+  }
   printf("Graph load (success): %d verts, %llu edges %g second(s)\n", V, (unsigned long long)E, now_s() - t_load);
   printf("Read Graph!\n");
   int32_t max_deg = 0, max_idx = 0;
@@ -252,14 +261,6 @@ int main(int argc, char** argv) {
                              F.metapath ? label.data() : nullptr, F.umgraph ? FW_GRAPH_HOST_PINNED : FW_GRAPH_DEVICE,
                              &g) != FW_OK)
     return fail("uploading the graph");
-  if (F.node2vec) {  // the adjacency test binary-searches neighbour lists (include/gpu_graph.cuh:97-118)
-    int sorted = 0;
-    if (fw_graph_is_sorted(g, &sorted) != FW_OK) return fail("checking neighbour order");
-    if (!sorted) {
-      fprintf(stderr, "flowwalker: --node2vec needs ascending neighbour lists; this graph has unsorted lists\n");
-      return 2;
-    }
-  }
 
   fw_walk_params P;
   fw_walk_params_default_for(&P, F.deepwalk ? FW_APP_DEEPWALK : F.ppr ? FW_APP_PPR : F.node2vec ? FW_APP_NODE2VEC : FW_APP_METAPATH);

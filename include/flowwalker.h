@@ -79,6 +79,13 @@ typedef struct {
   double hub_kernel_ms;       /* sum over fw_hub_batch launches (and the fw_hub_scan launches in front of them) */
   uint64_t hub_steps;         /* steps taken in fw_hub_batch (included in steps) */
   uint64_t hub_sampled_edges; /* their source degrees (included in sampled_edges) */
+  /* Bytes the call's kernels requested from the memory system, from the run's own counters: every list pass in
+   * 16-byte quartets (a list is read once per walker step by the walk kernel, once per batch of up to 64 walkers
+   * or once per round by the hub kernels), 64 bytes for every scattered access (path entry, xadj pair, parking
+   * index, bucket counter, selected neighbour), 16 bytes per walker record moved.  node2vec: the probes of its
+   * adjacency test are not included.  What sits between the algorithmic bytes of src/main.cu:93-111
+   * (4 * sampled_edges + ...) and what the HBM counters of a profiler see. */
+  uint64_t requested_bytes;
 } fw_walk_stats;
 
 typedef struct fw_graph fw_graph; /* device CSR mirror: include/gpu_graph.cuh:28-78 */
@@ -159,7 +166,8 @@ int fw_graph_destroy(fw_graph* g);
 /* V, E and the maximum degree / its vertex (graph::print_max_degree, include/graph.cuh:209-220). */
 int fw_graph_info(const fw_graph* g, int32_t* V, uint64_t* E, int32_t* max_degree, int32_t* max_degree_vertex);
 
-/* 1 when every neighbour list is strictly ascending (needed by node2vec: include/gpu_graph.cuh:97-118). */
+/* 1 when every neighbour list is strictly ascending (needed by node2vec: include/gpu_graph.cuh:97-118; the walk
+ * entry points return FW_ERR_INVALID for FW_APP_NODE2VEC on a graph where this is 0). */
 int fw_graph_is_sorted(const fw_graph* g, int* sorted);
 
 /* Copies the device CSR back (any output pointer may be NULL). */
@@ -180,6 +188,14 @@ int fw_csr_load(const char* prefix, int32_t V, uint64_t E, uint32_t* h_xadj, int
 /* Writes the four files (weight / label only when given). */
 int fw_csr_write(const char* prefix, int32_t V, uint64_t E, const uint32_t* h_xadj, const int32_t* h_adjncy,
                  const float* h_weight, const int32_t* h_label);
+/*
+ * Host-side: sorts every neighbour list that is not ascending, weight and label moving with their edges
+ * (any of the two may be NULL); *lists_sorted (may be NULL) = number of lists that were changed.  The reference's
+ * converter writes lists in insertion order (data/EdgeListToCSR.cpp:182-191) although its node2vec binary-searches
+ * them (include/gpu_graph.cuh:97-118); the sampling law does not depend on the order inside a list.
+ */
+int fw_csr_sort_neighbours(int32_t V, const uint32_t* h_xadj, int32_t* h_adjncy, float* h_weight, int32_t* h_label,
+                           int64_t* lists_sorted);
 /* load + fw_graph_create: graph::graph(...) followed by gpu_graph::gpu_graph(graph*) (src/main.cu:312-325). */
 int fw_graph_load(const char* prefix, int want_weight, int want_label, fw_graph** out);
 /* The same with the edge arrays placed as fw_graph_create_placed does (--umgraph, src/main.cu:48). */

@@ -164,7 +164,29 @@ typedef struct {
   uint32_t prev_off;  /* CSR range of prev (node2vec) */
   int32_t prev_deg;
   int32_t want_label; /* metapath: schema[step % schema_len] */
+  /* exhaustive tests only (fw_oracle_enumerate_draw): draw (force_stream, force_index) of the step takes
+   * force_value instead of its Philox word, and the walker-independent rows of a group are kept between calls */
+  int force;
+  uint32_t force_stream, force_index;
+  float force_value;
+  struct group_rows* cache;
+  uint64_t cache_groups;
 } bias_ctx;
+
+enum { FW_EL = FW_GROUP_QUARTETS * FW_QUAD };
+/* What a group's part of the sampler computes before any draw: the 16 biases of every lane, the lane totals and
+ * their wave scan. */
+typedef struct group_rows {
+  float x[FW_WAVE][FW_EL];
+  float q[FW_WAVE], I[FW_WAVE];
+  int valid;
+} group_rows;
+
+/* n-th uniform of stream `stream` at (walker, step) */
+static float step_draw(const bias_ctx* c, uint32_t walker, uint32_t step, uint32_t stream, uint32_t n) {
+  if (c->force && stream == c->force_stream && n == c->force_index) return c->force_value;
+  return u24(draw_bits(c->p->seed, walker, step, stream, n));
+}
 
 /* include/gpu_graph.cuh:97-112 */
 static int sorted_contains(const int32_t* arr, int32_t size, int32_t target) {
@@ -226,8 +248,7 @@ static int pick_by_prefix(const float* v, const float* prefix, int n, float targ
 static int32_t group_sample(const bias_ctx* c, uint32_t off, int32_t deg, int nw, uint32_t walker,
                             uint32_t step) {
   if (deg <= 0) return -1;
-  enum { U = FW_GROUP_QUARTETS, EL = FW_GROUP_QUARTETS * FW_QUAD, G = FW_WAVE * FW_GROUP_QUARTETS };
-  const uint64_t seed = c->p->seed;
+  enum { U = FW_GROUP_QUARTETS, EL = FW_EL, G = FW_WAVE * FW_GROUP_QUARTETS };
   const uint64_t a0 = (uint64_t)off & ~(uint64_t)(FW_QUAD - 1);
   const uint64_t end = (uint64_t)off + (uint64_t)deg;
   const uint64_t nq = (end - a0 + FW_QUAD - 1) / FW_QUAD;
@@ -240,42 +261,47 @@ static int32_t group_sample(const bias_ctx* c, uint32_t off, int32_t deg, int nw
     int32_t sel = -1;
     uint32_t nd = 0;
     for (uint64_t g = (uint64_t)wv; g < ngroups; g += (uint64_t)nw) {
-      float x[FW_WAVE][EL];
-      float q[FW_WAVE], I[FW_WAVE];
-      for (int l = 0; l < FW_WAVE; ++l) {
-        float s = 0.0f;
-        for (int j = 0; j < U; ++j) {
-          const uint64_t k = g * G + (uint64_t)j * FW_WAVE + (uint64_t)l;
-          for (int e = 0; e < FW_QUAD; ++e) {
-            const uint64_t a = a0 + FW_QUAD * k + (uint64_t)e;
-            const float b = (k < nq && a >= off && a < end) ? bias_at(c, a) : 0.0f;
-            x[l][j * FW_QUAD + e] = b;
-            s = s + b;
+      group_rows local;
+      group_rows* r = (c->cache && g < c->cache_groups) ? &c->cache[g] : &local;
+      if (r == &local || !r->valid) {
+        for (int l = 0; l < FW_WAVE; ++l) {
+          float s = 0.0f;
+          for (int j = 0; j < U; ++j) {
+            const uint64_t k = g * G + (uint64_t)j * FW_WAVE + (uint64_t)l;
+            for (int e = 0; e < FW_QUAD; ++e) {
+              const uint64_t a = a0 + FW_QUAD * k + (uint64_t)e;
+              const float b = (k < nq && a >= off && a < end) ? bias_at(c, a) : 0.0f;
+              r->x[l][j * FW_QUAD + e] = b;
+              s = s + b;
+            }
           }
+          r->q[l] = s;
+          r->I[l] = s;
         }
-        q[l] = s;
-        I[l] = s;
+        fw_oracle_wave_scan(r->I);
+        r->valid = 1;
       }
-      fw_oracle_wave_scan(I);
+      const float* q = r->q;
+      const float* I = r->I;
       const float T = I[FW_WAVE - 1];
       const float Snew = S + T;
       const float lhs = Snew * u;
       if (lhs > Sj) {
-        const float u2 = u24(draw_bits(seed, walker, step, (uint32_t)wv, nd++));
+        const float u2 = step_draw(c, walker, step, (uint32_t)wv, nd++);
         const float target = u2 * T;
         const int lane = pick_by_prefix(q, I, FW_WAVE, target);
         /* lane >= 0: acceptance implies T > 0, hence some q > 0 */
         float pre[EL];
         float e = I[lane] - q[lane];
         for (int i = 0; i < EL; ++i) {
-          e = e + x[lane][i];
+          e = e + r->x[lane][i];
           pre[i] = e;
         }
-        const int pick = pick_by_prefix(x[lane], pre, EL, target);
+        const int pick = pick_by_prefix(r->x[lane], pre, EL, target);
         const uint64_t k = g * G + (uint64_t)(pick / FW_QUAD) * FW_WAVE + (uint64_t)lane;
         sel = (int32_t)(a0 + FW_QUAD * k + (uint64_t)(pick % FW_QUAD) - off);
         Sj = Snew;
-        u = u24(draw_bits(seed, walker, step, (uint32_t)wv, nd++));
+        u = step_draw(c, walker, step, (uint32_t)wv, nd++);
       }
       S = Snew;
     }
@@ -287,7 +313,7 @@ static int32_t group_sample(const bias_ctx* c, uint32_t off, int32_t deg, int nw
   float J[16];
   for (int wv = 0; wv < nw; ++wv) J[wv] = W[wv];
   row_scan(J, nw);
-  const float u3 = u24(draw_bits(seed, walker, step, FW_STREAM_WAVE, 0u));
+  const float u3 = step_draw(c, walker, step, FW_STREAM_WAVE, 0u);
   const float target = u3 * J[nw - 1];
   const int wv = pick_by_prefix(W, J, nw, target);
   return wv < 0 ? -1 : wsel[wv];
@@ -300,6 +326,7 @@ int32_t fw_oracle_sample(const fw_oracle_graph* g, const fw_oracle_params* p, in
   bias_ctx c;
   c.g = g; c.p = p; c.prev = prev;
   c.prev_off = 0; c.prev_deg = 0;
+  c.force = 0; c.cache = NULL; c.cache_groups = 0;
   if (prev >= 0) { c.prev_off = g->xadj[prev]; c.prev_deg = (int32_t)(g->xadj[prev + 1] - g->xadj[prev]); }
   c.want_label = (p->app == FW_APP_METAPATH && p->schema_len > 0) ? p->schema[step % (uint32_t)p->schema_len] : 0;
   uint32_t off = g->xadj[cur];
@@ -344,8 +371,9 @@ static void walk_one(const fw_oracle_graph* g, const fw_oracle_params* p, int32_
  * (include/walker.cuh:1342, :1379-1381).  steps / edges as src/main.cu:93-104.
  * nthreads <= 0: all cores (OpenMP schedule(dynamic) over walkers).
  */
-int fw_oracle_walk(const fw_oracle_graph* g, const fw_oracle_params* p, const int32_t* starts, int64_t n,
-                   int32_t* paths, uint64_t* steps_out, uint64_t* edges_out, int nthreads) {
+static int walk_many(const fw_oracle_graph* g, const fw_oracle_params* p, const int32_t* starts,
+                     const uint32_t* walker_ids, int64_t n, int32_t* paths, uint64_t* steps_out, uint64_t* edges_out,
+                     int nthreads) {
   if (p->wg_threads % FW_WAVE != 0 || p->wg_threads > FW_MAX_GROUP || p->wg_threads < FW_WAVE) return -1;
   if (p->app == FW_APP_METAPATH && (p->schema_len <= 0 || p->schema_len > FW_MAX_SCHEMA)) return -1;
   uint64_t steps = 0, edges = 0;
@@ -357,13 +385,27 @@ int fw_oracle_walk(const fw_oracle_graph* g, const fw_oracle_params* p, const in
 #pragma omp parallel for schedule(dynamic, 64) reduction(+ : steps, edges)
   for (int64_t q = 0; q < n; ++q) {
     uint64_t s = 0, e = 0;
-    walk_one(g, p, starts[q], p->walker_base + (uint32_t)q, paths + (uint64_t)q * p->max_depth, &s, &e);
+    const uint32_t walker = walker_ids ? walker_ids[q] : p->walker_base + (uint32_t)q;
+    walk_one(g, p, starts[q], walker, paths + (uint64_t)q * p->max_depth, &s, &e);
     steps += s;
     edges += e;
   }
   if (steps_out) *steps_out = steps;
   if (edges_out) *edges_out = edges;
   return 0;
+}
+
+int fw_oracle_walk(const fw_oracle_graph* g, const fw_oracle_params* p, const int32_t* starts, int64_t n,
+                   int32_t* paths, uint64_t* steps_out, uint64_t* edges_out, int nthreads) {
+  return walk_many(g, p, starts, NULL, n, paths, steps_out, edges_out, nthreads);
+}
+
+/* The same for chosen rows of a larger job: query i is the walk of global walker id walker_ids[i] (draws are
+ * addressed by walker id, so row r of a job equals this walk with walker_ids[i] = walker_base + r). */
+int fw_oracle_walk_ids(const fw_oracle_graph* g, const fw_oracle_params* p, const int32_t* starts,
+                       const uint32_t* walker_ids, int64_t n, int32_t* paths, uint64_t* steps_out,
+                       uint64_t* edges_out, int nthreads) {
+  return walk_many(g, p, starts, walker_ids, n, paths, steps_out, edges_out, nthreads);
 }
 
 int fw_oracle_num_threads(void) {
@@ -391,4 +433,85 @@ int32_t fw_oracle_sequential_reservoir(const float* w, const float* u, int32_t n
     }
   }
   return pick;
+}
+
+/* ---- exhaustive enumeration of one draw (tests only) ------------------------------------------ */
+
+/*
+ * A sampling step is a deterministic function of its uniforms, and a uniform has only 2^24 values.  For a list
+ * of `deg` biases whose first element sits at absolute CSR index `off` (0..3: only the alignment matters), sampled by `nw`
+ * waves, this runs the step once for every value v * 2^-24 of draw number `index` of stream `stream` (stream w =
+ * the draws of wave w: target of its first accepted group, jump uniform, target of the next accepted group, ...;
+ * FW_STREAM_WAVE, index 0 = the draw that combines the waves) while all other draws keep their Philox words for
+ * (seed, walker, step), and counts how often each local index is returned: counts[i + 1] for index i, counts[0]
+ * for -1.  The exact law of those counts follows from the prefix sums of the biases alone.
+ */
+int fw_oracle_enumerate_draw(const float* bias, int32_t deg, uint32_t off, int32_t nw, uint32_t stream, uint32_t index,
+                             uint64_t seed, uint32_t walker, uint32_t step, uint64_t* counts) {
+  if (deg <= 0 || nw < 1 || nw > 16 || off > 3u) return -1; /* only off mod 4 matters: pass 0..3 */
+  float* padded = (float*)calloc((size_t)off + (size_t)deg + FW_QUAD, sizeof(float));
+  if (!padded) return -1;
+  memcpy(padded + off, bias, (size_t)deg * sizeof(float));
+  fw_oracle_params p;
+  memset(&p, 0, sizeof(p));
+  p.app = FW_APP_DEEPWALK;
+  p.seed = seed;
+  /* a graph whose weight array is addressed like a CSR that holds this list at `off` */
+  fw_oracle_graph g;
+  g.V = 1; g.xadj = NULL; g.adjncy = NULL; g.label = NULL;
+  g.weight = padded;
+  const uint64_t ngroups = (((uint64_t)(off & 3u) + (uint64_t)deg + 3u) / 4u + FW_WAVE * FW_GROUP_QUARTETS - 1) /
+                           (FW_WAVE * FW_GROUP_QUARTETS);
+  for (int32_t i = 0; i <= deg; ++i) counts[i] = 0;
+  int failed = 0;
+#pragma omp parallel
+  {
+    group_rows* cache = (group_rows*)calloc((size_t)ngroups, sizeof(group_rows));
+    uint64_t* mine = (uint64_t*)calloc((size_t)deg + 1, sizeof(uint64_t));
+    if (!cache || !mine) {
+#pragma omp atomic write
+      failed = 1;
+    } else {
+      bias_ctx c;
+      memset(&c, 0, sizeof(c));
+      c.g = &g; c.p = &p; c.prev = -1;
+      c.force = 1; c.force_stream = stream; c.force_index = index;
+      c.cache = cache; c.cache_groups = ngroups;
+#pragma omp for schedule(static)
+      for (int64_t v = 0; v < (1 << 24); ++v) {
+        c.force_value = (float)v * 0x1p-24f;
+        const int32_t s = group_sample(&c, off, deg, nw, walker, step);
+        mine[s + 1] += 1;
+      }
+#pragma omp critical
+      for (int32_t i = 0; i <= deg; ++i) counts[i] += mine[i];
+    }
+    free(cache);
+    free(mine);
+  }
+  free(padded);
+  return failed ? -1 : 0;
+}
+
+/* The same step for one forced value of that draw: the local index it returns (-1: none). */
+int32_t fw_oracle_sample_forced(const float* bias, int32_t deg, uint32_t off, int32_t nw, uint32_t stream, uint32_t index,
+                                float value, uint64_t seed, uint32_t walker, uint32_t step) {
+  if (deg <= 0 || nw < 1 || nw > 16 || off > 3u) return -2;
+  float* padded = (float*)calloc((size_t)off + (size_t)deg + FW_QUAD, sizeof(float));
+  if (!padded) return -2;
+  memcpy(padded + off, bias, (size_t)deg * sizeof(float));
+  fw_oracle_params p;
+  memset(&p, 0, sizeof(p));
+  p.app = FW_APP_DEEPWALK;
+  p.seed = seed;
+  fw_oracle_graph g;
+  g.V = 1; g.xadj = NULL; g.adjncy = NULL; g.label = NULL;
+  g.weight = padded;
+  bias_ctx c;
+  memset(&c, 0, sizeof(c));
+  c.g = &g; c.p = &p; c.prev = -1;
+  c.force = 1; c.force_stream = stream; c.force_index = index; c.force_value = value;
+  const int32_t sel = group_sample(&c, off, deg, nw, walker, step);
+  free(padded);
+  return sel;
 }

@@ -50,6 +50,13 @@ def lib():
                                      C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.c_int]
         L.fw_oracle_walk.restype = C.c_int
         L.fw_oracle_num_threads.restype = C.c_int
+        L.fw_oracle_enumerate_draw.argtypes = [C.c_void_p, C.c_int32, C.c_uint32, C.c_int32, C.c_uint32, C.c_uint32,
+                                               C.c_uint64, C.c_uint32, C.c_uint32, C.c_void_p]
+        L.fw_oracle_sample_forced.argtypes = [C.c_void_p, C.c_int32, C.c_uint32, C.c_int32, C.c_uint32, C.c_uint32,
+                                              C.c_float, C.c_uint64, C.c_uint32, C.c_uint32]
+        L.fw_oracle_sample_forced.restype = C.c_int32
+        L.fw_oracle_walk_ids.argtypes = [C.POINTER(OracleGraph), C.POINTER(OracleParams), C.c_void_p, C.c_void_p,
+                                         C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
         L.fw_oracle_sequential_reservoir.argtypes = [C.c_void_p, C.c_void_p, C.c_int32]
         L.fw_oracle_sequential_reservoir.restype = C.c_int32
         for name in ("fw_ref_sampler_thread", "fw_ref_sampler_zprs", "fw_ref_sampler_dprs"):
@@ -137,6 +144,18 @@ def walk(graph, params, starts, nthreads=0):
     return paths, steps.value, edges.value
 
 
+def walk_ids(graph, params, starts, walker_ids, nthreads=0):
+    """Walks of chosen global walker ids (rows of a larger job): returns the path rows."""
+    starts = np.ascontiguousarray(starts, dtype=np.int32)
+    ids = np.ascontiguousarray(walker_ids, dtype=np.uint32)
+    assert len(ids) == len(starts)
+    paths = np.empty((len(starts), params.max_depth), dtype=np.int32)
+    rc = lib().fw_oracle_walk_ids(C.byref(graph.c), C.byref(params), starts.ctypes.data, ids.ctypes.data, len(starts),
+                                  paths.ctypes.data, None, None, nthreads)
+    assert rc == 0, "oracle rejected the parameters"
+    return paths
+
+
 def sequential_reservoir(w, u):
     w = np.ascontiguousarray(w, dtype=np.float32)
     u = np.ascontiguousarray(u, dtype=np.float32)
@@ -156,3 +175,25 @@ def ref_sample_many(kind, w, u, width=32):
     if rc != 0:
         raise ValueError("fw_ref_sample_many: bad arguments")
     return out
+
+
+STREAM_WAVE = 0x40000000
+
+
+def enumerate_draw(bias, off, nw, stream, index, seed=1, walker=0, step=0):
+    """Counts, over all 2^24 values of one uniform of a sampling step, how often each local index is picked.
+    Returns int64[deg + 1]: entry 0 counts "no pick" (-1), entry i + 1 counts index i."""
+    bias = np.ascontiguousarray(bias, dtype=np.float32)
+    counts = np.zeros(len(bias) + 1, dtype=np.uint64)
+    rc = lib().fw_oracle_enumerate_draw(bias.ctypes.data, len(bias), off, nw, stream, index, seed, walker, step,
+                                        counts.ctypes.data)
+    if rc != 0:
+        raise ValueError("fw_oracle_enumerate_draw failed")
+    return counts.astype(np.int64)
+
+
+def sample_forced(bias, off, nw, stream, index, value, seed=1, walker=0, step=0):
+    """The local index one sampling step returns when one of its uniforms is forced to `value`."""
+    bias = np.ascontiguousarray(bias, dtype=np.float32)
+    return int(lib().fw_oracle_sample_forced(bias.ctypes.data, len(bias), off, nw, stream, index, float(value), seed,
+                                             walker, step))

@@ -171,3 +171,60 @@ def test_umgraph_keeps_edges_on_the_host(gpu, graph_files, tmp_path):
     text = _run("--input", prefix, "--deepwalk", "--all", "--d=10", "--seed=9", "--umgraph", "--savepaths", out)
     assert "umgraph: edge arrays stay in pinned host memory" in text
     assert (np.fromfile(out, dtype=np.int32).reshape(V, 11) == ref).all()
+
+
+def _shuffled_lists(csr, seed):
+    """The same graph with every neighbour list in random order (weights and labels move with their edges)."""
+    xadj, adj, w, lab = (a.copy() for a in csr)
+    rng = np.random.RandomState(seed)
+    for v in range(len(xadj) - 1):
+        b, e = int(xadj[v]), int(xadj[v + 1])
+        perm = rng.permutation(e - b)
+        adj[b:e], w[b:e], lab[b:e] = adj[b:e][perm], w[b:e][perm], lab[b:e][perm]
+    return xadj, adj, w, lab
+
+
+def test_node2vec_on_unsorted_lists(gpu, graph_files, tmp_path):
+    """The reference's converter writes neighbour lists in insertion order (data/EdgeListToCSR.cpp:182-191) and its
+    README runs --node2vec on such files.  The command line sorts them at load (weights follow their edges), so the
+    walks equal those on the sorted graph; the C ABI refuses node2vec on an unsorted device graph instead of
+    computing wrong biases."""
+    prefix, csr = graph_files
+    V = len(csr[0]) - 1
+    shuffled = _shuffled_lists(csr, seed=4)
+    assert (shuffled[1] != csr[1]).any()
+    sp = str(tmp_path / "shuffled")
+    gpu.csr_write(sp, *shuffled)
+    out = str(tmp_path / "n2v.bin")
+    text = _run("--input", sp, "--node2vec", "--n=500", "--seq", "--d=12", "--seed=21", "--dprs", "--savepaths", out)
+    assert re.search(r"node2vec: \d+ neighbour lists were not ascending and have been sorted", text)
+    ref, _, _ = orc.walk(orc.Graph(*csr), orc.make_params(app=2, max_depth=13, seed=21, hub_threshold=(1 << 31) - 1),
+                         np.arange(500, dtype=np.int32))
+    assert (np.fromfile(out, dtype=np.int32).reshape(500, 13) == ref).all()
+
+    g = gpu.Graph.from_csr(*shuffled)
+    try:
+        assert not g.is_sorted()
+        with pytest.raises(gpu.FlowWalkerError) as e:
+            g.walk(gpu.default_params(app=gpu.APP_NODE2VEC, max_depth=5), np.arange(10, dtype=np.int32))
+        assert e.value.status == 1 and "ascending" in str(e.value)
+        g.walk(gpu.default_params(app=gpu.APP_DEEPWALK, max_depth=5), np.arange(10, dtype=np.int32))  # others do not care
+    finally:
+        g.destroy()
+
+
+REF_WIKI = "/root/reference/data/wiki-Vote"
+
+
+@pytest.mark.skipif(not os.path.exists(REF_WIKI + "_xadj.bin"), reason="the reference's data directory is not mounted here")
+def test_readme_node2vec_command_on_the_shipped_graph(gpu, tmp_path):
+    """`flowwalker --input ../data/wiki-Vote --node2vec --n=100 --dprs` (README.md:99-105) on the reference's own files,
+    3,990 of whose 7,115 lists are not ascending."""
+    out = str(tmp_path / "wiki.bin")
+    text = _run("--input", REF_WIKI, "--node2vec", "--n=100", "--seq", "--dprs", "--seed=3", "--savepaths", out)
+    assert "node2vec: 3990 neighbour lists were not ascending and have been sorted" in text
+    xadj, adj, w, _ = gpu.csr_read(REF_WIKI)
+    assert gpu.csr_sort_neighbours(xadj, adj, w) == 3990
+    ref, _, _ = orc.walk(orc.Graph(xadj, adj, w), orc.make_params(app=2, max_depth=81, seed=3, hub_threshold=(1 << 31) - 1),
+                         np.arange(100, dtype=np.int32))
+    assert (np.fromfile(out, dtype=np.int32).reshape(100, 81) == ref).all()

@@ -63,7 +63,7 @@ def test_ppr_lengths(gpu, hub_graph):
     obs = np.bincount(L[ok], minlength=d + 1)[1:]
     # dead ends are rare here; compare the remaining walks with the geometric law
     assert deadend.mean() < 0.2
-    assert chisquare(obs, exp * obs.sum()).pvalue > 0.001 or deadend.mean() > 0
+    assert chisquare(obs, exp * obs.sum()).pvalue > 0.01
     assert abs(L[ok].mean() - 1 / tp) < 0.2
 
 

@@ -1,10 +1,32 @@
-"""The benchmark configurations at their real sizes, checked through size-independent properties
-(the oracle would need minutes to hours at these sizes): start column, -1 suffix, every hop a CSR edge, workload
-counters recomputed from the paths, and byte-identical output under a different launch shape."""
+"""The benchmark configurations at their real sizes and with the library's default parameters.  The whole output is
+checked through size-independent properties (the oracle would need minutes to hours for all of it): start column, -1
+suffix, every hop a CSR edge, workload counters recomputed from the paths, byte-identical output under a different
+launch shape.  Draws are addressed by walker id, so any row of the full job equals the oracle's walk of that walker:
+the first rows, the last rows and the rows that start on the highest-degree vertices are compared bit for bit."""
 import numpy as np
 import pytest
 
+import fw_oracle_binding as orc
+
 pytestmark = pytest.mark.gpu
+
+
+def _check_rows_against_oracle(xadj, adj, w, lab, p, starts, paths, k=2000, walker_base=0):
+    """Rows [0, k), [n - k, n) and the (at most k) rows that start on the k highest-degree vertices."""
+    og = orc.Graph(xadj, adj, w, lab)
+    n = len(starts)
+    deg = np.diff(xadj.astype(np.int64))
+    top = np.argpartition(deg, len(deg) - k)[len(deg) - k:]
+    is_top = np.zeros(len(deg), dtype=bool)
+    is_top[top] = True
+    hub_rows = np.nonzero(is_top[starts])[0][:k]
+    rows = np.unique(np.concatenate([np.arange(min(k, n)), np.arange(max(n - k, 0), n), hub_rows]))
+    op = orc.from_walk_params(p)
+    ref = orc.walk_ids(og, op, starts[rows], (rows + walker_base).astype(np.uint32))
+    bad = np.nonzero((paths[rows] != ref).any(axis=1))[0]
+    assert len(bad) == 0, "row %d differs:\n gpu %s\n ref %s" % (rows[bad[0]], paths[rows[bad[0]]], ref[bad[0]])
+    print("oracle rows compared: %d (of which start on a top-%d vertex: %d, max degree %d)" % (
+        len(rows), k, len(hub_rows), deg.max()), flush=True)
 
 
 def _check_paths(xadj, adj, paths, starts, st, max_depth, sample=200000, label=None, schema=None):
@@ -44,6 +66,7 @@ def test_config2_deepwalk_rmat22(gpu):
         p = gpu.default_params(app=gpu.APP_DEEPWALK, max_depth=81, seed=1)
         paths, st = g.walk_batch(p, starts, batch_size=0)                       # --all: autobatch
         L = _check_paths(xadj, adj, paths, starts, st, 81)
+        _check_rows_against_oracle(xadj, adj, w, None, p, starts, paths)
         deg = np.diff(xadj.astype(np.int64))
         assert (L[deg == 0] == 1).all()                                         # sinks: the walk is its start
         p2 = gpu.default_params(app=gpu.APP_DEEPWALK, max_depth=81, seed=1, grid=97)
@@ -61,28 +84,35 @@ def test_config3_ppr_rmat22(gpu):
         p = gpu.default_params(app=gpu.APP_PPR, max_depth=81, tp=0.2, seed=1)
         paths, st = g.walk(p, starts)
         L = _check_paths(xadj, adj, paths, starts, st, 81)
+        _check_rows_against_oracle(xadj, adj, w, None, p, starts, paths)
         assert L.max() <= 81
     finally:
         g.destroy()
 
 
 def test_config4_rmat24_symmetrised(gpu):
-    """Headline graph: DeepWalk from every vertex and node2vec (p = 2, q = 0.5) on a 2M-query prefix."""
+    """Headline graph: DeepWalk and node2vec (p = 2, q = 0.5), one query per vertex each, library defaults."""
     g = gpu.Graph.rmat(24, 16, symmetrise=True, seed=1)
     try:
         assert g.is_sorted()
-        xadj, adj, _, _ = g.download(weights=False)
+        xadj, adj, w, _ = g.download()
         starts = np.arange(g.V, dtype=np.int32)
         p = gpu.default_params(app=gpu.APP_DEEPWALK, max_depth=81, seed=1)
+        print("deepwalk, %d queries" % g.V, flush=True)
         paths, st = g.walk(p, starts)
+        assert st.launches > 3 and st.hub_steps > 0                             # the default rule parks at this size
         L = _check_paths(xadj, adj, paths, starts, st, 81, sample=50000)
         deg = np.diff(xadj.astype(np.int64))
         assert (L[deg > 0] == 81).all()                                         # undirected: no dead ends
+        _check_rows_against_oracle(xadj, adj, w, None, p, starts, paths)
         del paths
-        sub = starts[:2_000_000]
         p = gpu.default_params(app=gpu.APP_NODE2VEC, max_depth=81, p=2.0, q=0.5, seed=1)
-        paths, st = g.walk(p, sub)
-        _check_paths(xadj, adj, paths, sub, st, 81, sample=50000)
+        print("node2vec, %d queries" % g.V, flush=True)
+        paths, st = g.walk(p, starts)
+        print("node2vec done: %.0f ms" % st.kernel_ms, flush=True)
+        L = _check_paths(xadj, adj, paths, starts, st, 81, sample=50000)
+        assert (L[deg > 0] == 81).all()
+        _check_rows_against_oracle(xadj, adj, w, None, p, starts, paths, k=700)
     finally:
         g.destroy()
 
@@ -98,6 +128,7 @@ def test_config5_metapath_rmat26(gpu):
         p = gpu.default_params(app=gpu.APP_METAPATH, max_depth=6, schema=schema, seed=1)
         paths, st = g.walk(p, starts)
         _check_paths(xadj, adj, paths, starts, st, 6, sample=500000, label=lab, schema=schema)
+        _check_rows_against_oracle(xadj, adj, None, lab, p, starts, paths, k=20000)
     finally:
         g.destroy()
 
@@ -106,8 +137,6 @@ def test_csr_offsets_above_two_to_the_31(gpu):
     """A CSR with more than 2^31 entries (the format's offsets are uint32, include/graph.cuh:93-136): the walkers
     live on the vertices whose lists start above 2^31, among them eight lists of 200,000 neighbours (workgroup
     sampler, crowded buckets) and 32,760 of 520 (wave sampler, parked or not).  Bit-exact against the oracle."""
-    import fw_oracle_binding as orc
-
     V, d, n_hubs, d_hub, C = 1 << 22, 520, 8, 200_000, 1 << 15
     deg = np.full(V, d, dtype=np.int64)
     deg[-n_hubs:] = d_hub
@@ -155,7 +184,6 @@ def test_path_matrix_of_more_than_two_to_the_32_entries(gpu):
     index for every query past 53 million.  The first and the last rows equal the oracle's walks with the same
     walker ids (draws are addressed by walker id), with parking (crowded buckets of millions) and without."""
     import _graphs
-    import fw_oracle_binding as orc
 
     xadj, adj, w, lab = _graphs.hub_graph(V=12000, hub_degrees=(9000, 2500, 700), base_degree=5, seed=11)
     n, depth, k = 54_000_000, 81, 4000

@@ -331,3 +331,61 @@ def test_randomized_configurations(gpu):
                 assert (st.steps, st.sampled_edges) == (steps, edges), (hubs, kw)
         finally:
             g.destroy()
+
+
+def test_one_walk_call_at_a_time_per_graph(gpu):
+    """The parking index, the parking lists and the launch record are cached in the fw_graph, so a second call on
+    the same graph while one is running is refused with a status code (it used to race); afterwards the graph works
+    as before, and a second graph walks while the first one is busy."""
+    import threading
+    import time
+
+    csr = _graphs.hub_graph(V=30000, hub_degrees=(20000, 8000), base_degree=8, seed=5)
+    g = gpu.Graph.from_csr(*csr)
+    g2 = gpu.Graph.from_csr(*csr)
+    n = 400000
+    starts = np.random.RandomState(1).randint(0, 30000, size=n).astype(np.int32)
+    long_p = gpu.default_params(app=gpu.APP_NODE2VEC, max_depth=81, seed=3)
+    short_p = gpu.default_params(app=gpu.APP_DEEPWALK, max_depth=5, seed=3)
+    d_starts = gpu.DeviceBuffer.from_numpy(starts)
+    d_long = gpu.DeviceBuffer(n * 81 * 4)
+    d_short = gpu.DeviceBuffer(100 * 5 * 4)
+    state = {"stop": False, "calls": 0, "error": None}
+
+    def keep_busy():  # one long call after the other, for at most ten seconds
+        t_end = time.time() + 10.0
+        try:
+            while not state["stop"] and time.time() < t_end:
+                try:
+                    g.walk_device(long_p, d_starts, n, d_long)
+                    state["calls"] += 1
+                except gpu.FlowWalkerError as e:  # the other thread's short call held the graph: that is the rule too
+                    if "another walk call" not in str(e):
+                        raise
+        except Exception as e:  # noqa: BLE001 - reported by the main thread
+            state["error"] = e
+
+    try:
+        th = threading.Thread(target=keep_busy)
+        th.start()
+        refused = False
+        t_end = time.time() + 9.0
+        while time.time() < t_end and th.is_alive() and not refused:
+            try:
+                g.walk_device(short_p, d_starts, 100, d_short)  # may slip in between two long calls: try again
+            except gpu.FlowWalkerError as e:
+                assert e.status == 1 and "another walk call" in str(e)
+                refused = True
+                g2.walk_device(short_p, d_starts, 100, d_short)  # a second graph is independent
+        state["stop"] = True
+        th.join()
+        assert state["error"] is None, state["error"]
+        assert refused, "no call was refused while %d long calls ran" % state["calls"]
+        paths, _ = g.walk(long_p, starts[:2000])  # the graph is free again and walks as before
+        ref, _ = g2.walk(long_p, starts[:2000])
+        assert (paths == ref).all()
+    finally:
+        for b in (d_starts, d_long, d_short):
+            b.free()
+        g.destroy()
+        g2.destroy()

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol(fw):
 def test_struct_layouts_match_the_header(fw):
     # fw_walk_params: 6 int32 + 64 int32 + 3 float + uint32 + uint64 + 2 int32
     assert C.sizeof(fw.WalkParams) == 6 * 4 + 64 * 4 + 3 * 4 + 4 + 8 + 8
-    assert C.sizeof(fw.WalkStats) == 8 + 8 + 8 + 8 + 4 + 4 + 8 + 8 + 8 + 8
+    assert C.sizeof(fw.WalkStats) == 8 + 8 + 8 + 8 + 4 + 4 + 8 + 8 + 8 + 8 + 8
     assert C.sizeof(fw.RmatParams) == 48
 
 
@@ -193,3 +193,22 @@ def test_cli_flag_surface(fw, tmp_path):
     src = np.repeat(np.arange(7115), np.diff(xadj.astype(np.int64)))
     assert (src != adj).all() and len(np.unique(src * 7115 + adj)) == 103689
     assert w.min() >= 1.0 and w.max() < 5.0
+
+
+def test_sort_neighbours_moves_weights_and_labels_with_their_edges(fw):
+    """fw_csr_sort_neighbours: every list ascending afterwards, the (neighbour, weight, label) triples of a vertex
+    unchanged as a set, lists that already ascend untouched."""
+    import _graphs
+    xadj, adj, w, lab = _graphs.uniform_graph(500, 6000, seed=2)
+    rng = np.random.RandomState(0)
+    a2, w2, l2 = adj.copy(), w.copy(), lab.copy()
+    shuffled = 0
+    for v in range(0, 500, 2):                                   # every other list in random order
+        b, e = int(xadj[v]), int(xadj[v + 1])
+        perm = rng.permutation(e - b)
+        if (perm != np.arange(e - b)).any():
+            shuffled += 1
+        a2[b:e], w2[b:e], l2[b:e] = a2[b:e][perm], w2[b:e][perm], l2[b:e][perm]
+    assert fw.csr_sort_neighbours(xadj, a2, w2, l2) == shuffled
+    assert (a2 == adj).all() and (w2 == w).all() and (l2 == lab).all()   # uniform_graph's lists ascend, no duplicates
+    assert fw.csr_sort_neighbours(xadj, a2, w2, l2) == 0
