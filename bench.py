@@ -175,6 +175,9 @@ def main():
     ap.add_argument("--hub-threshold", type=int, default=-1)
     ap.add_argument("--wg-threads", type=int, default=0)
     ap.add_argument("--park-threshold", type=int, default=0, help="0 = library default, -1 = hub parking off")
+    ap.add_argument("--sampler", default="native", choices=["native", "ref_zprs", "ref_dprs"],
+                    help="native = this engine's sampler; ref_zprs / ref_dprs = the reference's own samplers and round "
+                         "structure restated for 64-lane waves (ablation baseline, hub_threshold 1024 unless given)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run the plain copy kernel on 1 GiB (what rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE are "
                          "scaled against)")
@@ -191,7 +194,8 @@ def main():
     wl = dict(WORKLOADS[args.workload])
     if args.scale:
         wl["scale"] = args.scale
-    defaults = not args.scale and args.park_threshold == 0 and args.hub_threshold < 0 and args.wg_threads == 0
+    defaults = (not args.scale and args.park_threshold == 0 and args.hub_threshold < 0 and args.wg_threads == 0
+                and args.sampler == "native")
 
     t0 = time.time()
     g = make_graph(fw, wl)
@@ -206,6 +210,10 @@ def main():
     if args.wg_threads:
         params.wg_threads = args.wg_threads
     params.park_threshold = args.park_threshold
+    if args.sampler != "native":
+        params.sampler = fw.SAMPLER_REF_ZPRS if args.sampler == "ref_zprs" else fw.SAMPLER_REF_DPRS
+        if args.hub_threshold < 0:
+            params.hub_threshold = 1024  # THRESHOLD of the reference (include/walker.cuh:29)
     d_starts = fw.DeviceBuffer.from_numpy(starts)
     d_paths = fw.DeviceBuffer(n * params.max_depth * 4)
 
@@ -236,7 +244,8 @@ def main():
     value = steps_per_pass * args.steps / wall
     avg_kernel_ms = float(np.mean(kernel_ms))
     roofline = roofline_of(wl["app"], last, n, avg_kernel_ms)
-    roofline["kernel"] = "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_scan + fw_hub_batch pipeline"
+    roofline["kernel"] = ("fw_walk_ref" if args.sampler != "native" else
+                          "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_scan + fw_hub_batch pipeline")
     # the profiler's view of the same workload (library defaults only: any override makes it another run)
     prof = PROFILED_TRAFFIC.get(args.workload) if defaults and (last.launches > 1 or wl["app"] == "node2vec") else None
     roofline["traffic"] = prof[0] if prof else None
@@ -269,7 +278,8 @@ def main():
             "vertices": g.V, "csr_entries": g.E, "queries": n,
             "walk_steps_per_pass": int(last.steps), "sampled_edges_per_pass": int(last.sampled_edges),
             "wg_threads": params.wg_threads, "hub_threshold": params.hub_threshold,
-            "park_threshold": params.park_threshold, "launches_per_pass": last.launches, "grid": last.grid,
+            "park_threshold": params.park_threshold, "sampler": args.sampler, "launches_per_pass": last.launches,
+            "grid": last.grid,
             "graph_gen_s": round(gen_s, 2),
         },
         "roofline": roofline,

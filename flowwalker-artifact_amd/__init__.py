@@ -18,7 +18,7 @@ LIB_PATH = os.environ.get("FLOWWALKER_LIB") or os.path.join(_PKG, "lib", "libflo
 
 FW_MAX_SCHEMA = 64
 APP_DEEPWALK, APP_PPR, APP_NODE2VEC, APP_METAPATH = 0, 1, 2, 3
-SAMPLER_ZPRS, SAMPLER_DPRS = 0, 1
+SAMPLER_ZPRS, SAMPLER_DPRS, SAMPLER_REF_ZPRS, SAMPLER_REF_DPRS, SAMPLER_REF_STATIC = 0, 1, 2, 3, 0x100
 FW_OK = 0
 GRAPH_DEVICE, GRAPH_HOST_PINNED = 0, 1
 

@@ -945,6 +945,7 @@ static uint64_t two_pass_rows(const fw_graph* g, int labels) {
 // Decides whether a call parks walkers, and at which degree.  Returns INT_MAX for "no".
 static int32_t resolve_park_threshold(const fw_graph* g, const fw_walk_params* p, int32_t n) {
   if (p->app == FW_APP_NODE2VEC) return INT_MAX;  // its biases depend on the walker: nothing to share
+  if (p->sampler != FW_SAMPLER_ZPRS && p->sampler != FW_SAMPLER_DPRS) return INT_MAX;  // the reference's engine: one launch
   if (p->park_threshold < 0) return INT_MAX;
   if (p->park_threshold == 0) {
     if (n < kMinParkBatch) return INT_MAX;  // too few walkers to meet

@@ -184,6 +184,11 @@ int fw_check_hip(hipError_t e, const char* what, const char* file, int line);
 int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, uint32_t entries_hint,
                    hipStream_t stream, int* grid_used);
 
+// Launches the reference's walk engine restated for 64-lane waves (sampler = FW_SAMPLER_REF_ZPRS / _DPRS, optionally
+// with FW_SAMPLER_REF_STATIC).  grid = 0: twice the resident set.
+int fw_launch_ref_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int grid, hipStream_t stream,
+                       int* grid_used);
+
 // Launches the hub batch kernel.  tasks_hint: about how many wave-sized pieces of work it will find (sizes the grid;
 // 0 = no idea: one resident set).
 int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, uint32_t tasks_hint,

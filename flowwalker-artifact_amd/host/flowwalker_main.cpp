@@ -13,12 +13,16 @@
 // smaller n: src/main.cu:165), errors return a non-zero status with a message instead of exit() inside a
 // macro, --lognorm draws its weights from a seeded host generator, --umgraph keeps the edge arrays in pinned host
 // memory that the kernels read over the bus (the reference uses managed memory that migrates by page,
-// include/gpu_graph.cuh:46-54), and --walkmode selects the ablation levels of THIS engine (the reference's levels,
-// README.md:152-163, name optimisations of its CUDA kernels that have no counterpart here):
-//   --walkmode=9 / 10  the walk kernel alone, every list sampled by one wave (no workgroup sampler, no parking;
-//                      the counter-based RNG has one form, so 9 and 10 are the same)
-//   --walkmode=1       + the workgroup sampler for lists above --hub_threshold
-//   --walkmode=6       + parking: walkers waiting on the same vertex share one scan of its list (the default)
+// include/gpu_graph.cuh:46-54).  --walkmode keeps the reference's ablation levels (README.md:152-163), run by the
+// reference's own algorithms restated for 64-lane waves (FW_SAMPLER_REF_*: two-pass ZPRS / chunked DPRS, 64 task
+// slots per workgroup), and adds this engine's own levels:
+//   --walkmode=9 / 10  "FW" / "FW + RNG": the reference's DPRS samplers, static query assignment (the counter-based
+//                      RNG has one form, so 9 and 10 are the same)
+//   --walkmode=1       "FW + ZPRS": the reference's ZPRS samplers, static query assignment
+//   --walkmode=6       "FW + DS": the reference's ZPRS samplers with the global query dispenser (its default kernel)
+//   --walkmode=20      this engine's walk kernel alone, every list sampled by one wave (no workgroup sampler, no parking)
+//   --walkmode=21      + the workgroup sampler for lists above --hub_threshold
+//   --walkmode=22      + parking: walkers waiting on the same vertex share one scan of its list (the default)
 // --park_threshold passes fw_walk_params.park_threshold through (0 library rule, < 0 off, > 0 explicit degree).
 
 #include <stdint.h>
@@ -206,8 +210,10 @@ int main(int argc, char** argv) {
   Flags F;
   if (!parse_flags(argc, argv, &F)) return 2;
   if (F.umgraph) printf("umgraph: edge arrays stay in pinned host memory and are read over the bus\n");
-  if (F.walkmode >= 0 && F.walkmode != 1 && F.walkmode != 6 && F.walkmode != 9 && F.walkmode != 10) {
-    fprintf(stderr, "flowwalker: --walkmode must be 9, 10, 1 or 6 (ablation levels); %d ignored\n", F.walkmode);
+  if (F.walkmode >= 0 && F.walkmode != 1 && F.walkmode != 6 && F.walkmode != 9 && F.walkmode != 10 &&
+      (F.walkmode < 20 || F.walkmode > 22)) {
+    fprintf(stderr, "flowwalker: --walkmode must be 9, 10, 1, 6 (the reference's ablation levels) or 20, 21, 22 (this "
+                    "engine's); %d ignored\n", F.walkmode);
     F.walkmode = -1;
   }
   if (!(F.deepwalk || F.ppr || F.node2vec || F.metapath)) {  // src/walk.cu:565-568
@@ -317,12 +323,19 @@ int main(int argc, char** argv) {
   if (F.hub_threshold >= 0) P.hub_threshold = F.hub_threshold;
   if (F.wg_threads > 0) P.wg_threads = F.wg_threads;
   P.park_threshold = F.park_threshold;
-  if (F.walkmode >= 0) {  // ablation levels, lowest first
-    if (F.walkmode == 9 || F.walkmode == 10) P.hub_threshold = 0x7FFFFFFF;
-    if (F.walkmode != 6) P.park_threshold = -1;
+  if (F.walkmode >= 20) {  // this engine's levels, lowest first
+    if (F.walkmode == 20) P.hub_threshold = 0x7FFFFFFF;
+    if (F.walkmode != 22) P.park_threshold = -1;
     printf("ablation level %d: %s\n", F.walkmode,
-           F.walkmode == 6 ? "workgroup sampler and parking (the full engine)"
-                           : F.walkmode == 1 ? "workgroup sampler, no parking" : "wave sampler only, no parking");
+           F.walkmode == 22 ? "workgroup sampler and parking (the full engine)"
+                            : F.walkmode == 21 ? "workgroup sampler, no parking" : "wave sampler only, no parking");
+  } else if (F.walkmode >= 0) {  // the reference's levels (README.md:152-163), its algorithms on 64-lane waves
+    const bool dprs = F.walkmode == 9 || F.walkmode == 10;
+    const bool is_static = F.walkmode != 6;
+    P.sampler = (dprs ? FW_SAMPLER_REF_DPRS : FW_SAMPLER_REF_ZPRS) | (is_static ? FW_SAMPLER_REF_STATIC : 0);
+    if (F.hub_threshold < 0) P.hub_threshold = 1024;  // THRESHOLD, include/walker.cuh:29
+    printf("ablation level %d: the reference's %s samplers on 64-lane waves, %s\n", F.walkmode, dprs ? "DPRS" : "ZPRS",
+           is_static ? "static query assignment" : "global query dispenser");
   }
 
   // ---- walk (src/main.cu:346-357) ----

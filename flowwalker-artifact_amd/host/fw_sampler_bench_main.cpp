@@ -8,9 +8,16 @@
 // or workgroup (every list by a whole workgroup of --wg_threads).  The engine's kernels are measured as they
 // are, through the C ABI; nothing is re-implemented here.
 //
+// --type picks the algorithm, as TestSampler's --type does (src/sampler_test.cu:789-895): `native` = this engine's
+// one-pass group reservoir; `zprs` / `dprs` = the reference's own samplers restated for 64-lane waves
+// (include/sampler.cuh:46-127 and :129-200, FW_SAMPLER_REF_ZPRS / _DPRS: TestSampler types 1 / 2 and 3 / 4), run
+// on the same lists so that the columns can be compared.
+//
 //   fw_sampler_bench [--elements 268435456] [--gran 16,64,256,1024,4096,16384,65536] [--samples 4194304]
-//                    [--granularity wave|workgroup|both] [--wg_threads 512] [--reps 3] [--seed 1]
-// Output: one line per (gran, granularity): samples/s and GB/s of weights read (4 bytes per element).
+//                    [--granularity wave|workgroup|both] [--type native,zprs,dprs] [--wg_threads 512] [--reps 3]
+//                    [--seed 1]
+// Output: one line per (gran, type, granularity): samples/s and GB/s of weights (4 bytes per element and sample;
+// the two-pass ZPRS reads them twice, which is not counted).
 
 #include <stdint.h>
 #include <stdio.h>
@@ -32,7 +39,7 @@ static int fail(const char* what) {
 int main(int argc, char** argv) {
   unsigned long long elements = 1ull << 28, seed = 1;
   long long samples = 1ll << 22;
-  std::string grans = "16,64,256,1024,4096,16384,65536", granularity = "both";
+  std::string grans = "16,64,256,1024,4096,16384,65536", granularity = "both", types = "native,zprs,dprs";
   int wg_threads = 512, reps = 3;
   for (int i = 1; i < argc; ++i) {
     const std::string k = argv[i];
@@ -44,6 +51,7 @@ int main(int argc, char** argv) {
     else if (k == "--gran") grans = val();
     else if (k == "--samples") samples = atoll(val());
     else if (k == "--granularity") granularity = val();
+    else if (k == "--type") types = val();
     else if (k == "--wg_threads") wg_threads = atoi(val());
     else if (k == "--reps") reps = atoi(val());
     else if (k == "--seed") seed = strtoull(val(), nullptr, 10);
@@ -69,7 +77,19 @@ int main(int argc, char** argv) {
     adj[i] = 0;
   }
 
-  printf("%-10s %-10s %12s %14s %12s %10s\n", "gran", "sampler", "samples", "samples/s", "GB/s", "ms");
+  struct Type { const char* name; int sampler; };
+  std::vector<Type> run_types;
+  for (size_t tp = 0; tp < types.size();) {
+    size_t c = types.find(',', tp);
+    if (c == std::string::npos) c = types.size();
+    const std::string t = types.substr(tp, c - tp);
+    tp = c + 1;
+    if (t == "native") run_types.push_back({"native", FW_SAMPLER_ZPRS});
+    else if (t == "zprs") run_types.push_back({"zprs", FW_SAMPLER_REF_ZPRS});
+    else if (t == "dprs") run_types.push_back({"dprs", FW_SAMPLER_REF_DPRS});
+    else { fprintf(stderr, "fw_sampler_bench: --type takes native, zprs, dprs (got %s)\n", t.c_str()); return 2; }
+  }
+  printf("%-10s %-8s %-10s %12s %14s %12s %10s\n", "gran", "type", "sampler", "samples", "samples/s", "GB/s", "ms");
   size_t pos = 0;
   while (pos < grans.size()) {
     size_t comma = grans.find(',', pos);
@@ -94,27 +114,30 @@ int main(int argc, char** argv) {
       return fail("allocating");
     if (fw_dev_upload(d_starts, starts.data(), (size_t)samples * 4) != FW_OK) return fail("uploading queries");
 
-    for (int mode = 0; mode < 2; ++mode) {
-      const char* name = mode == 0 ? "wave" : "workgroup";
-      if (granularity != "both" && granularity != name) continue;
-      fw_walk_params p;
-      fw_walk_params_default(&p);
-      p.app = FW_APP_DEEPWALK;
-      p.max_depth = 2;                 // the start vertex and one sampled neighbour
-      p.wg_threads = wg_threads;
-      p.hub_threshold = mode == 0 ? 0x7FFFFFFF : 0;  // every list by one wave / by the workgroup
-      p.park_threshold = -1;           // the plain sampler, no sharing of scans between walkers
-      p.seed = seed;
-      double best = 0.0;
-      fw_walk_stats st;
-      for (int r = 0; r <= reps; ++r) {  // first run warms up
-        if (fw_walk_device(g, &p, (const int32_t*)d_starts, (int32_t)samples, (int32_t*)d_paths, nullptr, &st) != FW_OK)
-          return fail("sampling");
-        if (r > 0 && (best == 0.0 || st.kernel_ms < best)) best = st.kernel_ms;
+    for (const Type& type : run_types) {
+      for (int mode = 0; mode < 2; ++mode) {
+        const char* name = mode == 0 ? "wave" : "workgroup";
+        if (granularity != "both" && granularity != name) continue;
+        fw_walk_params p;
+        fw_walk_params_default(&p);
+        p.app = FW_APP_DEEPWALK;
+        p.sampler = type.sampler;
+        p.max_depth = 2;                 // the start vertex and one sampled neighbour
+        p.wg_threads = wg_threads;
+        p.hub_threshold = mode == 0 ? 0x7FFFFFFF : 0;  // every list by one wave / by the workgroup
+        p.park_threshold = -1;           // the plain sampler, no sharing of scans between walkers
+        p.seed = seed;
+        double best = 0.0;
+        fw_walk_stats st;
+        for (int r = 0; r <= reps; ++r) {  // first run warms up
+          if (fw_walk_device(g, &p, (const int32_t*)d_starts, (int32_t)samples, (int32_t*)d_paths, nullptr, &st) != FW_OK)
+            return fail("sampling");
+          if (r > 0 && (best == 0.0 || st.kernel_ms < best)) best = st.kernel_ms;
+        }
+        printf("%-10lld %-8s %-10s %12llu %14.4g %12.1f %10.3f\n", gran, type.name, name, (unsigned long long)st.steps,
+               (double)st.steps / (best * 1e-3), 4.0 * (double)st.sampled_edges / (best * 1e-3) / 1e9, best);
+        fflush(stdout);
       }
-      printf("%-10lld %-10s %12llu %14.4g %12.1f %10.3f\n", gran, name, (unsigned long long)st.steps,
-             (double)st.steps / (best * 1e-3), 4.0 * (double)st.sampled_edges / (best * 1e-3) / 1e9, best);
-      fflush(stdout);
     }
     fw_dev_free(d_starts);
     fw_dev_free(d_paths);

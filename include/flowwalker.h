@@ -38,8 +38,24 @@ typedef enum {
  * functors of include/app.cuh:58-152. */
 typedef enum { FW_APP_DEEPWALK = 0, FW_APP_PPR = 1, FW_APP_NODE2VEC = 2, FW_APP_METAPATH = 3 } fw_app;
 
-/* Sampler selector: ZPRS kernel (include/walker.cuh:1307) or DPRS kernel (:1444, --dprs). */
-typedef enum { FW_SAMPLER_ZPRS = 0, FW_SAMPLER_DPRS = 1 } fw_sampler;
+/*
+ * Sampler selector: ZPRS kernel (include/walker.cuh:1307) or DPRS kernel (:1444, --dprs).  Both name this
+ * library's one-pass sampler (it evaluates every bias once, which is what the reference's DPRS kernel exists for).
+ * FW_SAMPLER_REF_ZPRS / FW_SAMPLER_REF_DPRS run the reference's own algorithms instead, restated for 64-lane waves:
+ * sampler_warp / sampler_block (include/sampler.cuh:46-127: two passes, one uniform per neighbour, key max-reduce)
+ * and sampler_warp_oneloop / sampler_block_oneloop (:129-200: chunked scan with carry) inside the reference's round
+ * structure (64 task slots per workgroup, include/walker.cuh:1357-1438).  They are the ablation baselines of
+ * README.md:152-163 and the columns of the sampler micro-benchmark; same sampling law, their own random streams, no
+ * parking.  OR FW_SAMPLER_REF_STATIC into either for the reference's static query assignment (src/walk.cu:46-61)
+ * instead of the global dispenser.
+ */
+typedef enum {
+  FW_SAMPLER_ZPRS = 0,
+  FW_SAMPLER_DPRS = 1,
+  FW_SAMPLER_REF_ZPRS = 2,
+  FW_SAMPLER_REF_DPRS = 3,
+  FW_SAMPLER_REF_STATIC = 0x100
+} fw_sampler;
 
 /*
  * Walk parameters.  Replaces the gflags globals read by src/walk.cu:36-44 (FLAGS_tp, FLAGS_p,

@@ -62,7 +62,12 @@
 #define FW_MAX_GROUP 1024
 
 enum { FW_APP_DEEPWALK = 0, FW_APP_PPR = 1, FW_APP_NODE2VEC = 2, FW_APP_METAPATH = 3 };
-enum { FW_SAMPLER_ZPRS = 0, FW_SAMPLER_DPRS = 1 };
+enum { FW_SAMPLER_ZPRS = 0, FW_SAMPLER_DPRS = 1, FW_SAMPLER_REF_ZPRS = 2, FW_SAMPLER_REF_DPRS = 3 };
+
+/* fw_ref_samplers.c */
+int32_t fw_ref64_zprs(const float* w, int32_t n, int32_t W, const float* u);
+int32_t fw_ref64_dprs(const float* w, int32_t n, int32_t W, const float* u);
+float fw_ref64_uniform(uint64_t seed, uint32_t walker, uint32_t step, uint32_t i, uint32_t W);
 
 #define FW_STREAM_WAVE 0x40000000u /* workgroup-level combine draw */
 #define FW_STREAM_STOP 0x80000000u /* PPR stop draw */
@@ -332,6 +337,22 @@ int32_t fw_oracle_sample(const fw_oracle_graph* g, const fw_oracle_params* p, in
   uint32_t off = g->xadj[cur];
   int32_t deg = (int32_t)(g->xadj[cur + 1] - off);
   const int nw = (deg > p->hub_threshold) ? p->wg_threads / FW_WAVE : 1;
+  const int kind = p->sampler & 0xFF;
+  if (kind == FW_SAMPLER_REF_ZPRS || kind == FW_SAMPLER_REF_DPRS) {
+    /* the reference's own samplers on 64-lane waves (fw_ref_samplers.c), fed with this build's biases and uniforms */
+    if (deg <= 0) return -1;
+    const int32_t W = nw * FW_WAVE;
+    float* w = (float*)malloc(sizeof(float) * (size_t)deg);
+    float* u = (float*)malloc(sizeof(float) * (size_t)deg);
+    for (int32_t i = 0; i < deg; ++i) {
+      w[i] = bias_at(&c, (uint64_t)off + (uint32_t)i);
+      u[i] = fw_ref64_uniform(p->seed, walker, step, (uint32_t)i, (uint32_t)W);
+    }
+    const int32_t sel = kind == FW_SAMPLER_REF_ZPRS ? fw_ref64_zprs(w, deg, W, u) : fw_ref64_dprs(w, deg, W, u);
+    free(w);
+    free(u);
+    return sel;
+  }
   return group_sample(&c, off, deg, nw, walker, step);
 }
 

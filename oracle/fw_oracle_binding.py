@@ -162,7 +162,7 @@ def sequential_reservoir(w, u):
     return int(lib().fw_oracle_sequential_reservoir(w.ctypes.data_as(C.c_void_p), u.ctypes.data_as(C.c_void_p), len(w)))
 
 
-REF_THREAD, REF_ZPRS, REF_DPRS = 0, 1, 2
+REF_THREAD, REF_ZPRS, REF_DPRS, REF64_ZPRS, REF64_DPRS = 0, 1, 2, 3, 4
 
 
 def ref_sample_many(kind, w, u, width=32):

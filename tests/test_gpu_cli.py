@@ -84,15 +84,17 @@ def test_metapath_and_ppr(gpu, graph_files, tmp_path):
 
 
 def test_sampler_micro_benchmark_and_converter(gpu, tmp_path):
-    """fw_sampler_bench (one sampling step at fixed list lengths, both granularities) runs and reports every sample;
+    """fw_sampler_bench (one sampling step at fixed list lengths, three algorithms, both granularities) runs and reports every sample;
     a graph written by fw_convert loads and walks."""
     tool = os.path.join(ROOT, "flowwalker-artifact_amd", "bin", "fw_sampler_bench")
     r = subprocess.run([tool, "--elements", "1048576", "--samples", "20000", "--gran", "16,1024", "--reps", "1"],
                        stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
     assert r.returncode == 0, r.stderr
     rows = [ln.split() for ln in r.stdout.splitlines()[1:]]
-    assert [(row[0], row[1]) for row in rows] == [("16", "wave"), ("16", "workgroup"), ("1024", "wave"), ("1024", "workgroup")]
-    assert all(int(row[2]) == 20000 and float(row[3]) > 0 for row in rows)
+    # per list length: this engine's sampler, then the reference's ZPRS and DPRS on 64-lane waves, each at both granularities
+    want = [(g, t, s) for g in ("16", "1024") for t in ("native", "zprs", "dprs") for s in ("wave", "workgroup")]
+    assert [(row[0], row[1], row[2]) for row in rows] == want
+    assert all(int(row[3]) == 20000 and float(row[4]) > 0 for row in rows)
 
     conv = os.path.join(ROOT, "flowwalker-artifact_amd", "bin", "fw_convert")
     rng = np.random.RandomState(11)
@@ -139,17 +141,24 @@ def test_save_degree_and_lognorm(gpu, graph_files, tmp_path):
 
 
 def test_ablation_levels_and_park_threshold(gpu, graph_files, tmp_path):
-    """--walkmode selects this engine's ablation levels (README.md:152-163 of the reference names its own): 9 / 10
-    the wave sampler alone, 1 adds the workgroup sampler, 6 adds parking.  Parking never changes a path, the
-    sampler's granularity is part of the sampling definition; every level equals the oracle run with its settings."""
+    """--walkmode 9 / 10 / 1 / 6 are the reference's ablation levels (README.md:152-163: DPRS static, ZPRS static, ZPRS
+    with the dispenser), run by its own samplers restated for 64-lane waves; 20 / 21 / 22 are this engine's levels
+    (wave sampler alone, + workgroup sampler, + parking).  Parking and the way queries are assigned never change a
+    path; the sampler and its granularity are part of the sampling definition: every level equals the oracle run
+    with its settings."""
     prefix, csr = graph_files
     V = len(csr[0]) - 1
     starts = np.arange(V, dtype=np.int32)
     og = orc.Graph(*csr)
     ref_wg, _, _ = orc.walk(og, orc.make_params(max_depth=11, seed=3, hub_threshold=1000), starts)
     ref_wave, _, _ = orc.walk(og, orc.make_params(max_depth=11, seed=3, hub_threshold=0x7FFFFFFF), starts)
-    for mode, ref, note in ((9, ref_wave, "wave sampler only"), (10, ref_wave, "wave sampler only"),
-                            (1, ref_wg, "no parking"), (6, ref_wg, "full engine")):
+    ref_zprs, _, _ = orc.walk(og, orc.make_params(sampler=2, max_depth=11, seed=3, hub_threshold=1000), starts)
+    ref_dprs, _, _ = orc.walk(og, orc.make_params(sampler=3, max_depth=11, seed=3, hub_threshold=1000), starts)
+    assert (ref_zprs != ref_wg).any() and (ref_dprs != ref_zprs).any()  # three samplers, three sets of walks
+    for mode, ref, note in ((9, ref_dprs, "DPRS samplers on 64-lane waves, static"), (10, ref_dprs, "DPRS"),
+                            (1, ref_zprs, "ZPRS samplers on 64-lane waves, static"),
+                            (6, ref_zprs, "ZPRS samplers on 64-lane waves, global query dispenser"),
+                            (20, ref_wave, "wave sampler only"), (21, ref_wg, "no parking"), (22, ref_wg, "full engine")):
         out = str(tmp_path / ("m%d.bin" % mode))
         text = _run("--input", prefix, "--deepwalk", "--all", "--d=10", "--seed=3", "--hub_threshold=1000",
                     "--walkmode=%d" % mode, "--savepaths", out)

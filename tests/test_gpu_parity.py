@@ -333,6 +333,27 @@ def test_randomized_configurations(gpu):
             g.destroy()
 
 
+@pytest.mark.parametrize("static", [0, 1])
+@pytest.mark.parametrize("sampler", ["ref_zprs", "ref_dprs"])
+def test_reference_engine_on_wave64(gpu, hub, sampler, static):
+    """FW_SAMPLER_REF_ZPRS / _DPRS: the reference's own samplers and round structure restated for 64-lane waves
+    (include/sampler.cuh:46-200, include/walker.cuh:1357-1438), with the global dispenser or static assignment.  The
+    oracle runs the CPU restatement of the same definition: bit-exact paths and counters, all four applications, wave
+    and workgroup granularity."""
+    sid = (gpu.SAMPLER_REF_ZPRS if sampler == "ref_zprs" else gpu.SAMPLER_REF_DPRS) | (gpu.SAMPLER_REF_STATIC if static else 0)
+    starts = np.random.RandomState(8).randint(0, 12000, size=1500).astype(np.int32)
+    starts[:40] = 0
+    starts[40:60] = 1
+    for kw in (dict(app=gpu.APP_DEEPWALK, max_depth=21, hub_threshold=1024, wg_threads=512),
+               dict(app=gpu.APP_DEEPWALK, max_depth=11, hub_threshold=1 << 30, wg_threads=256),
+               dict(app=gpu.APP_DEEPWALK, max_depth=11, hub_threshold=100, wg_threads=1024),
+               dict(app=gpu.APP_PPR, max_depth=41, tp=0.15, hub_threshold=1024),
+               dict(app=gpu.APP_NODE2VEC, max_depth=9, p=2.0, q=0.5, hub_threshold=2000, wg_threads=256),
+               dict(app=gpu.APP_METAPATH, max_depth=7, schema=[1, 3, 0], hub_threshold=1024)):
+        paths, st = _check(gpu, hub, starts, sampler=sid, seed=55, **kw)
+        assert st.launches == 1 and st.hub_steps == 0  # the reference's engine never parks
+
+
 def test_one_walk_call_at_a_time_per_graph(gpu):
     """The parking index, the parking lists and the launch record are cached in the fw_graph, so a second call on
     the same graph while one is running is refused with a status code (it used to race); afterwards the graph works

@@ -101,3 +101,47 @@ def test_all_samplers_follow_the_same_law():
         cnt = np.bincount(paths[:, 1], minlength=V)[:n].astype(np.float64)
         assert cnt.sum() == m and cnt[~pos].sum() == 0
         assert chisquare(cnt[pos], expect).pvalue > 0.01, thr
+
+
+@pytest.mark.parametrize("width", [64, 256, 512])
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 200, 511, 512, 513, 3000])
+def test_wave64_restatements_are_the_same_sequential_reservoirs(n, width):
+    """The two samplers for groups of 64-lane waves (what FW_SAMPLER_REF_ZPRS / _DPRS run on the GPU): ZPRS is the
+    sequential reservoir over the lane-major order, DPRS the one in list order, exactly, for integer-valued biases
+    (their sums are exact in any association, so the scan tree cannot matter)."""
+    rng = np.random.RandomState(31 * width + n)
+    for zero_fraction in (0.0, 0.3, 1.0):
+        w = _int_biases(rng, n, zero_fraction)
+        u = _uniforms(rng, (150, n))
+        order = np.concatenate([np.arange(l, n, width) for l in range(min(width, n))])
+        got = orc.ref_sample_many(orc.REF64_ZPRS, w, u, width)
+        seq = orc.ref_sample_many(orc.REF_THREAD, w[order], u[:, order], width)
+        assert (got == np.where(seq < 0, -1, order[np.maximum(seq, 0)])).all()
+        got = orc.ref_sample_many(orc.REF64_DPRS, w, u, width)
+        assert (got == orc.ref_sample_many(orc.REF_THREAD, w, u, width)).all()
+        # and they agree with the reference's own 32- / 512-lane forms wherever both are defined on the same width
+        if width == 512:
+            assert (orc.ref_sample_many(orc.REF64_ZPRS, w, u, 512) == orc.ref_sample_many(orc.REF_ZPRS, w, u, 512)).all()
+            assert (orc.ref_sample_many(orc.REF64_DPRS, w, u, 512) == orc.ref_sample_many(orc.REF_DPRS, w, u, 512)).all()
+
+
+def test_wave64_restatements_follow_the_law_in_whole_walks():
+    """First steps of the oracle's walks with sampler = reference ZPRS / DPRS on 64-lane waves (keyed Philox uniforms in
+    (0, 1]) from one vertex: chi-square against w / sum w at wave and at workgroup granularity."""
+    rng = np.random.RandomState(98)
+    n, m = 1500, 120000
+    w = (1.0 + 99.0 * rng.random_sample(n)).astype(np.float32)
+    w[rng.random_sample(n) < 0.1] = 0.0
+    pos = w > 0
+    expect = w[pos].astype(np.float64) / w.astype(np.float64).sum() * m
+    V = n + 2
+    xadj = np.zeros(V + 1, dtype=np.uint32)
+    xadj[2:] = n
+    g = orc.Graph(xadj, (np.arange(n) % V).astype(np.int32), w)
+    for sampler in (2, 3):
+        for thr in (1 << 30, 1000):
+            p = orc.make_params(sampler=sampler, max_depth=2, hub_threshold=thr, wg_threads=256, seed=78)
+            paths, _, _ = orc.walk(g, p, np.full(m, 1, dtype=np.int32))
+            cnt = np.bincount(paths[:, 1], minlength=V)[:n].astype(np.float64)
+            assert cnt.sum() == m and cnt[~pos].sum() == 0
+            assert chisquare(cnt[pos], expect).pvalue > 0.01, (sampler, thr)
