@@ -48,7 +48,6 @@ CONFIG_OF = {"deepwalk_rmat22": "C2", "ppr_rmat22": "C3", "node2vec_rmat24_sym":
 # bytes this run counts itself (roofline.requested_bytes), never instead of them.
 PROFILED_TRAFFIC = {
     "deepwalk_rmat24_sym": (5.73e11, "profiles/walk_pipeline_deepwalk_rmat24sym_pmc.txt"),
-    "node2vec_rmat24_sym": (5.24e13, "profiles/fw_walk_zprs_node2vec_rmat24sym_pmc.txt"),
 }
 
 
@@ -67,11 +66,12 @@ def roofline_of(app, st, n, kernel_ms):
     counted by the library: fw_walk_stats.requested_bytes) over the device time of the pass, so `frac` is a fraction
     of what the memory can deliver.  `algorithmic_rate` divides the bytes every walker would read alone
     (4*D + 16*S + 16*Q) by the same time: with hub parking a list is read once per batch of walkers, so this figure
-    exceeds the peak and `reuse_factor` = algorithmic / requested says by how much lists were shared.  node2vec never
-    parks and its requested bytes leave out the probes of the adjacency test, so its algorithmic bytes are used."""
+    exceeds the peak and `reuse_factor` = algorithmic / requested says by how much lists were shared.  node2vec's
+    algorithmic bytes are those of evaluating every neighbour's bias (8*D + 24*S + 16*Q); its two-stage step reads the
+    weights only, shares the passes, and makes one binary search per trial (counted as 16 lines per step)."""
     alg = algorithmic_bytes(app, st.steps, st.sampled_edges, n)
     req = int(st.requested_bytes)
-    hbm = alg if app == "node2vec" or req == 0 else req
+    hbm = alg if req == 0 else req
     sec = kernel_ms * 1e-3
     return {
         "bound": "hbm", "achieved": hbm / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -247,7 +247,7 @@ def main():
     roofline["kernel"] = ("fw_walk_ref" if args.sampler != "native" else
                           "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_scan + fw_hub_batch pipeline")
     # the profiler's view of the same workload (library defaults only: any override makes it another run)
-    prof = PROFILED_TRAFFIC.get(args.workload) if defaults and (last.launches > 1 or wl["app"] == "node2vec") else None
+    prof = PROFILED_TRAFFIC.get(args.workload) if defaults and last.launches > 1 else None
     roofline["traffic"] = prof[0] if prof else None
     if prof:
         roofline["traffic_source"] = prof[1]
@@ -290,7 +290,7 @@ def main():
         # the walk kernel against the roofline on the bytes it touches) and one line per benchmark configuration
         out["roofline"]["no_parking"] = one_config(fw, g, HEADLINE, wl, passes=1, warmup=0, park_threshold=-1)
         configs = [config1(fw)]
-        configs.append(one_config(fw, g, "node2vec_rmat24_sym", WORKLOADS["node2vec_rmat24_sym"], passes=1, warmup=0))
+        configs.append(one_config(fw, g, "node2vec_rmat24_sym", WORKLOADS["node2vec_rmat24_sym"], passes=3, warmup=1))
         cpu = None if args.no_cpu else cpu_baseline(fw, g, params, starts, args.cpu_seconds)
         g.destroy()
         g22 = make_graph(fw, WORKLOADS["deepwalk_rmat22"])

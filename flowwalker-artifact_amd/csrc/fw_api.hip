@@ -89,7 +89,6 @@ extern "C" void fw_walk_params_default_for(fw_walk_params* p, int app) {
   if (!p) return;
   fw_walk_params_default(p);
   p->app = app;
-  if (app == FW_APP_NODE2VEC) p->hub_threshold = INT_MAX;
 }
 
 extern "C" uint32_t fw_autobatch_size(size_t free_bytes, int32_t headroom_mb, int32_t max_depth, int sync,
@@ -462,6 +461,9 @@ static void fill_kargs(fw_kargs* a, const fw_graph* g, const fw_walk_params* p) 
   a->tp = p->tp;
   a->inv_p = 1.0f / p->p;
   a->inv_q = 1.0f / p->q;
+  a->n2v_fmax = 1.0f;
+  if (a->inv_p > a->n2v_fmax) a->n2v_fmax = a->inv_p;
+  if (a->inv_q > a->n2v_fmax) a->n2v_fmax = a->inv_q;
   a->schema_len = p->schema_len;
   for (int i = 0; i < FW_MAX_SCHEMA; ++i) a->schema[i] = (i < p->schema_len) ? p->schema[i] : 0;
   a->park_threshold = INT_MAX;
@@ -745,17 +747,23 @@ __global__ void fw_scatter_tagged_kernel(const fw_walker_rec* __restrict__ src, 
   }
 }
 
+// tagged_only (node2vec, whose records carry the previous vertex instead of a position): src is a batch launch's
+// output list, of which only the records tagged FW_REC_PARK take part.
 __global__ void fw_scatter_counted_kernel(const fw_walker_rec* __restrict__ src, uint32_t m,
                                           const uint32_t* __restrict__ bucket_count,
                                           const uint32_t* __restrict__ bucket_offset, uint32_t* bucket_fill,
-                                          fw_walker_rec* __restrict__ sorted) {
+                                          fw_walker_rec* __restrict__ sorted, int tagged_only) {
   const uint32_t stride = gridDim.x * blockDim.x;
   for (uint32_t i0 = blockIdx.x * blockDim.x; i0 < m; i0 += stride) {  // uniform in the wave: the ranks are taken together
     const uint32_t i = i0 + threadIdx.x;
-    const bool have = i < m;
+    bool have = i < m;
     fw_walker_rec r;
     r.q = 0; r.cur = 0; r.prev = 0; r.len = 0;
     if (have) r = src[i];
+    if (tagged_only) {
+      have = have && r.q >= 0 && (r.len & FW_REC_PARK) != 0;
+      r.len &= ~FW_REC_PARK;
+    }
     const uint32_t b = (uint32_t)r.cur;
     const uint32_t rank = fw_wave_count_keys<true>(bucket_fill, b, have);
     if (have) sorted[bucket_offset[b] + bucket_count[b] - 1u - rank] = r;
@@ -944,7 +952,9 @@ static uint64_t two_pass_rows(const fw_graph* g, int labels) {
 
 // Decides whether a call parks walkers, and at which degree.  Returns INT_MAX for "no".
 static int32_t resolve_park_threshold(const fw_graph* g, const fw_walk_params* p, int32_t n) {
-  if (p->app == FW_APP_NODE2VEC) return INT_MAX;  // its biases depend on the walker: nothing to share
+  // node2vec's proposals do not depend on the walker, so its walkers share scans like the others; their records keep
+  // the path length in 16 bits
+  if (p->app == FW_APP_NODE2VEC && p->max_depth > FW_REC_LEN_MASK) return INT_MAX;
   if (p->sampler != FW_SAMPLER_ZPRS && p->sampler != FW_SAMPLER_DPRS) return INT_MAX;  // the reference's engine: one launch
   if (p->park_threshold < 0) return INT_MAX;
   if (p->park_threshold == 0) {
@@ -1094,12 +1104,17 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
       unsigned blocks = (cnt + 255u) / 256u;
       return blocks > 8192u ? 8192u : blocks;
     };
-    if (n_out != 0u)
-      hipLaunchKernelGGL(fw_scatter_tagged_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
-                         pb->offset(), pb->sorted);
+    if (n_out != 0u) {
+      if (p->app == FW_APP_NODE2VEC)
+        hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
+                           pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 1);
+      else
+        hipLaunchKernelGGL(fw_scatter_tagged_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
+                           pb->offset(), pb->sorted);
+    }
     if (n_walked != 0u)
       hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_walked)), dim3(256), 0, stream, pb->walked,
-                         n_walked, pb->count(cur), pb->offset(), pb->fill(), pb->sorted);
+                         n_walked, pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 0);
     FW_HIP(hipGetLastError());
     hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs, pb->count(nxt),
                        pb->fill(), pb->n_buckets, a.dispenser);
@@ -1196,10 +1211,11 @@ static uint64_t requested_bytes_model(const fw_walk_params* p, int32_t n, bool p
   // walk launches.  A list is read from its first aligned quartet on (about 12 bytes of padding per step); lists of
   // up to 64 quartets bring their neighbours along with the biases, longer ones fetch the selected neighbour alone.
   const bool short_lists = parked && park_threshold <= 252;
-  const uint64_t per_entry_array = (n2v || short_lists) ? 2 : 1;
+  const uint64_t per_entry_array = short_lists ? 2 : 1;
   b += per_entry_array * (4 * walk_edges + 12 * walk_steps);
   if (!short_lists) b += kLine * walk_steps;                      // adjncy[off + sel]
   b += (kLine + kLine + (parked ? kLine : 0)) * walk_steps;       // path entry, xadj pair, parking index
+  if (n2v) b += 16 * kLine * (walk_steps + hub_steps);            // about one binary search in N(prev) per step
   b += (4 + kLine + kLine + (parked ? kLine : 0)) * (uint64_t)n;  // start vertex, path[0], xadj pair, parking index
   if (parked) {
     b += (kRec + kLine) * t.parked_records;                       // record out, bucket counter

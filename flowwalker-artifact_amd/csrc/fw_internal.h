@@ -72,6 +72,7 @@ struct fw_kargs {
   uint32_t seed_lo, seed_hi;
   uint32_t walker_base;
   float tp, inv_p, inv_q;
+  float n2v_fmax;                    // max(1, 1/p, 1/q): the envelope of node2vec's acceptance test
   int32_t schema_len;
   int32_t schema[FW_MAX_SCHEMA];
   // hub parking (park_threshold = INT32_MAX switches it off)
@@ -88,6 +89,13 @@ struct fw_kargs {
 
 // Tag in fw_walker_rec::len of a batch-kernel output record whose vertex is parked on again (stripped by readers).
 constexpr int32_t FW_REC_PARK = 0x40000000;
+// node2vec records: bits 0..15 of len hold the path length, bits 16..29 the rejected trials of the walker's current
+// step (a parked walker whose proposal is rejected waits on the same vertex for another round); prev is the previous
+// vertex in every record (its acceptance test searches N(prev)), so positions inside a bucket are handed out by the
+// scatter kernel, never carried in the record.
+constexpr int FW_REC_TRIAL_SHIFT = 16;
+constexpr int32_t FW_REC_TRIAL_MASK = 0x3FFF;
+constexpr int32_t FW_REC_LEN_MASK = 0xFFFF;
 
 // One batch: up to 64 walkers parked on vertex v, records sorted[rec_base .. rec_base + count).  32 bytes.
 struct fw_batch_task {

@@ -36,10 +36,13 @@ namespace {
 constexpr int kPipelineInFlight = 4;            // bundles of short lists a wave loads per turn in launches of the parking pipeline
 constexpr uint32_t kStreamWave = 0x40000000u;  // workgroup-level combine draw
 constexpr uint32_t kStreamStop = 0x80000000u;  // PPR stop draw
+constexpr uint32_t kStreamAccept = 0x10000000u;  // node2vec acceptance draw of a trial
+constexpr uint32_t kMaxTrials = 16384u;          // node2vec: trials per step (the trial index travels in 14 bits)
 constexpr int kHubChunk = 32;                  // hub tasks whose wave partials are parked in LDS at once
 constexpr int kGroupQuartets = 4;              // quartets per lane per group (part of the sampler's definition)
 constexpr int kFlagMoved = 1;
 constexpr int kFlagDead = 2;
+constexpr int kFlagRetry = 4;                  // node2vec: the proposal was rejected, the slot samples again
 
 // ---- per-step context (wave-uniform) -----------------------------------------------------------
 
@@ -52,163 +55,42 @@ struct StepCtx {
   int32_t want;  // metapath label of this step
   uint32_t walker;
   uint32_t step;
+  uint32_t sbase;  // added to every stream of the step's sampler draws: node2vec's trial << 8, else 0
 };
 
-// ---- node2vec adjacency test (include/gpu_graph.cuh:97-118) -----------------------------------------
-// The reference binary-searches the whole list of prev for every neighbour of cur.  Both lists are
-// ascending, so here (1) one wave-cooperative 64-ary search per group bounds the part of N(prev) that can
-// hold the group's vertices, and (2) every lane gallops forward from the position of its previous
-// neighbour.  The answers (is post in N(prev)?) are the same.
+// ---- node2vec: two-stage step -----------------------------------------------------------------------
+// The reference evaluates the bias w * f of every neighbour (f = 1/p for the return edge, 1 for a common neighbour
+// of prev and cur, 1/q otherwise: include/app.cuh:108-123), one binary search each.  Here a trial proposes a
+// neighbour with probability w_i / sum w through the sampler every application shares -- no adjacency test, and
+// walkers that stand on the same vertex can share the pass over its list -- and accepts it with probability
+// f_i / F, F = max(1, 1/p, 1/q): ONE search in N(prev) (include/gpu_graph.cuh:97-112).  A rejected trial is
+// followed by another with draws of its own (streams offset by trial << 8).  The accepted neighbour has the
+// reference's law, w_i f_i / sum_j w_j f_j.
 
-// number of entries of arr[lo, hi) that are <= x, plus lo; all 64 lanes probe one split point per round
-__device__ __forceinline__ uint32_t coop_upper_bound(const int32_t* __restrict__ arr, uint32_t lo, uint32_t hi,
-                                                     int32_t x, int lane) {
-  while (hi - lo > 64u) {
-    const uint32_t chunk = (hi - lo + 63u) >> 6;
-    uint32_t idx = lo + ((uint32_t)lane + 1u) * chunk - 1u;  // last entry of this lane's chunk
-    idx = idx < hi ? idx : hi - 1u;
-    const uint32_t cnt = (uint32_t)__builtin_popcountll(__ballot(arr[idx] <= x));
-    if (cnt == 64u) return hi;
-    const uint32_t nlo = lo + cnt * chunk;           // chunks before `cnt` are all <= x
-    const uint32_t nhi = lo + (cnt + 1u) * chunk - 1u;  // the last entry of chunk `cnt` is > x
-    lo = nlo;
-    hi = nhi < hi ? nhi : hi - 1u;
+// is `target` in the ascending arr[0, size)?  *probes += loads made
+__device__ __forceinline__ bool sorted_contains(const int32_t* __restrict__ arr, int32_t size, int32_t target,
+                                                uint32_t& probes) {
+  int32_t l = 0, r = size - 1;
+  while (l <= r) {
+    const int32_t m = l + ((r - l) >> 1);
+    const int32_t x = arr[m];
+    ++probes;
+    if (x == target) return true;
+    if (x < target) l = m + 1; else r = m - 1;
   }
-  const uint32_t i = lo + (uint32_t)lane;
-  const bool le = i < hi && arr[i] <= x;
-  return lo + (uint32_t)__builtin_popcountll(__ballot(le));
+  return false;
 }
 
-// first index in [lo, hi) with arr[index] >= x (hi if none), galloping from lo; step0 (a power of two) is the first
-// stride: 1 when x is expected right behind lo, more when the caller knows that it has jumped ahead in its own list
-__device__ __forceinline__ uint32_t gallop_lower_bound(const int32_t* __restrict__ arr, uint32_t lo, uint32_t hi,
-                                                       int32_t x, uint32_t step0 = 1u) {
-  uint32_t a = lo, b = lo + step0 - 1u, step = step0;
-  while (b < hi && arr[b] < x) {
-    a = b + 1u;
-    b = a + step - 1u;
-    step <<= 1;
-  }
-  uint32_t r = b < hi ? b : hi;
-  while (a < r) {
-    const uint32_t mid = (a + r) >> 1;
-    if (arr[mid] < x) a = mid + 1u; else r = mid;
-  }
-  return a;
-}
-
-// first index in [lo, hi) with arr[index] >= x (hi if none); all 64 lanes probe one split point per round
-__device__ __forceinline__ uint32_t coop_lower_bound(const int32_t* __restrict__ arr, uint32_t lo, uint32_t hi,
-                                                     int32_t x, int lane) {
-  while (hi - lo > 64u) {
-    const uint32_t chunk = (hi - lo + 63u) >> 6;
-    uint32_t idx = lo + ((uint32_t)lane + 1u) * chunk - 1u;
-    idx = idx < hi ? idx : hi - 1u;
-    const uint32_t cnt = (uint32_t)__builtin_popcountll(__ballot(arr[idx] < x));
-    if (cnt == 64u) return hi;
-    const uint32_t nlo = lo + cnt * chunk;
-    const uint32_t nhi = lo + (cnt + 1u) * chunk - 1u;
-    lo = nlo;
-    hi = nhi < hi ? nhi : hi - 1u;
-  }
-  const uint32_t i = lo + (uint32_t)lane;
-  const bool lt = i < hi && arr[i] < x;
-  return lo + (uint32_t)__builtin_popcountll(__ballot(lt));
-}
-
-// Per-wave LDS scratch of the adjacency test.  Forward test (neighbours of cur looked up in N(prev)): `window`
-// holds the part of N(prev) that can contain the current group's vertices, so the per-lane searches run in LDS.
-// Reversed test (entries of N(prev) looked up in N(cur)): `match` and `mask` share the same memory.
-constexpr int kN2vPerLane = 2;    // entries of N(prev) a lane resolves per refill
-constexpr int kN2vChunk = 64 * kN2vPerLane;  // entries of N(prev) resolved per refill
-constexpr int kN2vWindow = 1024;  // entries of N(prev) staged per group
-constexpr int kN2vMaxWindows = 16;   // longer stretches of N(prev) per group are searched in place
-// First strides of the forward test's gallops (powers of two; the answers do not depend on them).  A lane's
-// neighbours ascend, so the search for one starts where the search for the one before ended, but the first
-// neighbour of a quartet lies 252 neighbours of cur behind the lane's last one, a lane's first search in a streamed
-// window can end anywhere in it, and a stretch that is streamed or searched in place holds many entries of N(prev)
-// per neighbour of the group.  Measured on symmetrised R-MAT graphs, the doubling phase of a gallop that starts
-// with stride 1 costs more than it saves in all of these places: the strides below make such a search nearly a
-// binary search over what is left, and only the neighbours inside a quartet keep stride 1 when the stretch fits
-// one window.
-constexpr uint32_t kN2vQuartetStride = 256;
-constexpr uint32_t kN2vWindowStride = 512;
-constexpr uint32_t kN2vStreamedStride = 32;
-constexpr uint32_t kN2vInPlaceQuartetStride = 8192;
-constexpr uint32_t kN2vInPlaceStride = 128;
-constexpr uint64_t kN2vReverseRatio = 8;  // reversed test when N(prev) is at least this many times shorter than N(cur)
-struct N2vScratch {
-  union {
-    int32_t window[kN2vWindow];
-    struct {
-      int32_t match[kN2vChunk];  // local indices in N(cur) of common neighbours, ascending
-      uint32_t mask[64];         // per lane: bit i set = the lane's i-th bias of the current group is a common neighbour
-    };
-  };
-};
-
-// Wave-uniform cursor of the reversed test.
-struct N2vCursor {
-  uint32_t pc = 0;      // entries of N(prev) before this index are resolved
-  uint32_t cov = 0;     // local indices of N(cur) below this are resolved (all their matches are recorded)
-  uint32_t mcount = 0;  // matches in the buffer
-  uint32_t mpos = 0;    // matches already applied
-};
-
-// Resolves the next kN2vChunk entries of N(prev) (fewer at the end of the list): entry i of them is looked up in
-// N(cur), over the part of it that is not resolved yet, by lane i % 64 in its chain i / 64, and the hits are written
-// to scr.match in ascending order.  The chains of a lane do not depend on each other and the entries of a short
-// N(prev) lie far apart in N(cur): plain binary searches advancing together, one memory latency per round for all
-// of them.  A chain that no lane needs (fewer than 64 * chain entries left) costs nothing.
-__device__ __forceinline__ void n2v_refill(const int32_t* __restrict__ clist, uint32_t dc,
-                                           const int32_t* __restrict__ plist, uint32_t dp, N2vScratch& scr,
-                                           N2vCursor& k, int lane) {
-  constexpr int kP = kN2vPerLane;
-  const uint32_t cnt = (dp - k.pc) < (uint32_t)kN2vChunk ? (dp - k.pc) : (uint32_t)kN2vChunk;
-  int32_t y[kP];
-  uint32_t lo[kP], hi[kP];
-#pragma unroll
-  for (int e = 0; e < kP; ++e) {
-    const uint32_t i = 64u * (uint32_t)e + (uint32_t)lane;
-    const bool valid = i < cnt;
-    y[e] = valid ? plist[k.pc + i] : 0;
-    lo[e] = k.cov;
-    hi[e] = valid ? dc : k.cov;
-  }
-  for (uint32_t span = dc - k.cov; span != 0u; span >>= 1) {  // ceil(log2(span + 1)) rounds close every search
-#pragma unroll
-    for (int e = 0; e < kP; ++e) {
-      if (64u * (uint32_t)e < cnt) {  // uniform in the wave
-        const bool open = lo[e] < hi[e];
-        const uint32_t mid = (lo[e] + hi[e]) >> 1;
-        const int32_t val = open ? clist[mid] : 0;
-        const bool less = open && val < y[e];
-        lo[e] = less ? mid + 1u : lo[e];
-        hi[e] = (open && !less) ? mid : hi[e];
-      }
-    }
-  }
-  const uint64_t below = (1ull << lane) - 1ull;
-  const uint32_t last = cnt - 1u;  // the list's entries ascend: after this one, every index below its place is resolved
-  uint32_t total = 0u, cov = k.cov;
-#pragma unroll
-  for (int e = 0; e < kP; ++e) {
-    if (64u * (uint32_t)e < cnt) {
-      const bool valid = 64u * (uint32_t)e + (uint32_t)lane < cnt;
-      const bool hit = valid && lo[e] < dc && clist[lo[e]] == y[e];
-      const uint64_t m = __ballot(hit);
-      if (hit) scr.match[total + (uint32_t)__builtin_popcountll(m & below)] = (int32_t)lo[e];
-      total += (uint32_t)__builtin_popcountll(m);
-      if ((last >> 6) == (uint32_t)e)
-        cov = (uint32_t)__builtin_amdgcn_readlane((int)(lo[e] + (hit ? 1u : 0u)), (int)(last & 63u));
-    }
-  }
-  k.mcount = total;
-  k.mpos = 0u;
-  k.pc += cnt;
-  k.cov = k.pc >= dp ? dc : cov;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
+// Acceptance of the proposal `post` of trial `trial` at (walker, step); by one lane.
+__device__ __forceinline__ bool n2v_accept(const fw_kargs& a, int32_t post, int32_t prev, uint32_t prev_off,
+                                           int32_t prev_deg, uint32_t walker, uint32_t step, uint32_t trial,
+                                           uint32_t& probes) {
+  if (prev == -1 || trial == kMaxTrials - 1u) return true;
+  float f;
+  if (post == prev) f = a.inv_p;
+  else f = sorted_contains(a.adjncy + prev_off, prev_deg, post, probes) ? 1.0f : a.inv_q;
+  const uint32_t bits = philox4x32_10(walker, step, kStreamAccept | (trial << 8), 0u, a.seed_lo, a.seed_hi).x;
+  return u24(bits) * a.n2v_fmax < f;
 }
 
 // Wave-uniform queue of Philox words: draw n of a stream is word n & 3 of block n >> 2.
@@ -220,7 +102,7 @@ struct DrawQueue {
 
 __device__ __forceinline__ float next_uniform(DrawQueue& d, const fw_kargs& a, const StepCtx& c, uint32_t stream) {
   if (d.avail == 0u) {
-    const uint4 b = philox4x32_10(c.walker, c.step, stream, d.blk, a.seed_lo, a.seed_hi);
+    const uint4 b = philox4x32_10(c.walker, c.step, stream | c.sbase, d.blk, a.seed_lo, a.seed_hi);
     d.q0 = b.x; d.q1 = b.y; d.q2 = b.z; d.q3 = b.w;
     d.avail = 4u;
     ++d.blk;
@@ -237,7 +119,7 @@ __device__ __forceinline__ float next_uniform(DrawQueue& d, const fw_kargs& a, c
 // vertex.  Outputs: running total S of the wave's groups, selected local index (or -1), its vertex.
 template <int kApp, int kJ, bool kTrackV>
 __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c, const int lane, const uint32_t w,
-                                            const uint32_t nw, N2vScratch* scr, const DrawQueue& dq0, float& S_out,
+                                            const uint32_t nw, const DrawQueue& dq0, float& S_out,
                                             int32_t& sel_out, int32_t& selv_out) {
   constexpr uint32_t kG = 64u * kGroupQuartets;  // quartets per group
   constexpr int kEl = 4 * kJ;
@@ -247,45 +129,11 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
   const uint32_t ngroups = (nq + kG - 1u) / kG;
   const uint32_t* __restrict__ bias =
       reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
-  const bool n2v = kApp == FW_APP_NODE2VEC && c.prev != -1;
-  // reversed adjacency test: look the entries of the shorter list N(prev) up in N(cur) (wave granularity only)
-  const bool reversed = n2v && nw == 1u && (uint64_t)(uint32_t)c.prev_deg * kN2vReverseRatio <= (uint64_t)(uint32_t)c.deg;
-  const bool need_adj = kTrackV || (n2v && !reversed);
-  N2vCursor cur;
-  int32_t ret_idx = -1;  // local index of prev in N(cur): the return edge (include/app.cuh:113-114)
-  if (kApp == FW_APP_NODE2VEC && reversed) {
-    const int32_t* __restrict__ clist = a.adjncy + c.off;
-    const uint32_t r = coop_lower_bound(clist, 0u, (uint32_t)c.deg, c.prev, lane);
-    if (r < (uint32_t)c.deg && clist[r] == c.prev) ret_idx = (int32_t)r;
-  }
+  constexpr bool need_adj = kTrackV;
 
   float S = 0.0f, Sj = 0.0f, u = 1.0f;
   int32_t sel = -1, selv = -1;
   DrawQueue dq = dq0;  // empty, or block 0 of this wave's stream computed ahead by the slot's own thread
-  uint32_t seg_lo = 0u;  // node2vec: entries of N(prev) below this index are smaller than anything still to come
-  // node2vec, forward test, N(prev) short enough for the window: stage all of it once per step; every lane then
-  // gallops through it in LDS from where its previous neighbour ended (a lane's neighbours ascend across groups too)
-  bool p_staged = false;
-  uint32_t st_hi = 0u, lane_pos = 0u;
-  if (kApp == FW_APP_NODE2VEC && n2v && !reversed) {
-    const uint32_t wa = c.prev_off & ~3u;
-    const uint32_t p_end = c.prev_off + (uint32_t)c.prev_deg;
-    if (p_end - wa <= (uint32_t)kN2vWindow) {
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int k = 0; k < kN2vWindow / 256; ++k) {
-        const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
-        if (wa + wi < p_end)
-          *reinterpret_cast<int4*>(&scr->window[wi]) = *reinterpret_cast<const int4*>(a.adjncy + wa + wi);
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      p_staged = true;
-      lane_pos = c.prev_off - wa;
-      st_hi = p_end - wa;
-    }
-  }
 
   for (uint32_t g = w; g < ngroups; g += nw) {
     const uint32_t kb = g * kG + (uint32_t)lane;  // this lane's quartet for j = 0
@@ -307,7 +155,7 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
         const uint32_t k = kb + 64u * (uint32_t)j;
         const uint32_t base = a0 + 4u * k;
         raw[j] = make_uint4(0, 0, 0, 0);
-        adj[j] = make_int4(c.prev, c.prev, c.prev, c.prev);
+        adj[j] = make_int4(-1, -1, -1, -1);
         if (k < nq) {
           raw[j] = *reinterpret_cast<const uint4*>(bias + base);
           if (need_adj) adj[j] = *reinterpret_cast<const int4*>(a.adjncy + base);
@@ -342,204 +190,8 @@ __device__ __forceinline__ void wave_stream(const fw_kargs& a, const StepCtx& c,
         x[4 * j + 1] = in1 ? x[4 * j + 1] : 0.0f;
         x[4 * j + 2] = in2 ? x[4 * j + 2] : 0.0f;
         x[4 * j + 3] = in3 ? x[4 * j + 3] : 0.0f;
-        if (kApp == FW_APP_NODE2VEC) {  // never search for an entry of a foreign list
-          adj[j].x = in0 ? adj[j].x : c.prev; adj[j].y = in1 ? adj[j].y : c.prev;
-          adj[j].z = in2 ? adj[j].z : c.prev; adj[j].w = in3 ? adj[j].w : c.prev;
-        }
       }
     }
-    if (kApp == FW_APP_NODE2VEC && reversed) {
-      // include/app.cuh:108-123 with the roles of the two lists swapped: every bias becomes w/q except the
-      // common neighbours recorded in scr->match (w) and the return edge (w/p)
-      const int32_t* __restrict__ clist = a.adjncy + c.off;
-      const int32_t* __restrict__ plist = a.adjncy + c.prev_off;
-      const int32_t gs = (int32_t)(a0 + 4u * g * kG - c.off);  // local index of the group's first slot
-      const int32_t ge = gs + (int32_t)(4u * kG);
-      const uint32_t need = (uint32_t)ge < (uint32_t)c.deg ? (uint32_t)ge : (uint32_t)c.deg;
-      scr->mask[lane] = 0u;
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      for (;;) {
-        while (cur.mpos < cur.mcount) {  // 64 buffered matches at a time
-          const uint32_t i = cur.mpos + (uint32_t)lane;
-          const int32_t p = i < cur.mcount ? scr->match[i] : 0x7FFFFFFF;
-          const bool in = p < ge;
-          if (in) {
-            const uint32_t rel = (uint32_t)(p - gs);
-            const uint32_t qd = rel >> 2;
-            atomicOr(&scr->mask[qd & 63u], 1u << (((qd >> 6) << 2) | (rel & 3u)));
-          }
-          const uint32_t nin = (uint32_t)__builtin_popcountll(__ballot(in));
-          cur.mpos += nin;
-          if (nin < 64u) break;
-        }
-        if (cur.cov >= need) break;  // every index of this group is resolved
-        n2v_refill(clist, (uint32_t)c.deg, plist, (uint32_t)c.prev_deg, *scr, cur, lane);
-      }
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      const uint32_t common = scr->mask[lane];
-      int ret_slot = -1;  // which of this lane's biases is the return edge
-      if (ret_idx >= gs && ret_idx < ge) {
-        const uint32_t rel = (uint32_t)(ret_idx - gs);
-        const uint32_t qd = rel >> 2;
-        if ((int)(qd & 63u) == lane) ret_slot = (int)(((qd >> 6) << 2) | (rel & 3u));
-      }
-#pragma unroll
-      for (int i = 0; i < kEl; ++i) {
-        const float wq = x[i] * a.inv_q;
-        const float wp = x[i] * a.inv_p;
-        x[i] = (i == ret_slot) ? wp : (((common >> i) & 1u) ? x[i] : wq);
-      }
-    } else if (n2v && p_staged) {  // include/app.cuh:108-123 against the staged N(prev)
-      const int32_t* win = scr->window;
-#pragma unroll
-      for (int j = 0; j < kJ; ++j) {
-        const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (post[e] == c.prev) {  // the return edge, or an entry outside the list (bias 0 already)
-            x[4 * j + e] = x[4 * j + e] * a.inv_p;
-          } else {
-            lane_pos = gallop_lower_bound(win, lane_pos, st_hi, post[e], e == 0 ? kN2vQuartetStride : 1u);
-            const bool common = lane_pos < st_hi && win[lane_pos] == post[e];
-            x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
-          }
-        }
-      }
-    } else if (n2v) {  // include/app.cuh:108-123: w/p back to prev, w for common neighbours, w/q otherwise
-      const int32_t* __restrict__ plist = a.adjncy + c.prev_off;
-      // entries outside the list were replaced by prev above, so they never count as the group's maximum
-      int32_t vmax = (int)0x80000000;
-#pragma unroll
-      for (int j = 0; j < kJ; ++j) {
-        vmax = (adj[j].x != c.prev && adj[j].x > vmax) ? adj[j].x : vmax;
-        vmax = (adj[j].y != c.prev && adj[j].y > vmax) ? adj[j].y : vmax;
-        vmax = (adj[j].z != c.prev && adj[j].z > vmax) ? adj[j].z : vmax;
-        vmax = (adj[j].w != c.prev && adj[j].w > vmax) ? adj[j].w : vmax;
-      }
-      vmax = wave_max_i32(vmax);
-      // N(prev)[seg_lo, seg_hi) can hold this group's vertices; later groups only hold larger ones
-      if (nw > 1u) {  // this wave skipped the groups of the other waves: drop the entries below this group's first vertex
-        const int32_t gs = (int32_t)(a0 + 4u * g * kG - c.off);
-        const int32_t vmin = a.adjncy[c.off + (uint32_t)(gs > 0 ? gs : 0)];
-        seg_lo = coop_lower_bound(plist, seg_lo, (uint32_t)c.prev_deg, vmin, lane);
-      }
-      const uint32_t seg_hi = coop_upper_bound(plist, seg_lo, (uint32_t)c.prev_deg, vmax, lane);
-      const uint32_t p_lo = c.prev_off + seg_lo, p_hi = c.prev_off + seg_hi;  // the segment as CSR indices
-      const uint32_t wa = p_lo & ~3u;
-      if (p_hi - wa <= (uint32_t)kN2vWindow) {
-        // the segment fits the window: stage it with aligned 16-byte loads, then search in LDS
-        __builtin_amdgcn_wave_barrier();  // the previous group's searches are done
-#pragma unroll
-        for (int k = 0; k < kN2vWindow / 256; ++k) {
-          const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
-          if (wa + wi < p_hi)
-            *reinterpret_cast<int4*>(&scr->window[wi]) = *reinterpret_cast<const int4*>(a.adjncy + wa + wi);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        const int32_t* win = scr->window;
-        const uint32_t hi_w = p_hi - wa;
-        uint32_t pos = p_lo - wa;
-#pragma unroll
-        for (int j = 0; j < kJ; ++j) {
-          const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (post[e] == c.prev) {
-              x[4 * j + e] = x[4 * j + e] * a.inv_p;
-            } else {
-              pos = gallop_lower_bound(win, pos, hi_w, post[e], e == 0 ? kN2vQuartetStride : 1u);
-              const bool common = pos < hi_w && win[pos] == post[e];
-              x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
-            }
-          }
-        }
-      } else if (p_hi - wa <= (uint32_t)(kN2vMaxWindows * kN2vWindow)) {
-        // the segment is a few windows long: stream it through the window; a neighbour is resolved in the first
-        // window whose last entry is not smaller (both lists ascend, so a lane's neighbours come up in order)
-        uint32_t done = 0u;  // bit i: bias i is final
-#pragma unroll
-        for (int j = 0; j < kJ; ++j) {
-          const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (post[e] == c.prev) {
-              x[4 * j + e] = x[4 * j + e] * a.inv_p;
-              done |= 1u << (4 * j + e);
-            }
-          }
-        }
-        // the next window's entries are fetched into registers while the current window is searched
-        int4 ahead[kN2vWindow / 256];
-#pragma unroll
-        for (int k = 0; k < kN2vWindow / 256; ++k) {
-          const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
-          ahead[k] = make_int4(0, 0, 0, 0);
-          if (wa + wi < p_hi) ahead[k] = *reinterpret_cast<const int4*>(a.adjncy + wa + wi);
-        }
-        for (uint32_t ws = wa; ws < p_hi; ws += (uint32_t)kN2vWindow) {
-          __builtin_amdgcn_wave_barrier();  // the previous window's searches are done
-#pragma unroll
-          for (int k = 0; k < kN2vWindow / 256; ++k) {
-            const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
-            if (ws + wi < p_hi) *reinterpret_cast<int4*>(&scr->window[wi]) = ahead[k];
-          }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-          {
-            const uint32_t wn = ws + (uint32_t)kN2vWindow;
-#pragma unroll
-            for (int k = 0; k < kN2vWindow / 256; ++k) {
-              const uint32_t wi = 4u * ((uint32_t)lane + 64u * (uint32_t)k);
-              if (wn + wi < p_hi) ahead[k] = *reinterpret_cast<const int4*>(a.adjncy + wn + wi);
-            }
-          }
-          const int32_t* win = scr->window;
-          const uint32_t hi_w = (p_hi - ws) < (uint32_t)kN2vWindow ? (p_hi - ws) : (uint32_t)kN2vWindow;
-          const bool last = ws + (uint32_t)kN2vWindow >= p_hi;
-          const int32_t wmax = win[hi_w - 1u];
-          uint32_t pos = ws == wa ? p_lo - wa : 0u;
-          uint32_t stride = kN2vWindowStride;  // a lane's first search in a window starts anywhere in it
-#pragma unroll
-          for (int j = 0; j < kJ; ++j) {
-            const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int i = 4 * j + e;
-              if (((done >> i) & 1u) == 0u && (post[e] <= wmax || last)) {
-                pos = gallop_lower_bound(win, pos, hi_w, post[e], stride);
-                stride = kN2vStreamedStride;
-                const bool common = pos < hi_w && win[pos] == post[e];
-                x[i] = common ? x[i] : x[i] * a.inv_q;
-                done |= 1u << i;
-              }
-            }
-          }
-        }
-      } else {  // a long stretch of N(prev) against few neighbours: search it in place, galloping from hit to hit
-        uint32_t pos = seg_lo;
-#pragma unroll
-        for (int j = 0; j < kJ; ++j) {
-          const int32_t post[4] = {adj[j].x, adj[j].y, adj[j].z, adj[j].w};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (post[e] == c.prev) {
-              x[4 * j + e] = x[4 * j + e] * a.inv_p;
-            } else {
-              pos = gallop_lower_bound(plist, pos, seg_hi, post[e], e == 0 ? kN2vInPlaceQuartetStride : kN2vInPlaceStride);
-              const bool common = pos < seg_hi && plist[pos] == post[e];
-              x[4 * j + e] = common ? x[4 * j + e] : x[4 * j + e] * a.inv_q;
-            }
-          }
-        }
-      }
-      seg_lo = seg_hi;
-    }
-
     float q = 0.0f;
 #pragma unroll
     for (int i = 0; i < kEl; ++i) q = q + x[i];
@@ -629,8 +281,8 @@ struct TaskTable {
   // wave partials of the hub chunk in flight
   float hub_w[kHubChunk][16];
   int32_t hub_sel[kHubChunk][16];
-  // node2vec only: one scratch block per wave for the reversed adjacency test
-  N2vScratch n2v[kApp == FW_APP_NODE2VEC ? kWGT / 64 : 1];
+  // node2vec only: trials of the slot's current step that were rejected so far
+  int32_t trial[kApp == FW_APP_NODE2VEC ? kWGT : 1];
   // metapath only: the schema, so that the per-step label is an LDS read (a dynamic index into the
   // by-value kernel arguments would force a private copy of the whole array)
   int32_t schema[kApp == FW_APP_METAPATH ? FW_MAX_SCHEMA : 1];
@@ -649,6 +301,7 @@ __device__ __forceinline__ StepCtx load_ctx(const fw_kargs& a, const TaskTable<k
   c.walker = a.walker_base + (uint32_t)__builtin_amdgcn_readfirstlane(tt.walker[slot]);
   c.step = (uint32_t)(__builtin_amdgcn_readfirstlane(tt.len[slot]) - 1);
   c.want = 0;
+  c.sbase = kApp == FW_APP_NODE2VEC ? (uint32_t)__builtin_amdgcn_readfirstlane(tt.trial[slot]) << 8 : 0u;
   return c;
 }
 
@@ -660,6 +313,16 @@ __device__ __forceinline__ void commit(const fw_kargs& a, TaskTable<kWGT, kApp>&
   if (!ok) {
     tt.flag[slot] = kFlagDead;
     return;
+  }
+  if (kApp == FW_APP_NODE2VEC) {  // v is a proposal: accept it or sample again next round
+    uint32_t probes = 0u;
+    const uint32_t trial = c.sbase >> 8;
+    if (!n2v_accept(a, v, c.prev, c.prev_off, c.prev_deg, c.walker, c.step, trial, probes)) {
+      tt.trial[slot] = (int32_t)trial + 1;
+      tt.flag[slot] = kFlagRetry;
+      return;
+    }
+    tt.trial[slot] = 0;
   }
   const int32_t len = (int32_t)c.step + 1;
   a.paths[(uint64_t)(uint32_t)tt.walker[slot] * (uint64_t)a.max_depth + (uint64_t)len] = v;
@@ -785,11 +448,25 @@ __device__ __forceinline__ void packed_finish(const fw_kargs& a, TaskTable<kWGT,
   v = pick == 3 ? adj.w : v;
   const int32_t selv = __builtin_amdgcn_ds_bpermute((seg_first + l) << 2, v);
   if (active && c == 0) {  // commit (include/walker.cuh:1372-1385, Task::update include/gpu_task.cuh:70-77)
+    bool rejected = false;
+    if (kApp == FW_APP_NODE2VEC && accept) {  // selv is a proposal: accept it or sample again next round
+      uint32_t probes = 0u;
+      const uint32_t trial = (uint32_t)tt.trial[slot];
+      rejected = !n2v_accept(a, selv, tt.prev[slot], tt.prev_off[slot], tt.prev_deg[slot],
+                             a.walker_base + (uint32_t)tt.walker[slot], (uint32_t)(len - 1), trial, probes);
+      tt.trial[slot] = rejected ? (int32_t)trial + 1 : 0;
+    }
     if (!accept) {
       tt.flag[slot] = kFlagDead;
+    } else if (rejected) {
+      tt.flag[slot] = kFlagRetry;
     } else {
       a.paths[(uint64_t)(uint32_t)tt.walker[slot] * (uint64_t)a.max_depth + (uint64_t)len] = selv;
       tt.prev[slot] = tt.cur[slot];
+      if (kApp == FW_APP_NODE2VEC) {
+        tt.prev_off[slot] = off;
+        tt.prev_deg[slot] = (int32_t)deg;
+      }
       tt.cur[slot] = selv;
       tt.len[slot] = len + 1;
       tt.flag[slot] = kFlagMoved;
@@ -815,7 +492,7 @@ __device__ __forceinline__ void packed_step(const fw_kargs& a, TaskTable<kWGT, k
 // get); kPipelineInFlight for the launches of the parking pipeline, which are rounds of refills and packed steps
 // on short lists and wait for one bundle's loads after the other otherwise (110 VGPRs, two workgroups per CU).
 template <int kApp, int kWGT, int kPackedInFlight>
-__global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFlight == 1 ? 8 : 4)) void fw_walk_zprs(
+__global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zprs(
     const fw_kargs a) {
   constexpr int kNW = kWGT / 64;
   __shared__ TaskTable<kWGT, kApp> tt;
@@ -823,7 +500,6 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFligh
   const int tid = (int)threadIdx.x;
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  N2vScratch* const scr = &tt.n2v[kApp == FW_APP_NODE2VEC ? wave : 0];
   unsigned long long n_steps = 0ull, n_edges = 0ull;
   // entries of this launch and the slots a workgroup fills: from the host, or (a launch queued before its input's
   // size was known to the host) from the device, with the same rule: small inputs are spread over the grid
@@ -837,6 +513,7 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFligh
 
   tt.len[tid] = -1;
   tt.flag[tid] = 0;
+  if (kApp == FW_APP_NODE2VEC) tt.trial[tid] = 0;
   if (kApp == FW_APP_METAPATH && tid == 0) {
 #pragma unroll
     for (int i = 0; i < FW_MAX_SCHEMA; ++i) tt.schema[i] = a.schema[i];
@@ -874,7 +551,7 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFligh
           if (kApp == FW_APP_METAPATH) c.want = tt.schema[c.step % (uint32_t)a.schema_len];
           float W;
           int32_t sel, selv;
-          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, (uint32_t)wave, (uint32_t)kNW, scr, DrawQueue(), W, sel,
+          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, (uint32_t)wave, (uint32_t)kNW, DrawQueue(), W, sel,
                                                    selv);
           if (lane == 0) {
             tt.hub_w[h][wave] = W;
@@ -894,7 +571,7 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFligh
           // inverse transform over the wave totals (lanes >= kNW hold 0 and never qualify)
           const float J = row_scan(W);
           const float total = readlane_f(J, kNW - 1);
-          const uint32_t bits = philox4x32_10(c.walker, c.step, kStreamWave, 0u, a.seed_lo, a.seed_hi).x;
+          const uint32_t bits = philox4x32_10(c.walker, c.step, kStreamWave | c.sbase, 0u, a.seed_lo, a.seed_hi).x;
           const float target = u24(bits) * total;
           const bool pos = W > 0.0f;
           uint64_t m = __ballot(pos && J > target);
@@ -915,7 +592,7 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFligh
       }
 
       // ---- phase A: remaining slots, claimed dynamically: four or two short lists per wave, else one ----
-      if (kApp != FW_APP_NODE2VEC) {
+      {
         // kPackedInFlight bundles per turn: their loads are in flight together, so a wave waits for memory once per
         // turn instead of once per bundle (the registers are there: two workgroups per CU fit with up to 128)
         for (;;) {
@@ -969,10 +646,10 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFligh
         dq0.avail = 4u;
         dq0.blk = 1u;
         if (nq <= 64u) {  // one quartet per lane: fetch the adjacency with the biases, no dependent load
-          wave_stream<kApp, 1, true>(a, c, lane, 0u, 1u, scr, dq0, W, sel, selv);
+          wave_stream<kApp, 1, true>(a, c, lane, 0u, 1u, dq0, W, sel, selv);
           v = selv;
         } else {
-          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, 0u, 1u, scr, dq0, W, sel, selv);
+          wave_stream<kApp, kGroupQuartets, false>(a, c, lane, 0u, 1u, dq0, W, sel, selv);
           if (sel >= 0) v = a.adjncy[c.off + (uint32_t)sel];
         }
         if (lane == 0) commit(a, tt, slot, c, v, sel >= 0, n_steps, n_edges);
@@ -1018,6 +695,9 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFligh
           }
           need = stop;
           park = !stop && hidx >= 0;  // same as deg > park_threshold
+        } else if (kApp == FW_APP_NODE2VEC && tt.flag[tid] == kFlagRetry) {
+          need = false;  // the proposal was rejected: the walker stays and samples again (tt.trial counts)
+          deg = tt.deg[tid];
         }
         // kFlagDead: dead end (no neighbour with positive bias), include/walker.cuh:1373-1374
       }
@@ -1073,12 +753,16 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFligh
             q = pos < (uint64_t)n_entries ? (uint32_t)pos : 0xFFFFFFFFu;
           }
           if (q < n_entries) {
-            int32_t wq, sp, pv, ln;
+            int32_t wq, sp, pv, ln, tr = 0;
             if (a.resume != nullptr) {  // a walker coming back from its batch step
               const fw_walker_rec rec = a.resume[q];
               wq = rec.q; sp = rec.cur; pv = rec.prev; ln = rec.len;
               // the list has holes: walks that ended, and walkers that wait on their next vertex already
               if (rec.q < 0 || (rec.len & FW_REC_PARK) != 0) sp = -1;
+              if (kApp == FW_APP_NODE2VEC) {  // the rejected trials of the walker's current step travel with its length
+                tr = (ln >> FW_REC_TRIAL_SHIFT) & FW_REC_TRIAL_MASK;
+                ln &= FW_REC_LEN_MASK;
+              }
             } else {                    // a fresh query (include/walker.cuh:1340-1343)
               wq = (int32_t)q; sp = a.starts[q]; pv = -1; ln = 1;
               a.paths[(uint64_t)q * (uint64_t)a.max_depth] = sp;
@@ -1096,6 +780,14 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFligh
                 tt.deg[tid] = deg;
                 tt.prev_off[tid] = 0;
                 tt.prev_deg[tid] = 0;
+                if (kApp == FW_APP_NODE2VEC) {
+                  tt.trial[tid] = tr;
+                  if (pv >= 0) {  // the acceptance test searches N(prev)
+                    const uint32_t po = a.xadj[pv];
+                    tt.prev_off[tid] = po;
+                    tt.prev_deg[tid] = (int32_t)(a.xadj[pv + 1] - po);
+                  }
+                }
                 len = ln;
                 need = false;
                 park = hidx >= 0;  // same as deg > park_threshold
@@ -1117,15 +809,16 @@ __global__ __launch_bounds__(kWGT, kApp == FW_APP_NODE2VEC ? 1 : (kPackedInFligh
         } else {
           const uint32_t o = tt.off[tid];
           const uint32_t nq = (o + (uint32_t)deg - (o & ~3u) + 3u) >> 2;
-          if (kApp != FW_APP_NODE2VEC && nq <= 16u) {
+          if (nq <= 16u) {
             tt.tiny_list[np][atomicAdd(&tt.tiny_count[np], 1)] = (uint16_t)tid;
-          } else if (kApp != FW_APP_NODE2VEC && nq <= 32u) {
+          } else if (nq <= 32u) {
             tt.half_list[np][atomicAdd(&tt.half_count[np], 1)] = (uint16_t)tid;
           } else {
             tt.small_list[np][atomicAdd(&tt.small_count[np], 1)] = (uint16_t)tid;
           }
           if (kApp == FW_APP_METAPATH) tt.want[tid] = tt.schema[(uint32_t)(len - 1) % (uint32_t)a.schema_len];
-          const uint4 b = philox4x32_10(a.walker_base + (uint32_t)tt.walker[tid], (uint32_t)(len - 1), 0u, 0u,
+          const uint32_t sbase = kApp == FW_APP_NODE2VEC ? (uint32_t)tt.trial[tid] << 8 : 0u;
+          const uint4 b = philox4x32_10(a.walker_base + (uint32_t)tt.walker[tid], (uint32_t)(len - 1), sbase, 0u,
                                         a.seed_lo, a.seed_hi);
           tt.draw[0][tid] = b.x;
           tt.draw[1][tid] = b.y;
@@ -1187,7 +880,8 @@ template <int kApp>
 __device__ __forceinline__ void batch_stream(const fw_kargs& a, const uint32_t* __restrict__ bias, const uint32_t off,
                                              const uint32_t deg, const int32_t want, const uint32_t w,
                                              const uint32_t nw, const bool have, const uint32_t walker,
-                                             const uint32_t step, const int lane, float& S_out, int32_t& sel_out) {
+                                             const uint32_t step, const uint32_t sbase, const int lane, float& S_out,
+                                             int32_t& sel_out) {
   constexpr uint32_t kG = 64u * kGroupQuartets;
   constexpr int kEl = 4 * kGroupQuartets;
   const uint32_t a0 = off & ~3u;
@@ -1251,7 +945,7 @@ __device__ __forceinline__ void batch_stream(const fw_kargs& a, const uint32_t* 
     const uint64_t macc = __ballot(acc);
     if (macc != 0ull) {
       float target = 0.0f;
-      if (acc) target = next_uniform_lane(dq, a, walker, step, w) * T;
+      if (acc) target = next_uniform_lane(dq, a, walker, step, w | sbase) * T;
       // which lane's biases hold the target of walker k: first lane with a positive total whose prefix
       // exceeds it, else the last lane with a positive total
       const bool pos = q > 0.0f;
@@ -1288,7 +982,7 @@ __device__ __forceinline__ void batch_stream(const fw_kargs& a, const uint32_t* 
         const uint32_t abs_idx = a0 + 4u * (g * kG + (uint32_t)src) + 256u * (uint32_t)(pick >> 2) + (uint32_t)(pick & 3);
         sel = (int32_t)(abs_idx - off);
         Sj = Snew;
-        u = next_uniform_lane(dq, a, walker, step, w);
+        u = next_uniform_lane(dq, a, walker, step, w | sbase);
       }
     }
     S = Snew;
@@ -1447,7 +1141,7 @@ __device__ __forceinline__ int32_t resolve_pick(const uint32_t* __restrict__ bia
 // test that failed on S fails again.
 __device__ __forceinline__ void table_reservoir(const fw_kargs& a, const float* totals, const uint32_t ngroups,
                                                 const uint32_t seq, const uint32_t nw, const uint32_t walker,
-                                                const uint32_t step, int32_t& gsel, float& tsel) {
+                                                const uint32_t step, const uint32_t sbase, int32_t& gsel, float& tsel) {
   float S = 0.0f, Sj = 0.0f, u = 1.0f;
   LaneDraw dq;
   gsel = -1;
@@ -1463,10 +1157,10 @@ __device__ __forceinline__ void table_reservoir(const fw_kargs& a, const float* 
     for (int j = 0; j < 4; ++j) {
       const float Snew = S + t4[j];
       if (Snew * u > Sj) {
-        tsel = next_uniform_lane(dq, a, walker, step, seq) * t4[j];
+        tsel = next_uniform_lane(dq, a, walker, step, seq | sbase) * t4[j];
         gsel = (int32_t)(g0 + (uint32_t)j * nw);
         Sj = Snew;
-        u = next_uniform_lane(dq, a, walker, step, seq);
+        u = next_uniform_lane(dq, a, walker, step, seq | sbase);
       }
       S = Snew;
     }
@@ -1478,8 +1172,9 @@ __device__ __forceinline__ void table_reservoir(const fw_kargs& a, const float* 
 template <int kApp, int kNW>
 __device__ __forceinline__ int32_t table_sample(const fw_kargs& a, const uint32_t* __restrict__ bias, const uint32_t off,
                                                 const uint32_t deg, const int32_t want, const bool wg, const bool have,
-                                                const uint32_t walker, const uint32_t step, const int lane,
-                                                const float* totals, const float* rows, const int32_t* lastpos) {
+                                                const uint32_t walker, const uint32_t step, const uint32_t sbase,
+                                                const int lane, const float* totals, const float* rows,
+                                                const int32_t* lastpos) {
   constexpr uint32_t kG = 64u * kGroupQuartets;
   const uint32_t nq = (off + deg - (off & ~3u) + 3u) >> 2;
   const uint32_t ngroups = (nq + kG - 1u) / kG;
@@ -1502,7 +1197,7 @@ __device__ __forceinline__ int32_t table_sample(const fw_kargs& a, const uint32_
     }
     const float J = row_scan(Wl);
     const float total = readlane_f(J, kNW - 1);
-    const float target = u24(philox4x32_10(walker, step, kStreamWave, 0u, a.seed_lo, a.seed_hi).x) * total;
+    const float target = u24(philox4x32_10(walker, step, kStreamWave | sbase, 0u, a.seed_lo, a.seed_hi).x) * total;
     int wlast = -1;
     wsel = -1;
 #pragma unroll
@@ -1519,7 +1214,7 @@ __device__ __forceinline__ int32_t table_sample(const fw_kargs& a, const uint32_
   // only the sequence the walker ends up in needs running: the draws of a sequence are addressed by the sequence
   int32_t gsel = -1;
   float tsel = 0.0f;
-  if (have && wsel >= 0) table_reservoir(a, totals, ngroups, (uint32_t)wsel, nw, walker, step, gsel, tsel);
+  if (have && wsel >= 0) table_reservoir(a, totals, ngroups, (uint32_t)wsel, nw, walker, step, sbase, gsel, tsel);
   int32_t pick = -1;
   if (gsel >= 0) pick = resolve_pick<kApp>(bias, off, deg, want, rows, lastpos, gsel, tsel);
   return pick;
@@ -1529,18 +1224,32 @@ __device__ __forceinline__ int32_t table_sample(const fw_kargs& a, const uint32_
 // goes back to its own position of the output list, so no list counter is contended: finished walks are marked
 // (q = -1), walkers whose new vertex is parked on again are tagged and carry their position inside that vertex's
 // bucket, the others are picked up from the same list by the next walk launch.
+// node2vec: `pick` is a proposal.  A walker whose proposal is rejected stays parked on v with one more trial on its
+// record; records carry the previous vertex instead of a position (the scatter kernel hands the positions out).
 template <int kApp>
 __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_args& h, const int32_t v,
                                              const uint32_t off, const uint32_t deg, const uint32_t rec_base,
-                                             const fw_walker_rec rec, const bool have, const int32_t pick,
-                                             const uint32_t walker, const uint32_t step, const int lane,
-                                             unsigned long long& n_steps, unsigned long long& n_edges,
-                                             uint32_t (&n_out)[2]) {
-  const bool moved = have && pick >= 0;
+                                             const fw_walker_rec rec, const uint32_t trial, const bool have,
+                                             const int32_t pick, const uint32_t walker, const uint32_t step,
+                                             const int lane, unsigned long long& n_steps,
+                                             unsigned long long& n_edges, uint32_t (&n_out)[2]) {
+  bool moved = have && pick >= 0;
+  bool retry = false;
   bool go_on = false;
   int32_t nv = -1;
   if (moved) {
     nv = a.adjncy[off + (uint32_t)pick];
+    if (kApp == FW_APP_NODE2VEC && rec.prev >= 0) {
+      uint32_t probes = 0u;
+      const uint32_t po = a.xadj[rec.prev];
+      const int32_t pd = (int32_t)(a.xadj[rec.prev + 1] - po);
+      if (!n2v_accept(a, nv, rec.prev, po, pd, walker, step, trial, probes)) {
+        moved = false;
+        retry = true;
+      }
+    }
+  }
+  if (moved) {
     a.paths[(uint64_t)(uint32_t)rec.q * (uint64_t)a.max_depth + (uint64_t)rec.len] = nv;
     go_on = rec.len + 1 < a.max_depth;
     if (kApp == FW_APP_PPR && go_on) {
@@ -1563,18 +1272,29 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
     go_on = hidx != -2;
     park = hidx >= 0;
   }
+  if (kApp == FW_APP_NODE2VEC && retry) {  // back into the bucket it came from
+    hidx = a.hub_index[v];
+    go_on = true;
+    park = true;
+  }
   const uint32_t label_slot = kApp == FW_APP_METAPATH ? (uint32_t)rec.len % (uint32_t)a.n_labels_per_hub : 0u;
   const uint32_t bucket = (uint32_t)hidx * (uint32_t)a.n_labels_per_hub + label_slot;
-  const uint32_t rank = fw_wave_count_keys<true>(h.bucket_out, bucket, go_on && park);
+  uint32_t rank = 0u;
+  if (kApp == FW_APP_NODE2VEC) fw_wave_count_keys<false>(h.bucket_out, bucket, go_on && park);
+  else rank = fw_wave_count_keys<true>(h.bucket_out, bucket, go_on && park);
   if (have) {
     fw_walker_rec out;
     out.q = go_on ? rec.q : -1;
     out.cur = nv;
     out.prev = v;
     out.len = rec.len + 1;
-    if (go_on && park) {
+    if (kApp == FW_APP_NODE2VEC && retry) {
+      out.cur = (int32_t)bucket;
+      out.prev = rec.prev;
+      out.len = rec.len | (int32_t)((trial + 1u) << FW_REC_TRIAL_SHIFT) | FW_REC_PARK;
+    } else if (go_on && park) {
       out.cur = (int32_t)bucket;  // the vertex follows from the bucket
-      out.prev = (int32_t)rank;
+      if (kApp != FW_APP_NODE2VEC) out.prev = (int32_t)rank;
       out.len |= FW_REC_PARK;
     }
     h.out[rec_base + (uint32_t)lane] = out;
@@ -1635,13 +1355,18 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     fw_walker_rec rec;
     rec.q = 0; rec.cur = v; rec.prev = -1; rec.len = 1;
     if (have) rec = h.sorted[rec_base + (uint32_t)lane];
+    uint32_t trial = 0u;
+    if (kApp == FW_APP_NODE2VEC) {
+      trial = (uint32_t)((rec.len >> FW_REC_TRIAL_SHIFT) & FW_REC_TRIAL_MASK);
+      rec.len &= FW_REC_LEN_MASK;
+    }
     const uint32_t walker = a.walker_base + (uint32_t)rec.q;
     const uint32_t step = (uint32_t)(rec.len - 1);
 
     const int32_t sel = table_sample<kApp, kNW>(a, bias, off, deg, want, (int32_t)deg > a.hub_threshold, have, walker,
-                                               step, lane, h.totals + row_base, h.rows + (size_t)row_base * 128u,
-                                               h.lastpos + row_base);
-    batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, have, sel, walker, step, lane, n_steps, n_edges, n_out);
+                                               step, trial << 8, lane, h.totals + row_base,
+                                               h.rows + (size_t)row_base * 128u, h.lastpos + row_base);
+    batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, trial, have, sel, walker, step, lane, n_steps, n_edges, n_out);
   }
 
   // ---- then wave tasks: lists up to hub_threshold, sampled at wave granularity, one batch per wave; the tasks are
@@ -1659,13 +1384,18 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     fw_walker_rec rec;
     rec.q = 0; rec.cur = v; rec.prev = -1; rec.len = 1;
     if (have) rec = h.sorted[rec_base + (uint32_t)lane];
+    uint32_t trial = 0u;
+    if (kApp == FW_APP_NODE2VEC) {
+      trial = (uint32_t)((rec.len >> FW_REC_TRIAL_SHIFT) & FW_REC_TRIAL_MASK);
+      rec.len &= FW_REC_LEN_MASK;
+    }
     const uint32_t walker = a.walker_base + (uint32_t)rec.q;
     const uint32_t step = (uint32_t)(rec.len - 1);
 
     float S;
     int32_t sel;
-    batch_stream<kApp>(a, bias, off, deg, want, 0u, 1u, have, walker, step, lane, S, sel);
-    batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, have, sel, walker, step, lane, n_steps, n_edges, n_out);
+    batch_stream<kApp>(a, bias, off, deg, want, 0u, 1u, have, walker, step, trial << 8, lane, S, sel);
+    batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, trial, have, sel, walker, step, lane, n_steps, n_edges, n_out);
   }
 
   // ---- then workgroup tasks: lists above hub_threshold, sampled at workgroup granularity.  They are few, long and
@@ -1689,13 +1419,18 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     fw_walker_rec rec;
     rec.q = 0; rec.cur = task.v; rec.prev = -1; rec.len = 1;
     if (have) rec = h.sorted[task.rec_base + (uint32_t)lane];
+    uint32_t trial = 0u;
+    if (kApp == FW_APP_NODE2VEC) {
+      trial = (uint32_t)((rec.len >> FW_REC_TRIAL_SHIFT) & FW_REC_TRIAL_MASK);
+      rec.len &= FW_REC_LEN_MASK;
+    }
     const uint32_t walker = a.walker_base + (uint32_t)rec.q;
     const uint32_t step = (uint32_t)(rec.len - 1);
 
     float S;
     int32_t sel;
-    batch_stream<kApp>(a, bias, task.off, task.deg, want, (uint32_t)wave, (uint32_t)kNW, have, walker, step, lane, S,
-                       sel);
+    batch_stream<kApp>(a, bias, task.off, task.deg, want, (uint32_t)wave, (uint32_t)kNW, have, walker, step, trial << 8,
+                       lane, S, sel);
     s_sel[wave][lane] = sel;
     if (lane == 0) s_w[wave] = S;
     __syncthreads();
@@ -1707,7 +1442,7 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
       const float total = readlane_f(J, kNW - 1);
       int32_t pick = -1;
       if (have) {
-        const float target = u24(philox4x32_10(walker, step, kStreamWave, 0u, a.seed_lo, a.seed_hi).x) * total;
+        const float target = u24(philox4x32_10(walker, step, kStreamWave | (trial << 8), 0u, a.seed_lo, a.seed_hi).x) * total;
         int wsel = -1, wlast = -1;
 #pragma unroll
         for (int w = 0; w < kNW; ++w) {
@@ -1721,7 +1456,7 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
         wsel = wsel < 0 ? wlast : wsel;
         if (wsel >= 0) pick = s_sel[wsel][lane];
       }
-      batch_commit<kApp>(a, h, task.v, task.off, task.deg, task.rec_base, rec, have, pick, walker, step, lane,
+      batch_commit<kApp>(a, h, task.v, task.off, task.deg, task.rec_base, rec, trial, have, pick, walker, step, lane,
                          n_steps, n_edges, n_out);
     }
   }
@@ -1731,13 +1466,16 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
   if (n_steps != 0ull) {
     atomicAdd(&s_acc[0], n_steps);
     atomicAdd(&s_acc[1], n_edges);
-    atomicAdd(&s_out[0], n_out[0]);
-    atomicAdd(&s_out[1], n_out[1]);
   }
+  // (a wave of node2vec walkers whose proposals were all rejected has walkers to hand on and no steps)
+  if (n_out[0] != 0u) atomicAdd(&s_out[0], n_out[0]);
+  if (n_out[1] != 0u) atomicAdd(&s_out[1], n_out[1]);
   __syncthreads();
-  if (tid == 0 && s_acc[0] != 0ull) {
-    atomicAdd(&a.counters[2], s_acc[0]);
-    atomicAdd(&a.counters[3], s_acc[1]);
+  if (tid == 0) {
+    if (s_acc[0] != 0ull) {
+      atomicAdd(&a.counters[2], s_acc[0]);
+      atomicAdd(&a.counters[3], s_acc[1]);
+    }
     if (s_out[0] != 0u) atomicAdd(&h.out_counts[0], s_out[0]);
     if (s_out[1] != 0u) atomicAdd(&h.out_counts[1], s_out[1]);
   }
@@ -1873,7 +1611,7 @@ template <int kApp, int kWGT>
 int launch_one(fw_kargs a, int grid, uint32_t entries_hint, hipStream_t stream, int* grid_used) {
   // launches of the parking pipeline (they park, or they continue parked walkers) take the variant with several
   // bundles in flight
-  constexpr int kFlight = kApp == FW_APP_NODE2VEC ? 1 : kPipelineInFlight;
+  constexpr int kFlight = kPipelineInFlight;
   const bool pipeline = kFlight != 1 && (a.park_threshold != 0x7FFFFFFF || a.resume != nullptr);
   if (grid <= 0) {
     int cus = 0, per_cu = 0;
@@ -1919,9 +1657,10 @@ int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, uint32_
   switch (app) {
     case FW_APP_DEEPWALK: return launch_hub_scan_app<FW_APP_DEEPWALK>(a, h, tasks_hint, stream);
     case FW_APP_PPR: return launch_hub_scan_app<FW_APP_PPR>(a, h, tasks_hint, stream);
+    case FW_APP_NODE2VEC: return launch_hub_scan_app<FW_APP_DEEPWALK>(a, h, tasks_hint, stream);  // the same rows: plain weights
     case FW_APP_METAPATH: return launch_hub_scan_app<FW_APP_METAPATH>(a, h, tasks_hint, stream);
     default:
-      fw_set_error("the hub scan kernel serves DeepWalk, PPR and MetaPath");
+      fw_set_error("unknown app %d", app);
       return FW_ERR_INVALID;
   }
 }
@@ -1931,9 +1670,10 @@ int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg
   switch (app) {
     case FW_APP_DEEPWALK: return launch_hub_app<FW_APP_DEEPWALK>(a, h, wg_threads, tasks_hint, stream);
     case FW_APP_PPR: return launch_hub_app<FW_APP_PPR>(a, h, wg_threads, tasks_hint, stream);
+    case FW_APP_NODE2VEC: return launch_hub_app<FW_APP_NODE2VEC>(a, h, wg_threads, tasks_hint, stream);
     case FW_APP_METAPATH: return launch_hub_app<FW_APP_METAPATH>(a, h, wg_threads, tasks_hint, stream);
     default:
-      fw_set_error("the hub batch kernel serves DeepWalk, PPR and MetaPath (node2vec biases depend on the walker)");
+      fw_set_error("unknown app %d", app);
       return FW_ERR_INVALID;
   }
 }

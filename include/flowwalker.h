@@ -79,7 +79,8 @@ typedef struct {
   int32_t park_threshold; /* hub parking, an execution strategy that never changes results: walkers that arrive on a
                             vertex of larger degree wait there and are served 64 at a time by one shared scan of its
                             list (by a workgroup above hub_threshold, by one wave below).  0 = library default (on
-                            for batches >= 65536 queries), < 0 = off, > 0 = degree.  Not used by node2vec. */
+                            for batches >= 65536 queries), < 0 = off, > 0 = degree.  node2vec: the shared scan
+                            proposes, each walker accepts with its own adjacency test (max_depth <= 65535). */
 } fw_walk_params;
 
 /* What src/main.cu:82-113 (calculate_workload) and the timing code of src/walk.cu report. */
@@ -98,8 +99,8 @@ typedef struct {
   /* Bytes the call's kernels requested from the memory system, from the run's own counters: every list pass in
    * 16-byte quartets (a list is read once per walker step by the walk kernel, once per batch of up to 64 walkers
    * or once per round by the hub kernels), 64 bytes for every scattered access (path entry, xadj pair, parking
-   * index, bucket counter, selected neighbour), 16 bytes per walker record moved.  node2vec: the probes of its
-   * adjacency test are not included.  What sits between the algorithmic bytes of src/main.cu:93-111
+   * index, bucket counter, selected neighbour), 16 bytes per walker record moved, node2vec: 16 lines per step for
+   * the binary search of its acceptance test.  What sits between the algorithmic bytes of src/main.cu:93-111
    * (4 * sampled_edges + ...) and what the HBM counters of a profiler see. */
   uint64_t requested_bytes;
 } fw_walk_stats;
@@ -120,10 +121,9 @@ int fw_device_mem_info(size_t* free_bytes, size_t* total_bytes);
 /* Fills defaults: app DeepWalk, d = 80, tp 0.2, p 2.0, q 0.5, schema 0,1,2,3,4, seed 1337 (src/main.cu:40-80). */
 void fw_walk_params_default(fw_walk_params* p);
 
-/* The same defaults with `app` set and what the library would choose for that application: node2vec samples every
- * list at wave granularity (hub_threshold INT32_MAX), because only a single wave can look a short N(prev) up in
- * N(cur) instead of testing every neighbour of cur.  The reference also picks node2vec's kernel by application
- * (the one-pass sampler, src/walk.cu:403). */
+/* The same defaults with `app` set and whatever the library would choose differently for that application (the
+ * reference picks node2vec's kernel by application, src/walk.cu:403; this library's choices are the same for all
+ * four today). */
 void fw_walk_params_default_for(fw_walk_params* p, int app);
 
 /*

@@ -41,7 +41,17 @@
  *       aligned vector loads on the GPU).
  *   - PPR stop draw is made once per completed step of a live walk, from its own stream
  *       (the reference also draws for empty slots, include/walker.cuh:1422-1431).
- *   - node2vec multiplies by host-computed f32 reciprocals 1/p and 1/q instead of dividing.
+ *   - node2vec samples in two stages.  The reference evaluates the bias w * f (f = 1/p for the return edge, 1 for a
+ *       common neighbour of prev and cur, 1/q otherwise; include/app.cuh:108-123) of EVERY neighbour, one binary
+ *       search each, inside its one-pass sampler.  Here a trial proposes a neighbour with probability w_i / sum w
+ *       through the same sampler DeepWalk uses (no adjacency test at all) and accepts it with probability f_i / F,
+ *       F = max(1, 1/p, 1/q), which takes ONE adjacency test (include/gpu_graph.cuh:97-118); a rejected trial is
+ *       followed by another with its own draws.  P(i) = (w_i / sum w)(f_i / F) / sum_j (w_j / sum w)(f_j / F) =
+ *       w_i f_i / sum_j w_j f_j: the reference's law exactly (its own rejection sampler has the same structure,
+ *       include/sampler.cuh:202-266).  Draws of trial t use the streams of a plain step offset by t << 8; the
+ *       acceptance uniform is word 0 of block 0 of stream FW_STREAM_ACCEPT | t << 8; trial FW_MAX_TRIALS - 1 is accepted
+ *       unconditionally (never reached in practice: the acceptance probability is at least min(f) / F).
+ *       f uses host-computed f32 reciprocals 1/p and 1/q; the test is u * F < f, no division.
  *   - --dprs selects nothing different: the one sampler already has DPRS's property (one bias
  *       evaluation per neighbour, include/sampler.cuh:129-200), so FW_SAMPLER_DPRS is an alias.
  *
@@ -69,8 +79,10 @@ int32_t fw_ref64_zprs(const float* w, int32_t n, int32_t W, const float* u);
 int32_t fw_ref64_dprs(const float* w, int32_t n, int32_t W, const float* u);
 float fw_ref64_uniform(uint64_t seed, uint32_t walker, uint32_t step, uint32_t i, uint32_t W);
 
-#define FW_STREAM_WAVE 0x40000000u /* workgroup-level combine draw */
-#define FW_STREAM_STOP 0x80000000u /* PPR stop draw */
+#define FW_STREAM_WAVE 0x40000000u   /* workgroup-level combine draw */
+#define FW_STREAM_STOP 0x80000000u   /* PPR stop draw */
+#define FW_STREAM_ACCEPT 0x10000000u /* node2vec acceptance draw of a trial */
+#define FW_MAX_TRIALS 16384u         /* node2vec: trials per step (the trial index travels in 14 bits) */
 
 typedef struct {
   int32_t app;           /* FW_APP_* */
@@ -169,6 +181,9 @@ typedef struct {
   uint32_t prev_off;  /* CSR range of prev (node2vec) */
   int32_t prev_deg;
   int32_t want_label; /* metapath: schema[step % schema_len] */
+  int n2v_full;       /* node2vec: 1 = the full bias w * f of every neighbour (the reference's samplers), 0 = the plain
+                         weight (proposal stage of this build's two-stage step) */
+  uint32_t stream_base; /* added to every stream of the step's sampler draws: trial << 8 */
   /* exhaustive tests only (fw_oracle_enumerate_draw): draw (force_stream, force_index) of the step takes
    * force_value instead of its Philox word, and the walker-independent rows of a group are kept between calls */
   int force;
@@ -190,7 +205,7 @@ typedef struct group_rows {
 /* n-th uniform of stream `stream` at (walker, step) */
 static float step_draw(const bias_ctx* c, uint32_t walker, uint32_t step, uint32_t stream, uint32_t n) {
   if (c->force && stream == c->force_stream && n == c->force_index) return c->force_value;
-  return u24(draw_bits(c->p->seed, walker, step, stream, n));
+  return u24(draw_bits(c->p->seed, walker, step, stream | c->stream_base, n));
 }
 
 /* include/gpu_graph.cuh:97-112 */
@@ -211,7 +226,7 @@ static float bias_at(const bias_ctx* c, uint64_t a) {
       return c->g->label[a] == c->want_label ? 1.0f : 0.0f;
     case FW_APP_NODE2VEC: {
       float w = c->g->weight[a];
-      if (c->prev == -1) return w;
+      if (c->prev == -1 || !c->n2v_full) return w;
       int32_t post = c->g->adjncy[a];
       if (post == c->prev) return w * c->p->inv_p;
       if (!sorted_contains(c->g->adjncy + c->prev_off, c->prev_deg, post)) return w * c->p->inv_q;
@@ -332,6 +347,7 @@ int32_t fw_oracle_sample(const fw_oracle_graph* g, const fw_oracle_params* p, in
   c.g = g; c.p = p; c.prev = prev;
   c.prev_off = 0; c.prev_deg = 0;
   c.force = 0; c.cache = NULL; c.cache_groups = 0;
+  c.n2v_full = 0; c.stream_base = 0;
   if (prev >= 0) { c.prev_off = g->xadj[prev]; c.prev_deg = (int32_t)(g->xadj[prev + 1] - g->xadj[prev]); }
   c.want_label = (p->app == FW_APP_METAPATH && p->schema_len > 0) ? p->schema[step % (uint32_t)p->schema_len] : 0;
   uint32_t off = g->xadj[cur];
@@ -341,6 +357,7 @@ int32_t fw_oracle_sample(const fw_oracle_graph* g, const fw_oracle_params* p, in
   if (kind == FW_SAMPLER_REF_ZPRS || kind == FW_SAMPLER_REF_DPRS) {
     /* the reference's own samplers on 64-lane waves (fw_ref_samplers.c), fed with this build's biases and uniforms */
     if (deg <= 0) return -1;
+    c.n2v_full = 1;
     const int32_t W = nw * FW_WAVE;
     float* w = (float*)malloc(sizeof(float) * (size_t)deg);
     float* u = (float*)malloc(sizeof(float) * (size_t)deg);
@@ -353,7 +370,25 @@ int32_t fw_oracle_sample(const fw_oracle_graph* g, const fw_oracle_params* p, in
     free(u);
     return sel;
   }
-  return group_sample(&c, off, deg, nw, walker, step);
+  if (p->app != FW_APP_NODE2VEC || prev < 0) return group_sample(&c, off, deg, nw, walker, step);
+  /* node2vec after the first step: propose by weight, accept by f / F (include/app.cuh:108-123 for f) */
+  float F = 1.0f;
+  if (p->inv_p > F) F = p->inv_p;
+  if (p->inv_q > F) F = p->inv_q;
+  for (uint32_t trial = 0;; ++trial) {
+    c.stream_base = trial << 8;
+    const int32_t sel = group_sample(&c, off, deg, nw, walker, step);
+    if (sel < 0) return -1; /* no positive weight: dead end, whatever the trial */
+    if (trial == FW_MAX_TRIALS - 1u) return sel;
+    const int32_t post = g->adjncy[(uint64_t)off + (uint32_t)sel];
+    float f;
+    if (post == prev) f = p->inv_p;
+    else if (sorted_contains(g->adjncy + c.prev_off, c.prev_deg, post)) f = 1.0f;
+    else f = p->inv_q;
+    const float u = u24(draw_bits(p->seed, walker, step, FW_STREAM_ACCEPT | (trial << 8), 0u));
+    const float lhs = u * F;
+    if (lhs < f) return sel;
+  }
 }
 
 /* ---- whole walks (include/walker.cuh:1338-1438) --------------------------------------------- */

@@ -68,18 +68,27 @@ def test_node2vec(gpu, hub):
     _check(gpu, hub, starts, app=gpu.APP_NODE2VEC, max_depth=16, p=2.0, q=0.5, hub_threshold=1000, seed=6)
 
 
-def test_node2vec_adjacency_test_strategies(gpu):
-    """The node2vec bias needs "is this neighbour of cur also a neighbour of prev?".  The kernel answers it in four
-    ways depending on the two list lengths (N(prev) entries looked up in N(cur); the stretch of N(prev) staged in LDS,
-    one window or several; searched in place) at wave and at workgroup granularity.  All must give the oracle's walks."""
+def test_node2vec_on_lists_of_every_length(gpu):
+    """node2vec proposes by weight and accepts with one search in N(prev): hubs of 30,000 / 20,000 / 5,000 / 600 / 70
+    neighbours as cur and as prev, p < 1 < q and p > 1 > q (rejections on every kind of neighbour), wave and
+    workgroup granularity, with and without parking (rejected walkers wait on their vertex for another round)."""
     csr = _graphs.hub_graph(V=40000, hub_degrees=(30000, 20000, 5000, 600, 70), base_degree=4, seed=23)
     starts = np.random.RandomState(6).randint(0, 40000, size=4000).astype(np.int32)
-    starts[:300] = 0    # 30000-degree hub: its neighbours see it as prev (a stretch of many windows, or in place)
+    starts[:300] = 0
     starts[300:500] = 1
     starts[500:600] = 2
     for thr in (64, 4096, 1 << 30):
         _check(gpu, csr, starts, app=gpu.APP_NODE2VEC, max_depth=9, p=0.5, q=2.0, hub_threshold=thr, seed=31)
     _check(gpu, csr, starts, app=gpu.APP_NODE2VEC, max_depth=9, p=4.0, q=0.25, hub_threshold=1000, wg_threads=256, seed=32)
+    for park, thr in ((3, 1000), (500, 64), (2000, 100000)):
+        _, st = _check(gpu, csr, starts, app=gpu.APP_NODE2VEC, max_depth=13, p=0.25, q=4.0, hub_threshold=thr,
+                       park_threshold=park, seed=33)
+        assert st.launches >= 3 and st.hub_steps > 0
+    # 15,000 walkers on one hub: crowded buckets (rows made once per round), rejected walkers stay in them
+    many = np.zeros(15000, dtype=np.int32)
+    _, st = _check(gpu, csr, many, app=gpu.APP_NODE2VEC, max_depth=6, p=0.5, q=3.0, hub_threshold=4096, park_threshold=100,
+                   seed=34)
+    assert st.hub_steps > 0
 
 
 def test_metapath(gpu, hub):
@@ -314,8 +323,8 @@ def test_randomized_configurations(gpu):
                     starts = rng.randint(0, min(V, 8), size=n)
                 kw = dict(app=app, max_depth=depth, wg_threads=int(rng.choice([256, 512, 1024])),
                           hub_threshold=int(rng.choice([0, 64, 500, 1024, 16384, 1 << 30])),
-                          park_threshold=int(rng.choice([-1, 0])) if app == gpu.APP_NODE2VEC
-                          else int(rng.choice([-1, 0, 1, 4, 16, 64, 200, 3000])), seed=int(rng.randint(0, 1 << 31)))
+                          park_threshold=int(rng.choice([-1, 0, 1, 4, 16, 64, 200, 3000])),
+                          seed=int(rng.randint(0, 1 << 31)))
                 if app == gpu.APP_NODE2VEC:
                     kw["p"], kw["q"] = float(rng.choice([0.25, 1.0, 2.0])), float(rng.choice([0.5, 1.0, 4.0]))
                 if app == gpu.APP_PPR:

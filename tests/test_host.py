@@ -41,15 +41,12 @@ def test_default_params_follow_the_reference_flags(fw):
 
 
 def test_default_params_per_application(fw):
-    """Per-application defaults differ from the plain ones only where the library chooses differently: node2vec
-    samples every list at wave granularity."""
+    """Per-application defaults are the plain ones with the application set: no application needs other choices."""
     base = fw.default_params()
-    for app in (fw.APP_DEEPWALK, fw.APP_PPR, fw.APP_METAPATH):
+    for app in (fw.APP_DEEPWALK, fw.APP_PPR, fw.APP_NODE2VEC, fw.APP_METAPATH):
         p = fw.default_params(app=app)
         assert p.app == app and p.hub_threshold == base.hub_threshold
-    p = fw.default_params(app=fw.APP_NODE2VEC)
-    assert p.app == fw.APP_NODE2VEC and p.hub_threshold == 2 ** 31 - 1
-    assert (p.max_depth, p.wg_threads, p.seed) == (base.max_depth, base.wg_threads, base.seed)
+        assert (p.max_depth, p.wg_threads, p.seed) == (base.max_depth, base.wg_threads, base.seed)
     assert fw.default_params(app=fw.APP_NODE2VEC, hub_threshold=4096).hub_threshold == 4096
 
 
