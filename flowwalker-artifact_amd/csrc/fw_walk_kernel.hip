@@ -67,30 +67,105 @@ struct StepCtx {
 // followed by another with draws of its own (streams offset by trial << 8).  The accepted neighbour has the
 // reference's law, w_i f_i / sum_j w_j f_j.
 
-// is `target` in the ascending arr[0, size)?  *probes += loads made
-__device__ __forceinline__ bool sorted_contains(const int32_t* __restrict__ arr, int32_t size, int32_t target,
-                                                uint32_t& probes) {
+// is `target` in the ascending arr[0, size)?  (one lane on its own: the hub batch kernel, where every lane serves
+// another walker)
+__device__ __forceinline__ bool sorted_contains(const int32_t* __restrict__ arr, int32_t size, int32_t target) {
   int32_t l = 0, r = size - 1;
   while (l <= r) {
     const int32_t m = l + ((r - l) >> 1);
     const int32_t x = arr[m];
-    ++probes;
     if (x == target) return true;
     if (x < target) l = m + 1; else r = m - 1;
   }
   return false;
 }
 
-// Acceptance of the proposal `post` of trial `trial` at (walker, step); by one lane.
-__device__ __forceinline__ bool n2v_accept(const fw_kargs& a, int32_t post, int32_t prev, uint32_t prev_off,
-                                           int32_t prev_deg, uint32_t walker, uint32_t step, uint32_t trial,
-                                           uint32_t& probes) {
-  if (prev == -1 || trial == kMaxTrials - 1u) return true;
-  float f;
-  if (post == prev) f = a.inv_p;
-  else f = sorted_contains(a.adjncy + prev_off, prev_deg, post, probes) ? 1.0f : a.inv_q;
+// The same question answered by a whole wave for one (wave-uniform) list and target: 64 probes per round instead
+// of one, so a list of 100,000 entries takes three dependent loads instead of seventeen.  Lane l probes the last
+// entry of the l-th of 64 chunks; the entries ascend, so the lanes whose probe is smaller than the target form a
+// prefix and the first entry that is not smaller lies in the chunk after it.
+__device__ __forceinline__ bool wave_contains(const int32_t* __restrict__ arr, uint32_t size, int32_t target, int lane) {
+  uint32_t lo = 0u, hi = size;
+  while (hi - lo > 64u) {  // wave-uniform
+    const uint32_t chunk = (hi - lo + 63u) >> 6;
+    uint32_t idx = lo + ((uint32_t)lane + 1u) * chunk - 1u;
+    idx = idx < hi ? idx : hi - 1u;
+    const uint32_t cnt = (uint32_t)__builtin_popcountll(__ballot(arr[idx] < target));
+    if (cnt == 64u) return false;  // every entry is smaller
+    lo += cnt * chunk;
+    hi = lo + chunk < hi ? lo + chunk : hi;
+  }
+  const uint32_t i = lo + (uint32_t)lane;
+  return __ballot(i < hi && arr[i] == target) != 0ull;
+}
+
+// And by the kSeg lanes of a segment of a wave, every segment for a list and a target of its own (size 0: nothing
+// to look for): kSeg probes per round.  All lanes of the wave call it together.
+template <int kSeg>
+__device__ __forceinline__ bool segment_contains(const int32_t* __restrict__ arr, uint32_t size, int32_t target,
+                                                 int lane) {
+  constexpr uint32_t kS = (uint32_t)kSeg;
+  constexpr uint32_t kShift = kSeg == 32 ? 5u : 4u;
+  const uint32_t c = (uint32_t)lane & (kS - 1u);
+  const int seg_first = lane & ~(kSeg - 1);
+  const uint32_t seg_mask = kSeg == 32 ? 0xFFFFFFFFu : 0xFFFFu;
+  uint32_t lo = 0u, hi = size;
+  for (;;) {
+    const bool big = hi - lo > kS;  // uniform in the segment
+    if (__ballot(big) == 0ull) break;
+    const uint32_t chunk = (hi - lo + kS - 1u) >> kShift;
+    uint32_t idx = lo + (c + 1u) * chunk - 1u;
+    idx = idx < hi ? idx : hi - 1u;
+    const bool less = big && arr[idx] < target;
+    const uint32_t cnt = (uint32_t)__builtin_popcount((uint32_t)(__ballot(less) >> seg_first) & seg_mask);
+    if (big) {
+      if (cnt == kS) {
+        lo = hi;  // every entry is smaller
+      } else {
+        lo += cnt * chunk;
+        hi = lo + chunk < hi ? lo + chunk : hi;
+      }
+    }
+  }
+  const uint32_t i = lo + c;
+  const uint64_t m = __ballot(i < hi && arr[i] == target);
+  return ((uint32_t)(m >> seg_first) & seg_mask) != 0u;
+}
+
+// The acceptance test u * F < f of trial `trial` at (walker, step) in two halves, so that the search for the proposal
+// in N(prev) is only made when its answer matters: f is 1/p for the return edge, else 1 (common neighbour) or 1/q, so a
+// threshold u * F below both is accepted and one that reaches both is rejected whichever it is.
+struct N2vTest {
+  float uF;          // u * F
+  bool decided;      // no search needed
+  bool accept;       // the decision when decided
+};
+
+__device__ __forceinline__ N2vTest n2v_test(const fw_kargs& a, int32_t post, int32_t prev, uint32_t walker, uint32_t step,
+                                            uint32_t trial) {
+  N2vTest t;
+  t.uF = 0.0f;
+  t.decided = true;
+  t.accept = true;
+  if (prev == -1 || trial == kMaxTrials - 1u) return t;
   const uint32_t bits = philox4x32_10(walker, step, kStreamAccept | (trial << 8), 0u, a.seed_lo, a.seed_hi).x;
-  return u24(bits) * a.n2v_fmax < f;
+  t.uF = u24(bits) * a.n2v_fmax;
+  if (post == prev) {
+    t.accept = t.uF < a.inv_p;
+    return t;
+  }
+  const float f_lo = a.inv_q < 1.0f ? a.inv_q : 1.0f;
+  const float f_hi = a.inv_q < 1.0f ? 1.0f : a.inv_q;
+  if (t.uF < f_lo) return t;            // accepted as a common neighbour and as any other
+  t.accept = false;
+  if (!(t.uF < f_hi)) return t;         // rejected as either
+  t.decided = false;
+  return t;
+}
+
+// the other half: `common` = the proposal is a neighbour of prev
+__device__ __forceinline__ bool n2v_finish(const fw_kargs& a, const N2vTest& t, bool common) {
+  return t.decided ? t.accept : t.uF < (common ? 1.0f : a.inv_q);
 }
 
 // Wave-uniform queue of Philox words: draw n of a stream is word n & 3 of block n >> 2.
@@ -305,19 +380,31 @@ __device__ __forceinline__ StepCtx load_ctx(const fw_kargs& a, const TaskTable<k
   return c;
 }
 
+// node2vec, all lanes of the wave: is the (wave-uniform) proposal v of the step accepted?  The lanes look it up in
+// N(prev) together when the answer matters.
+template <int kApp>
+__device__ __forceinline__ bool n2v_wave_accept(const fw_kargs& a, const StepCtx& c, int32_t v, bool ok, int lane) {
+  if (kApp != FW_APP_NODE2VEC || !ok) return true;
+  const N2vTest t = n2v_test(a, v, c.prev, c.walker, c.step, c.sbase >> 8);  // wave-uniform
+  bool common = false;
+  if (!t.decided) common = wave_contains(a.adjncy + c.prev_off, (uint32_t)c.prev_deg, v, lane);
+  return n2v_finish(a, t, common);
+}
+
 // Step commit by one lane: include/walker.cuh:1372-1385 and Task::update (include/gpu_task.cuh:70-77).
-// The CSR range of the new vertex is reloaded in phase C by the slot's own thread.
+// The CSR range of the new vertex is reloaded in phase C by the slot's own thread.  node2vec: the wave has made
+// the acceptance test of the proposal before (n2v_wave_accept).
 template <int kWGT, int kApp>
 __device__ __forceinline__ void commit(const fw_kargs& a, TaskTable<kWGT, kApp>& tt, int slot, const StepCtx& c, int32_t v,
-                                       bool ok, unsigned long long& n_steps, unsigned long long& n_edges) {
+                                       bool ok, bool accepted, unsigned long long& n_steps,
+                                       unsigned long long& n_edges) {
   if (!ok) {
     tt.flag[slot] = kFlagDead;
     return;
   }
-  if (kApp == FW_APP_NODE2VEC) {  // v is a proposal: accept it or sample again next round
-    uint32_t probes = 0u;
+  if (kApp == FW_APP_NODE2VEC) {  // v is a proposal: accepted, or the slot samples again next round
     const uint32_t trial = c.sbase >> 8;
-    if (!n2v_accept(a, v, c.prev, c.prev_off, c.prev_deg, c.walker, c.step, trial, probes)) {
+    if (!accepted) {
       tt.trial[slot] = (int32_t)trial + 1;
       tt.flag[slot] = kFlagRetry;
       return;
@@ -447,13 +534,28 @@ __device__ __forceinline__ void packed_finish(const fw_kargs& a, TaskTable<kWGT,
   v = pick == 2 ? adj.z : v;
   v = pick == 3 ? adj.w : v;
   const int32_t selv = __builtin_amdgcn_ds_bpermute((seg_first + l) << 2, v);
+  bool n2v_ok = true;
+  if (kApp == FW_APP_NODE2VEC) {  // selv is a proposal: the acceptance test, its search made by the segment's lanes together
+    N2vTest t;
+    t.uF = 0.0f; t.decided = true; t.accept = true;
+    uint32_t psize = 0u;
+    const int32_t* plist = a.adjncy;
+    if (active && accept) {
+      t = n2v_test(a, selv, tt.prev[slot], a.walker_base + (uint32_t)tt.walker[slot], (uint32_t)(len - 1),
+                   (uint32_t)tt.trial[slot]);  // the same in every lane of the segment
+      if (!t.decided) {
+        plist = a.adjncy + tt.prev_off[slot];
+        psize = (uint32_t)tt.prev_deg[slot];
+      }
+    }
+    const bool common = segment_contains<kSeg>(plist, psize, selv, lane);
+    n2v_ok = n2v_finish(a, t, common);
+  }
   if (active && c == 0) {  // commit (include/walker.cuh:1372-1385, Task::update include/gpu_task.cuh:70-77)
     bool rejected = false;
-    if (kApp == FW_APP_NODE2VEC && accept) {  // selv is a proposal: accept it or sample again next round
-      uint32_t probes = 0u;
+    if (kApp == FW_APP_NODE2VEC && accept) {  // accept the proposal or sample again next round
       const uint32_t trial = (uint32_t)tt.trial[slot];
-      rejected = !n2v_accept(a, selv, tt.prev[slot], tt.prev_off[slot], tt.prev_deg[slot],
-                             a.walker_base + (uint32_t)tt.walker[slot], (uint32_t)(len - 1), trial, probes);
+      rejected = !n2v_ok;
       tt.trial[slot] = rejected ? (int32_t)trial + 1 : 0;
     }
     if (!accept) {
@@ -582,11 +684,10 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
             m = __ballot(pos);
             if (m != 0ull) pick = __builtin_amdgcn_readlane(s, 63 - __builtin_clzll(m));
           }
-          if (lane == 0) {
-            int32_t v = -1;
-            if (pick >= 0) v = a.adjncy[c.off + (uint32_t)pick];
-            commit(a, tt, slot, c, v, pick >= 0, n_steps, n_edges);
-          }
+          int32_t v = -1;
+          if (pick >= 0) v = a.adjncy[c.off + (uint32_t)pick];  // wave-uniform
+          const bool accepted = n2v_wave_accept<kApp>(a, c, v, pick >= 0, lane);
+          if (lane == 0) commit(a, tt, slot, c, v, pick >= 0, accepted, n_steps, n_edges);
         }
         if (hb + kHubChunk < nh) __syncthreads();  // the partial buffers are reused by the next chunk
       }
@@ -652,7 +753,8 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
           wave_stream<kApp, kGroupQuartets, false>(a, c, lane, 0u, 1u, dq0, W, sel, selv);
           if (sel >= 0) v = a.adjncy[c.off + (uint32_t)sel];
         }
-        if (lane == 0) commit(a, tt, slot, c, v, sel >= 0, n_steps, n_edges);
+        const bool accepted = n2v_wave_accept<kApp>(a, c, v, sel >= 0, lane);
+        if (lane == 0) commit(a, tt, slot, c, v, sel >= 0, accepted, n_steps, n_edges);
       }
       __syncthreads();
       if (tid == 0) {  // this round's lists are drained; they become the lists produced two rounds later
@@ -1240,10 +1342,13 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
   if (moved) {
     nv = a.adjncy[off + (uint32_t)pick];
     if (kApp == FW_APP_NODE2VEC && rec.prev >= 0) {
-      uint32_t probes = 0u;
-      const uint32_t po = a.xadj[rec.prev];
-      const int32_t pd = (int32_t)(a.xadj[rec.prev + 1] - po);
-      if (!n2v_accept(a, nv, rec.prev, po, pd, walker, step, trial, probes)) {
+      const N2vTest t = n2v_test(a, nv, rec.prev, walker, step, trial);
+      bool common = false;
+      if (!t.decided) {
+        const uint32_t po = a.xadj[rec.prev];
+        common = sorted_contains(a.adjncy + po, (int32_t)(a.xadj[rec.prev + 1] - po), nv);
+      }
+      if (!n2v_finish(a, t, common)) {
         moved = false;
         retry = true;
       }
