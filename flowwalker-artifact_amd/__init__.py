@@ -30,7 +30,11 @@ EXPORTED = [
     "fw_graph_download", "fw_walk_device", "fw_walk_batch", "fw_host_alloc_pinned", "fw_host_free_pinned",
     "fw_gen_rmat", "fw_csr_read_header", "fw_csr_load", "fw_csr_write", "fw_graph_load",
     "fw_graph_create_placed", "fw_graph_load_placed", "fw_walk_device_noalloc", "fw_csr_sort_neighbours",
+    "fw_sampler_baseline_run",
 ]
+
+
+BASELINE_ITS, BASELINE_RJS = 0, 1
 
 
 class WalkParams(C.Structure):
@@ -115,6 +119,8 @@ def lib():
         L.fw_csr_sort_neighbours.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                              C.POINTER(C.c_int64)]
         L.fw_graph_load.argtypes = [C.c_char_p, C.c_int, C.c_int, C.POINTER(C.c_void_p)]
+        L.fw_sampler_baseline_run.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_uint64, C.c_uint32, C.c_void_p, C.c_uint32,
+                                              C.c_int, C.c_uint64, C.c_void_p, C.POINTER(C.c_double)]
         L.fw_graph_load_placed.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p)]
         _lib = L
     return _lib
@@ -329,3 +335,25 @@ class Graph:
             self.destroy()
         except Exception:
             pass
+
+
+def sampler_baseline(kind, weights, list_len, tasks=None, workgroup=False, wg_threads=512, seed=1):
+    """fw_sampler_baseline_run on host arrays: one index per task from its list_len-element slice of `weights`
+    by inverse transform (BASELINE_ITS) or rejection sampling (BASELINE_RJS).  Returns (indices, kernel_ms)."""
+    weights = np.ascontiguousarray(weights, dtype=np.float32)
+    n = len(tasks) if tasks is not None else len(weights) // int(list_len)
+    d_w = DeviceBuffer.from_numpy(weights)
+    d_t = DeviceBuffer.from_numpy(np.ascontiguousarray(tasks, dtype=np.uint32)) if tasks is not None else None
+    d_o = DeviceBuffer(max(n, 1) * 4)
+    ms = C.c_double(0.0)
+    try:
+        check(lib().fw_sampler_baseline_run(int(kind), int(bool(workgroup)), d_w.ptr, len(weights), int(list_len),
+                                            d_t.ptr if d_t is not None else None, n, int(wg_threads), int(seed),
+                                            d_o.ptr, C.byref(ms)))
+        out = d_o.to_numpy(np.int32, (n,))
+    finally:
+        d_w.free()
+        d_o.free()
+        if d_t is not None:
+            d_t.free()
+    return out, ms.value

@@ -28,7 +28,7 @@ HIP_FLAGS = [
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
 ]
 
-KERNEL_SOURCES = ["fw_walk_kernel.hip", "fw_ref_walk.hip", "fw_api.hip", "fw_gen.hip", "fw_csr_io.hip"]
+KERNEL_SOURCES = ["fw_walk_kernel.hip", "fw_ref_walk.hip", "fw_sampler_baselines.hip", "fw_api.hip", "fw_gen.hip", "fw_csr_io.hip"]
 HOST_TOOLS = {"flowwalker": ["flowwalker_main.cpp"], "fw_gen": ["fw_gen_main.cpp"], "fw_convert": ["fw_convert_main.cpp"],
               "fw_sampler_bench": ["fw_sampler_bench_main.cpp"]}
 

@@ -11,10 +11,11 @@
 // --type picks the algorithm, as TestSampler's --type does (src/sampler_test.cu:789-895): `native` = this engine's
 // one-pass group reservoir; `zprs` / `dprs` = the reference's own samplers restated for 64-lane waves
 // (include/sampler.cuh:46-127 and :129-200, FW_SAMPLER_REF_ZPRS / _DPRS: TestSampler types 1 / 2 and 3 / 4), run
-// on the same lists so that the columns can be compared.
+// on the same lists so that the columns can be compared; `its` / `rjs` = inverse transform and rejection sampling on
+// the same slices of the weight array (TestSampler types 5 / 6 and its RJS kernels, fw_sampler_baseline_run).
 //
 //   fw_sampler_bench [--elements 268435456] [--gran 16,64,256,1024,4096,16384,65536] [--samples 4194304]
-//                    [--granularity wave|workgroup|both] [--type native,zprs,dprs] [--wg_threads 512] [--reps 3]
+//                    [--granularity wave|workgroup|both] [--type native,zprs,dprs,its,rjs] [--wg_threads 512] [--reps 3]
 //                    [--seed 1]
 // Output: one line per (gran, type, granularity): samples/s and GB/s of weights (4 bytes per element and sample;
 // the two-pass ZPRS reads them twice, which is not counted).
@@ -87,8 +88,16 @@ int main(int argc, char** argv) {
     if (t == "native") run_types.push_back({"native", FW_SAMPLER_ZPRS});
     else if (t == "zprs") run_types.push_back({"zprs", FW_SAMPLER_REF_ZPRS});
     else if (t == "dprs") run_types.push_back({"dprs", FW_SAMPLER_REF_DPRS});
-    else { fprintf(stderr, "fw_sampler_bench: --type takes native, zprs, dprs (got %s)\n", t.c_str()); return 2; }
+    else if (t == "its") run_types.push_back({"its", -1 - FW_BASELINE_ITS});
+    else if (t == "rjs") run_types.push_back({"rjs", -1 - FW_BASELINE_RJS});
+    else { fprintf(stderr, "fw_sampler_bench: --type takes native, zprs, dprs, its, rjs (got %s)\n", t.c_str()); return 2; }
   }
+  void* d_w = nullptr;  // the baselines read the weight array itself, not a graph
+  for (const Type& type : run_types)
+    if (type.sampler < 0 && !d_w) {
+      if (fw_dev_alloc((size_t)elements * 4, &d_w) != FW_OK || fw_dev_upload(d_w, w.data(), (size_t)elements * 4) != FW_OK)
+        return fail("uploading the weight array");
+    }
   printf("%-10s %-8s %-10s %12s %14s %12s %10s\n", "gran", "type", "sampler", "samples", "samples/s", "GB/s", "ms");
   size_t pos = 0;
   while (pos < grans.size()) {
@@ -118,6 +127,20 @@ int main(int argc, char** argv) {
       for (int mode = 0; mode < 2; ++mode) {
         const char* name = mode == 0 ? "wave" : "workgroup";
         if (granularity != "both" && granularity != name) continue;
+        if (type.sampler < 0) {
+          double best = 0.0, ms = 0.0;
+          for (int r = 0; r <= reps; ++r) {
+            if (fw_sampler_baseline_run(-1 - type.sampler, mode, (const float*)d_w, elements, (uint32_t)gran,
+                                        (const uint32_t*)d_starts, (uint32_t)samples, wg_threads, seed, (int32_t*)d_paths,
+                                        &ms) != FW_OK)
+              return fail("sampling");
+            if (r > 0 && (best == 0.0 || ms < best)) best = ms;
+          }
+          printf("%-10lld %-8s %-10s %12lld %14.4g %12.1f %10.3f\n", gran, type.name, name, samples,
+                 (double)samples / (best * 1e-3), 4.0 * (double)samples * (double)gran / (best * 1e-3) / 1e9, best);
+          fflush(stdout);
+          continue;
+        }
         fw_walk_params p;
         fw_walk_params_default(&p);
         p.app = FW_APP_DEEPWALK;
@@ -143,5 +166,6 @@ int main(int argc, char** argv) {
     fw_dev_free(d_paths);
     fw_graph_destroy(g);
   }
+  if (d_w) fw_dev_free(d_w);
   return 0;
 }
