@@ -588,6 +588,7 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
   // they are dealt out by a scan over the waves' totals
   constexpr int kKinds = 4;  // workgroup, wave, table, scan
   __shared__ uint32_t s_tot[kKinds][16];
+  __shared__ unsigned long long s_q[16];
   __shared__ uint32_t s_base[kKinds];
   __shared__ uint32_t s_cmax;
   if (threadIdx.x == 0) s_cmax = 0u;
@@ -596,6 +597,8 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
   const int lane = (int)(threadIdx.x & 63u);
   const int wave = (int)(threadIdx.x >> 6);
   const int rounds = (n_buckets + stride - 1) / stride;  // every thread runs every round: scans and barriers
+  unsigned long long my_quartets = 0ull;  // traffic figures of the round: summed per thread, one update per workgroup
+  uint32_t my_table_walkers = 0u;
 
   for (int r = 0; r < rounds; ++r) {
     const int b = r * stride + (int)(blockIdx.x * blockDim.x + threadIdx.x);
@@ -629,17 +632,8 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
     {
       // what the round's hub launches will stream: a list once per batch task, or once by the scan tasks
       const unsigned long long nq = c != 0u ? (((t.off & 3u) + t.deg + 3u) >> 2) : 0u;
-      unsigned long long quartets = two_pass ? nq : nq * nb;
-      uint32_t table_walkers = two_pass ? c : 0u;
-#pragma unroll
-      for (int d = 32; d >= 1; d >>= 1) {
-        quartets += __shfl_xor(quartets, d);
-        table_walkers += __shfl_xor(table_walkers, d);
-      }
-      if (lane == 0 && quartets != 0ull) {
-        atomicAdd(reinterpret_cast<unsigned long long*>(ctrs + 14), quartets);
-        if (table_walkers != 0u) atomicAdd(&ctrs[13], table_walkers);
-      }
+      my_quartets += two_pass ? nq : nq * nb;
+      my_table_walkers += two_pass ? c : 0u;
     }
     uint32_t x[kKinds];
     x[0] = !two_pass && wg ? nb : 0u;
@@ -714,6 +708,26 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
       }
     }
     __syncthreads();  // s_tot / s_base are reused by the next round
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    my_quartets += __shfl_xor(my_quartets, d);
+    my_table_walkers += __shfl_xor(my_table_walkers, d);
+  }
+  if (lane == 0) {
+    s_q[wave] = my_quartets;
+    s_tot[2][wave] = my_table_walkers;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long q = 0ull;
+    uint32_t tw = 0u;
+    for (int w = 0; w < (int)(blockDim.x >> 6); ++w) {
+      q += s_q[w];
+      tw += s_tot[2][w];
+    }
+    if (q != 0ull) atomicAdd(reinterpret_cast<unsigned long long*>(ctrs + 14), q);
+    if (tw != 0u) atomicAdd(&ctrs[13], tw);
   }
 }
 
@@ -818,11 +832,17 @@ __global__ __launch_bounds__(1024) void fw_compact_resume_kernel(const fw_walker
 }
 
 // Parked records name their bucket; the walk kernel wants the vertex (used when the last few walkers leave the
-// park / batch loop).
+// park / batch loop).  The batch kernel may have left the path entry of a walker it parked again to the walker's next
+// step there (entries are stored in pairs); these walkers take that step in the walk kernel, so the entry is stored here.
 __global__ void fw_bucket_to_vertex_kernel(fw_walker_rec* recs, uint32_t m, const fw_hub_info* __restrict__ hub_info,
-                                           int labels) {
+                                           int labels, int32_t* __restrict__ paths, int32_t max_depth, int n2v) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < m) recs[i].cur = hub_info[(uint32_t)recs[i].cur / (uint32_t)labels].v;
+  if (i >= m) return;
+  const fw_walker_rec r = recs[i];
+  const int32_t v = hub_info[(uint32_t)r.cur / (uint32_t)labels].v;
+  recs[i].cur = v;
+  const int32_t len = n2v != 0 ? (r.len & FW_REC_LEN_MASK) : r.len;
+  if (r.q >= 0 && len >= 1) paths[(uint64_t)(uint32_t)r.q * (uint64_t)max_depth + (uint64_t)(len - 1)] = v;
 }
 
 // Device buffers of one park / batch / resume loop (one per stream in flight).  Three record lists: `walked`
@@ -1123,7 +1143,8 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
       // default rule only (an explicit threshold keeps every round in the loop): too few walkers are left to
       // meet anywhere, so they finish in one walk launch that does not park
       hipLaunchKernelGGL(fw_bucket_to_vertex_kernel, dim3(((unsigned)m + 255u) / 256u), dim3(256), 0, stream,
-                         pb->sorted, (uint32_t)m, g->hub_info, labels);
+                         pb->sorted, (uint32_t)m, g->hub_info, labels, a.paths, a.max_depth,
+                         p->app == FW_APP_NODE2VEC ? 1 : 0);
       FW_HIP(hipGetLastError());
       a.resume = pb->sorted;
       a.n_dev = nullptr;

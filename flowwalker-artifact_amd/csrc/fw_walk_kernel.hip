@@ -1355,7 +1355,6 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
     }
   }
   if (moved) {
-    a.paths[(uint64_t)(uint32_t)rec.q * (uint64_t)a.max_depth + (uint64_t)rec.len] = nv;
     go_on = rec.len + 1 < a.max_depth;
     if (kApp == FW_APP_PPR && go_on) {
       const uint32_t bits = philox4x32_10(walker, step, kStreamStop, 0u, a.seed_lo, a.seed_hi).x;
@@ -1381,6 +1380,22 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
     hidx = a.hub_index[v];
     go_on = true;
     park = true;
+  }
+  if (have && !retry) {
+    // Path entries are written in aligned pairs where that is possible: a scattered 4-byte store costs the memory
+    // system a read-modify-write of its line, and a pair costs the same.  The walker stands on v = entry len - 1 and
+    // moves to nv = entry len.  When entry len is the upper half of an aligned pair, both are stored together.  When
+    // it is the lower half and the walker is parked again, nothing is stored: its next step is taken here too and
+    // stores the pair (the last few walkers that leave the parking loop instead have their latest entry written by
+    // fw_bucket_to_vertex_kernel).  A walk that ends here without a step stores a lower-half v that may be pending.
+    int32_t* const at = a.paths + ((uint64_t)(uint32_t)rec.q * (uint64_t)a.max_depth + (uint64_t)rec.len);
+    const bool upper = (reinterpret_cast<uintptr_t>(at) & 4u) != 0u;
+    if (moved) {
+      if (upper) *reinterpret_cast<int2*>(at - 1) = make_int2(v, nv);
+      else if (!(go_on && park)) *at = nv;
+    } else if (upper) {
+      at[-1] = v;
+    }
   }
   const uint32_t label_slot = kApp == FW_APP_METAPATH ? (uint32_t)rec.len % (uint32_t)a.n_labels_per_hub : 0u;
   const uint32_t bucket = (uint32_t)hidx * (uint32_t)a.n_labels_per_hub + label_slot;
