@@ -583,7 +583,7 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
                                        const uint32_t* __restrict__ bucket_offset, int n_buckets, int labels,
                                        const fw_hub_info* __restrict__ hub_info, const TaskPlan plan,
                                        fw_batch_task* tasks, fw_batch_task* wtasks, fw_batch_task* ttasks,
-                                       fw_batch_task* stasks, uint32_t* ctrs) {
+                                       fw_batch_task* stasks, uint32_t* rows_made, uint32_t* ctrs) {
   // slots and rows: one update of the (contended) global counters per workgroup and kind; inside the workgroup
   // they are dealt out by a scan over the waves' totals
   constexpr int kKinds = 4;  // workgroup, wave, table, scan
@@ -627,19 +627,23 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
     }
     const bool two_pass = c > plan.two_pass_walkers && hub_row != FW_NO_ROWS;
     if (two_pass) t.row = hub_row * (uint32_t)labels + (uint32_t)t.slot * ngroups;
+    // the rows of a list do not depend on the walkers: they are made in the first round that wants them and serve
+    // every later round of the call
+    const bool scan = two_pass && rows_made[b] == 0u;
+    if (scan) rows_made[b] = 1u;
     const bool wg = (int32_t)t.deg > plan.hub_threshold;
     const uint32_t nb = (c + 63u) >> 6;
     {
       // what the round's hub launches will stream: a list once per batch task, or once by the scan tasks
       const unsigned long long nq = c != 0u ? (((t.off & 3u) + t.deg + 3u) >> 2) : 0u;
-      my_quartets += two_pass ? nq : nq * nb;
+      my_quartets += two_pass ? (scan ? nq : 0ull) : nq * nb;
       my_table_walkers += two_pass ? c : 0u;
     }
     uint32_t x[kKinds];
     x[0] = !two_pass && wg ? nb : 0u;
     x[1] = !two_pass && !wg ? nb : 0u;
     x[2] = two_pass ? nb : 0u;
-    x[3] = two_pass ? (ngroups + kScanRun - 1u) / kScanRun : 0u;
+    x[3] = scan ? (ngroups + kScanRun - 1u) / kScanRun : 0u;
     uint32_t inc[kKinds];
 #pragma unroll
     for (int k = 0; k < kKinds; ++k) inc[k] = x[k];
@@ -698,7 +702,7 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
         t.count = (int32_t)(c - 64u * k < 64u ? c - 64u * k : 64u);
         out[t0 + k] = t;
       }
-      if (two_pass) {
+      if (scan) {
         const uint32_t s0 = s_base[3] + s_tot[3][wave] + inc[3] - x[3];
         for (uint32_t k = 0; k < x[3]; ++k) {
           t.rec_base = k * kScanRun;
@@ -856,7 +860,8 @@ struct ParkBuffers {
   fw_walker_rec* sorted = nullptr;
   fw_walker_rec* out = nullptr;
   fw_walker_rec* resume = nullptr;    // the records of `out` that continue in the walk kernel, dense
-  uint32_t* buckets = nullptr;        // [4 * n_buckets]: count of round parity 0, of parity 1, offset, fill
+  uint32_t* buckets = nullptr;        // [5 * n_buckets]: count of round parity 0, of parity 1, offset, fill, and
+                                      // whether the bucket's rows have been made in this call
   fw_batch_task* tasks = nullptr;
   fw_batch_task* wtasks = nullptr;
   uint32_t* ctrs = nullptr;           // [0] walkers in `walked`, [1] records of `out` that resume, [2] that are parked
@@ -876,6 +881,7 @@ struct ParkBuffers {
   uint32_t* count(int parity) const { return buckets + (size_t)parity * n_buckets; }
   uint32_t* offset() const { return buckets + (size_t)2 * n_buckets; }
   uint32_t* fill() const { return buckets + (size_t)3 * n_buckets; }
+  uint32_t* rows_made() const { return buckets + (size_t)4 * n_buckets; }
 
   int alloc(size_t walkers, int n, uint64_t rows_wanted) {
     cap = walkers;
@@ -885,7 +891,7 @@ struct ParkBuffers {
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&sorted), cap * sizeof(fw_walker_rec)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&out), cap * sizeof(fw_walker_rec)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&resume), cap * sizeof(fw_walker_rec)));
-    FW_HIP(hipMalloc(reinterpret_cast<void**>(&buckets), (size_t)4 * n * sizeof(uint32_t)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&buckets), (size_t)5 * n * sizeof(uint32_t)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&tasks), ntask * sizeof(fw_batch_task)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&wtasks), ntask * sizeof(fw_batch_task)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), kParkCtrs * sizeof(uint32_t)));
@@ -1088,6 +1094,11 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   if (rblocks > 2048u) rblocks = 2048u;
   if (rblocks == 0u) rblocks = 1u;
 
+  if (two_pass_possible) {  // no bucket has rows yet
+    hipLaunchKernelGGL(fw_fill_i32_kernel, dim3(rblocks), dim3(256), 0, stream, reinterpret_cast<int32_t*>(pb->rows_made()),
+                       0, (size_t)pb->n_buckets);
+    FW_HIP(hipGetLastError());
+  }
   // first walk launch: fresh queries; the walkers it parks are counted in bucket array 0
   int cur = 0;
   hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs, pb->count(0),
@@ -1164,7 +1175,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     if (tblocks > 1024u) tblocks = 1024u;
     hipLaunchKernelGGL(fw_bucket_tasks_kernel, dim3(tblocks), dim3(1024), 0, stream, pb->count(cur), pb->offset(),
                        pb->n_buckets, labels, g->hub_info, plan, pb->tasks, pb->wtasks, pb->ttasks, pb->stasks,
-                       pb->ctrs);
+                       pb->rows_made(), pb->ctrs);
     FW_HIP(hipGetLastError());
     h.bucket_out = pb->count(nxt);
     TimedLaunch th;
