@@ -482,7 +482,7 @@ static void fill_kargs(fw_kargs* a, const fw_graph* g, const fw_walk_params* p) 
 // Every such list has rows of its own (520 bytes per 1024 elements and label a walker can want), set aside when
 // the lists are numbered, so that nothing has to be handed out while the walks run; kMaxHubRows bounds them
 // (lists past it are served by batches, however crowded).
-constexpr uint32_t kTwoPassWalkers = 256;
+constexpr uint32_t kTwoPassWalkers = 128;
 constexpr uint32_t kTwoPassDegree = 2048;
 constexpr uint32_t kMaxHubRows = 1u << 21;             // per label: 1 GiB of rows
 constexpr uint64_t kMaxRows = (4ull << 30) / 520u;     // all labels together: 4 GiB
