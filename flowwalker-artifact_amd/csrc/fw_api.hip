@@ -569,7 +569,8 @@ constexpr int kParkCtrs = 16;                    // counters of a parking round
 // is served in two passes (scan tasks of up to kScanRun groups that make the list's rows, one table task per 64
 // walkers); every other bucket gets one batch task per 64 walkers:
 // a workgroup task when its vertex is sampled at workgroup granularity (degree above hub_threshold), a wave task
-// otherwise.  ctrs (out): [3] workgroup tasks, [4] their dispenser, [5] wave tasks, [7] table tasks, [8] scan tasks,
+// otherwise -- or, on a list of at most 64 aligned quartets, one quad task per 16 walkers (four of those share a
+// wave).  ctrs (out): [3] workgroup tasks, [4] their dispenser, [5] wave tasks, [7] table tasks, [8] scan tasks, [9] quad tasks,
 // [12] walkers in the fullest bucket when that is more than half of kTwoPassWalkers, [13] walkers served by table
 // tasks, [14..15] (one 64-bit word) 16-byte quartets the round's batch and scan tasks stream.
 constexpr uint32_t kScanRun = 16;
@@ -577,16 +578,18 @@ constexpr uint32_t kScanRun = 16;
 struct TaskPlan {
   int32_t hub_threshold;
   uint32_t two_pass_walkers;  // 0xFFFFFFFF: never
+  int32_t quad_tasks;         // lists of at most 64 aligned quartets are served four to a wave
 };
 
 __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* __restrict__ bucket_count,
                                        const uint32_t* __restrict__ bucket_offset, int n_buckets, int labels,
                                        const fw_hub_info* __restrict__ hub_info, const TaskPlan plan,
                                        fw_batch_task* tasks, fw_batch_task* wtasks, fw_batch_task* ttasks,
-                                       fw_batch_task* stasks, uint32_t* rows_made, uint32_t* ctrs) {
+                                       fw_batch_task* stasks, fw_batch_task* qtasks, uint32_t* rows_made,
+                                       uint32_t* ctrs) {
   // slots and rows: one update of the (contended) global counters per workgroup and kind; inside the workgroup
   // they are dealt out by a scan over the waves' totals
-  constexpr int kKinds = 4;  // workgroup, wave, table, scan
+  constexpr int kKinds = 5;  // workgroup, wave, table, scan, quad
   __shared__ uint32_t s_tot[kKinds][16];
   __shared__ unsigned long long s_q[16];
   __shared__ uint32_t s_base[kKinds];
@@ -632,7 +635,10 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
     const bool scan = two_pass && rows_made[b] == 0u;
     if (scan) rows_made[b] = 1u;
     const bool wg = (int32_t)t.deg > plan.hub_threshold;
-    const uint32_t nb = (c + 63u) >> 6;
+    const uint32_t nq_list = c != 0u ? (((t.off & 3u) + t.deg + 3u) >> 2) : 0u;
+    const bool quad = plan.quad_tasks != 0 && c != 0u && !two_pass && !wg && nq_list <= 64u;
+    const uint32_t per_task = quad ? 16u : 64u;
+    const uint32_t nb = (c + per_task - 1u) / per_task;
     {
       // what the round's hub launches will stream: a list once per batch task, or once by the scan tasks
       const unsigned long long nq = c != 0u ? (((t.off & 3u) + t.deg + 3u) >> 2) : 0u;
@@ -641,8 +647,9 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
     }
     uint32_t x[kKinds];
     x[0] = !two_pass && wg ? nb : 0u;
-    x[1] = !two_pass && !wg ? nb : 0u;
+    x[1] = !two_pass && !wg && !quad ? nb : 0u;
     x[2] = two_pass ? nb : 0u;
+    x[4] = quad ? nb : 0u;
     x[3] = scan ? (ngroups + kScanRun - 1u) / kScanRun : 0u;
     uint32_t inc[kKinds];
 #pragma unroll
@@ -671,13 +678,13 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
         s_tot[threadIdx.x][w] = total;
         total += v;
       }
-      const int ctr = threadIdx.x == 0 ? 3 : (threadIdx.x == 1 ? 5 : (threadIdx.x == 2 ? 7 : 8));
+      const int ctr = threadIdx.x == 0 ? 3 : (threadIdx.x == 1 ? 5 : (threadIdx.x == 2 ? 7 : (threadIdx.x == 3 ? 8 : 9)));
       s_base[threadIdx.x] = total != 0u ? atomicAdd(&ctrs[ctr], total) : 0u;
     }
     __syncthreads();
-    const int kind = two_pass ? 2 : (wg ? 0 : 1);
+    const int kind = two_pass ? 2 : (wg ? 0 : (quad ? 4 : 1));
     // (selected, not indexed: the arrays stay in registers)
-    const uint32_t mine = two_pass ? inc[2] - x[2] : (wg ? inc[0] - x[0] : inc[1] - x[1]);
+    const uint32_t mine = two_pass ? inc[2] - x[2] : (wg ? inc[0] - x[0] : (quad ? inc[4] - x[4] : inc[1] - x[1]));
     const uint32_t t0 = s_base[kind] + s_tot[kind][wave] + mine;
     const uint32_t base = c != 0u ? bucket_offset[b] : 0u;
     // a crowded bucket has thousands of tasks: those are written by the whole wave, one bucket after the other
@@ -688,18 +695,20 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
       bt.v = __shfl(t.v, l); bt.off = __shfl(t.off, l); bt.deg = __shfl(t.deg, l); bt.slot = __shfl(t.slot, l);
       bt.row = __shfl(t.row, l); bt.pad = 0;
       const uint32_t bc = __shfl(c, l), bbase = __shfl(base, l), bt0 = __shfl(t0, l), bnb = __shfl(nb, l);
-      fw_batch_task* bout = __shfl(kind, l) == 0 ? tasks : (__shfl(kind, l) == 1 ? wtasks : ttasks);
+      const int bkind = __shfl(kind, l);
+      const uint32_t bper = bkind == 4 ? 16u : 64u;
+      fw_batch_task* bout = bkind == 0 ? tasks : (bkind == 1 ? wtasks : (bkind == 2 ? ttasks : qtasks));
       for (uint32_t k = (uint32_t)lane; k < bnb; k += 64u) {
-        bt.rec_base = bbase + 64u * k;
-        bt.count = (int32_t)(bc - 64u * k < 64u ? bc - 64u * k : 64u);
+        bt.rec_base = bbase + bper * k;
+        bt.count = (int32_t)(bc - bper * k < bper ? bc - bper * k : bper);
         bout[bt0 + k] = bt;
       }
     }
     if (c != 0u) {
-      fw_batch_task* out = kind == 0 ? tasks : (kind == 1 ? wtasks : ttasks);
+      fw_batch_task* out = kind == 0 ? tasks : (kind == 1 ? wtasks : (kind == 2 ? ttasks : qtasks));
       for (uint32_t k = 0; k < (nb > kOwnTasks ? 0u : nb); ++k) {
-        t.rec_base = base + 64u * k;
-        t.count = (int32_t)(c - 64u * k < 64u ? c - 64u * k : 64u);
+        t.rec_base = base + per_task * k;
+        t.count = (int32_t)(c - per_task * k < per_task ? c - per_task * k : per_task);
         out[t0 + k] = t;
       }
       if (scan) {
@@ -864,6 +873,7 @@ struct ParkBuffers {
                                       // whether the bucket's rows have been made in this call
   fw_batch_task* tasks = nullptr;
   fw_batch_task* wtasks = nullptr;
+  fw_batch_task* qtasks = nullptr;    // quad tasks: up to 16 walkers each
   uint32_t* ctrs = nullptr;           // [0] walkers in `walked`, [1] records of `out` that resume, [2] that are parked
                                       // again, [3] workgroup tasks, [4] their dispenser, [5] wave tasks, [6] records in
                                       // `resume`, [7] table tasks, [8] scan tasks, [12] walkers in the fullest bucket
@@ -894,6 +904,7 @@ struct ParkBuffers {
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&buckets), (size_t)5 * n * sizeof(uint32_t)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&tasks), ntask * sizeof(fw_batch_task)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&wtasks), ntask * sizeof(fw_batch_task)));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&qtasks), (cap / 16 + (size_t)n + 1) * sizeof(fw_batch_task)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), kParkCtrs * sizeof(uint32_t)));
     FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), kParkCtrs * sizeof(uint32_t), hipHostMallocDefault));
     for (hipEvent_t& e : ev) FW_HIP(hipEventCreate(&e));
@@ -928,7 +939,7 @@ struct ParkBuffers {
   }
   void release() {
     release_rows();
-    void* dev[9] = {walked, sorted, out, resume, buckets, tasks, wtasks, ctrs, tmp};
+    void* dev[10] = {walked, sorted, out, resume, buckets, tasks, wtasks, qtasks, ctrs, tmp};
     for (void* p : dev) if (p) (void)hipFree(p);
     if (h_ctrs) (void)hipHostFree(h_ctrs);
     for (hipEvent_t& e : ev) {
@@ -937,7 +948,7 @@ struct ParkBuffers {
     }
     walked = sorted = out = resume = nullptr;
     buckets = ctrs = h_ctrs = nullptr;
-    tasks = wtasks = nullptr;
+    tasks = wtasks = qtasks = nullptr;
     tmp = nullptr;
   }
 };
@@ -1054,11 +1065,14 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   h.nstasks = &pb->ctrs[8];
   h.ttasks = pb->ttasks;
   h.nttasks = &pb->ctrs[7];
+  h.qtasks = pb->qtasks;
+  h.nqtasks = &pb->ctrs[9];
   h.totals = pb->totals;
   h.rows = pb->rows;
   h.lastpos = pb->lastpos;
   TaskPlan plan;
   plan.hub_threshold = p->hub_threshold;
+  plan.quad_tasks = 1;
   // Two-pass steps cost a launch per round that looks for scan tasks, so a round only gets them when the round
   // before had a bucket at least half as full as they need (the first round always does): a bucket may then miss
   // them for a round and is served by batches, with the same results.
@@ -1116,6 +1130,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   uint32_t n_out = 0;  // records in `out` (the previous batch launch's input size)
   uint32_t fullest = 0;  // walkers in the fullest bucket of the previous round
   uint32_t scan_tasks = 0;  // and its scan tasks
+  uint32_t quad_tasks = 0;  // and its quad tasks
   uint32_t resumed = 0;     // and the walkers that went on in its walk launch
   uint32_t batch_tasks = 0; // and its batch tasks, in waves
   uint32_t wg_task_waves = 0;  // of which workgroup tasks
@@ -1175,7 +1190,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     if (tblocks > 1024u) tblocks = 1024u;
     hipLaunchKernelGGL(fw_bucket_tasks_kernel, dim3(tblocks), dim3(1024), 0, stream, pb->count(cur), pb->offset(),
                        pb->n_buckets, labels, g->hub_info, plan, pb->tasks, pb->wtasks, pb->ttasks, pb->stasks,
-                       pb->rows_made(), pb->ctrs);
+                       pb->qtasks, pb->rows_made(), pb->ctrs);
     FW_HIP(hipGetLastError());
     h.bucket_out = pb->count(nxt);
     TimedLaunch th;
@@ -1193,6 +1208,9 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     uint32_t tasks_hint = n_out != 0u ? (uint32_t)((uint64_t)batch_tasks * m / n_out) + 1u : 0u;
     if ((uint64_t)wg_task_waves * 16u > batch_tasks) tasks_hint = 0u;
     rc = fw_launch_hub_batch(a, h, p->app, p->wg_threads, tasks_hint, stream);
+    if (rc != FW_OK) return rc;
+    // the short lists with few walkers, four to a wave (about as many as a round ago, scaled by the walkers)
+    rc = fw_launch_hub_quad(a, h, p->app, n_out != 0u ? (uint32_t)((uint64_t)quad_tasks * m / n_out) + 1u : 0u, stream);
     if (rc != FW_OK) return rc;
     if ((rc = th.end(stream)) != FW_OK) return rc;
     ++*launches;
@@ -1225,6 +1243,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     resumed = pb->h_ctrs[6];
     wg_task_waves = pb->h_ctrs[3] * (uint32_t)(p->wg_threads / 64);
     batch_tasks = pb->h_ctrs[5] + pb->h_ctrs[7] + wg_task_waves;
+    quad_tasks = pb->h_ctrs[9];
     scan_tasks = pb->h_ctrs[8];
     cur = nxt;
   }

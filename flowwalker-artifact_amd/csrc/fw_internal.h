@@ -133,6 +133,11 @@ struct fw_hub_args {
   const uint32_t* nstasks;
   const fw_batch_task* ttasks;
   const uint32_t* nttasks;
+  // Quad tasks: at most 16 walkers on a list of at most 64 aligned quartets (one group whose lanes hold one quartet
+  // each).  A wave serves four of them at once, one per 16-lane row: wave i of the grid takes tasks 4i .. 4i + 3,
+  // then 4 (i + waves) ..
+  const fw_batch_task* qtasks;
+  const uint32_t* nqtasks;
   float* totals;
   float* rows;
   int32_t* lastpos;
@@ -201,6 +206,7 @@ int fw_launch_ref_walk(const fw_kargs& a, int app, int sampler, int wg_threads, 
 // 0 = no idea: one resident set).
 int fw_launch_hub_batch(const fw_kargs& a, const fw_hub_args& h, int app, int wg_threads, uint32_t tasks_hint,
                         hipStream_t stream);
+int fw_launch_hub_quad(const fw_kargs& a, const fw_hub_args& h, int app, uint32_t quads_hint, hipStream_t stream);
 // Launches the scan kernel of the two-pass steps (it finds its task count in h.nstasks on the device).
 // tasks_hint: about how many scan tasks to expect, to size the grid (0 = no idea: a full resident set).
 int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, uint32_t tasks_hint, hipStream_t stream);

@@ -1328,9 +1328,11 @@ __device__ __forceinline__ int32_t table_sample(const fw_kargs& a, const uint32_
 // bucket, the others are picked up from the same list by the next walk launch.
 // node2vec: `pick` is a proposal.  A walker whose proposal is rejected stays parked on v with one more trial on its
 // record; records carry the previous vertex instead of a position (the scatter kernel hands the positions out).
-template <int kApp>
+// v, off, deg: the list the lane's walker stands on (the same in every lane, or one list per 16-lane row with
+// kPerLane, where every lane then counts its own step); out_at: the walker's position in the output list.
+template <int kApp, bool kPerLane = false>
 __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_args& h, const int32_t v,
-                                             const uint32_t off, const uint32_t deg, const uint32_t rec_base,
+                                             const uint32_t off, const uint32_t deg, const uint32_t out_at,
                                              const fw_walker_rec rec, const uint32_t trial, const bool have,
                                              const int32_t pick, const uint32_t walker, const uint32_t step,
                                              const int lane, unsigned long long& n_steps,
@@ -1361,11 +1363,18 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
       go_on = !(u24(bits) < a.tp);
     }
   }
-  const uint64_t mmoved = __ballot(moved);
-  if (lane == 0) {
-    const unsigned long long c = (unsigned long long)__builtin_popcountll(mmoved);
-    n_steps += c;
-    n_edges += c * (unsigned long long)deg;
+  if (kPerLane) {
+    if (moved) {
+      n_steps += 1ull;
+      n_edges += (unsigned long long)deg;
+    }
+  } else {
+    const uint64_t mmoved = __ballot(moved);
+    if (lane == 0) {
+      const unsigned long long c = (unsigned long long)__builtin_popcountll(mmoved);
+      n_steps += c;
+      n_edges += c * (unsigned long long)deg;
+    }
   }
   bool park = false;
   int32_t hidx = -1;
@@ -1417,7 +1426,7 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
       if (kApp != FW_APP_NODE2VEC) out.prev = (int32_t)rank;
       out.len |= FW_REC_PARK;
     }
-    h.out[rec_base + (uint32_t)lane] = out;
+    h.out[out_at] = out;
   }
   const uint64_t mpark = __ballot(go_on && park);
   const uint64_t mres = __ballot(go_on && !park);
@@ -1486,7 +1495,8 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     const int32_t sel = table_sample<kApp, kNW>(a, bias, off, deg, want, (int32_t)deg > a.hub_threshold, have, walker,
                                                step, trial << 8, lane, h.totals + row_base,
                                                h.rows + (size_t)row_base * 128u, h.lastpos + row_base);
-    batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, trial, have, sel, walker, step, lane, n_steps, n_edges, n_out);
+    batch_commit<kApp>(a, h, v, off, deg, rec_base + (uint32_t)lane, rec, trial, have, sel, walker, step, lane, n_steps,
+                       n_edges, n_out);
   }
 
   // ---- then wave tasks: lists up to hub_threshold, sampled at wave granularity, one batch per wave; the tasks are
@@ -1515,7 +1525,8 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     float S;
     int32_t sel;
     batch_stream<kApp>(a, bias, off, deg, want, 0u, 1u, have, walker, step, trial << 8, lane, S, sel);
-    batch_commit<kApp>(a, h, v, off, deg, rec_base, rec, trial, have, sel, walker, step, lane, n_steps, n_edges, n_out);
+    batch_commit<kApp>(a, h, v, off, deg, rec_base + (uint32_t)lane, rec, trial, have, sel, walker, step, lane, n_steps,
+                       n_edges, n_out);
   }
 
   // ---- then workgroup tasks: lists above hub_threshold, sampled at workgroup granularity.  They are few, long and
@@ -1576,8 +1587,8 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
         wsel = wsel < 0 ? wlast : wsel;
         if (wsel >= 0) pick = s_sel[wsel][lane];
       }
-      batch_commit<kApp>(a, h, task.v, task.off, task.deg, task.rec_base, rec, trial, have, pick, walker, step, lane,
-                         n_steps, n_edges, n_out);
+      batch_commit<kApp>(a, h, task.v, task.off, task.deg, task.rec_base + (uint32_t)lane, rec, trial, have, pick, walker,
+                         step, lane, n_steps, n_edges, n_out);
     }
   }
 
@@ -1588,6 +1599,193 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     atomicAdd(&s_acc[1], n_edges);
   }
   // (a wave of node2vec walkers whose proposals were all rejected has walkers to hand on and no steps)
+  if (n_out[0] != 0u) atomicAdd(&s_out[0], n_out[0]);
+  if (n_out[1] != 0u) atomicAdd(&s_out[1], n_out[1]);
+  __syncthreads();
+  if (tid == 0) {
+    if (s_acc[0] != 0ull) {
+      atomicAdd(&a.counters[2], s_acc[0]);
+      atomicAdd(&a.counters[3], s_acc[1]);
+    }
+    if (s_out[0] != 0u) atomicAdd(&h.out_counts[0], s_out[0]);
+    if (s_out[1] != 0u) atomicAdd(&h.out_counts[1], s_out[1]);
+  }
+}
+
+// Quad tasks: lists of at most 64 aligned quartets with at most 16 walkers, four tasks per wave, one per 16-lane row
+// (most parked-on lists are short and hold a few walkers: a wave of its own would leave most of its lanes idle
+// through the per-walker part of the step).  Such a list is one group whose lane L holds quartet L alone; lane i of a
+// row stands in for lanes i, 16 + i, 32 + i and 48 + i of that group, one after the other, and puts their prefixes
+// together exactly as the whole-wave scan does: row_bcast:15 adds the last prefix of row 0 to row 1 and that of row 2
+// to row 3, row_bcast:31 then adds lane 31's sum to rows 2 and 3.  The walkers then resolve their targets as the table
+// tasks do, from rows that the wave keeps in LDS.  A kernel of its own, so that its registers are not the batch
+// kernel's.
+template <int kApp>
+__global__ __launch_bounds__(256, 8) void fw_hub_quad(const fw_kargs a, const fw_hub_args h) {
+  constexpr int kNW = 4;
+  __shared__ __align__(16) float s_qrows[kNW][4][128];  // per wave and row: 64 running maxima, 64 prefixes
+  __shared__ int32_t s_schema[kApp == FW_APP_METAPATH ? FW_MAX_SCHEMA : 1];
+  __shared__ unsigned long long s_acc[2];
+  __shared__ uint32_t s_out[2];
+  const int tid = (int)threadIdx.x;
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (tid == 0) {
+    s_acc[0] = s_acc[1] = 0ull;
+    s_out[0] = s_out[1] = 0u;
+  }
+  if (kApp == FW_APP_METAPATH && threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < FW_MAX_SCHEMA; ++i) s_schema[i] = a.schema[i];
+  }
+  const uint32_t* __restrict__ bias =
+      reinterpret_cast<const uint32_t*>(kApp == FW_APP_METAPATH ? (const void*)a.label : (const void*)a.weight);
+  unsigned long long n_steps = 0ull, n_edges = 0ull;
+  uint32_t n_out[2] = {0u, 0u};
+  const uint32_t nwaves = gridDim.x * (uint32_t)kNW;
+  __syncthreads();
+  {
+    const int row = lane >> 4;
+    const int rl = lane & 15;
+    const uint32_t nqtasks = *h.nqtasks;
+    float* const myM = &s_qrows[wave][row][0];
+    float* const myE = &s_qrows[wave][row][64];
+    const int row_last = (lane | 15) << 2;  // byte address of the row's lane 15 for ds_bpermute
+    for (uint32_t t4 = 4u * (blockIdx.x * (uint32_t)kNW + (uint32_t)wave); t4 < nqtasks; t4 += 4u * nwaves) {
+      const uint32_t t = t4 + (uint32_t)row;
+      const bool live = t < nqtasks;
+      fw_batch_task task;
+      task.v = 0; task.off = 0; task.deg = 0; task.rec_base = 0; task.count = 0; task.slot = 0; task.row = 0; task.pad = 0;
+      if (live) task = h.qtasks[t];
+      const int32_t want = kApp == FW_APP_METAPATH ? s_schema[task.slot] : 0;
+      const bool have = rl < task.count;
+      fw_walker_rec rec;
+      rec.q = 0; rec.cur = task.v; rec.prev = -1; rec.len = 1;
+      if (have) rec = h.sorted[task.rec_base + (uint32_t)rl];
+      uint32_t trial = 0u;
+      if (kApp == FW_APP_NODE2VEC) {
+        trial = (uint32_t)((rec.len >> FW_REC_TRIAL_SHIFT) & FW_REC_TRIAL_MASK);
+        rec.len &= FW_REC_LEN_MASK;
+      }
+      const uint32_t walker = a.walker_base + (uint32_t)rec.q;
+      const uint32_t step = (uint32_t)(rec.len - 1);
+
+      const uint32_t a0 = task.off & ~3u;
+      const uint32_t nq = (task.off + task.deg - a0 + 3u) >> 2;
+      float x[4][4];
+      float q[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const uint32_t k = 16u * (uint32_t)s + (uint32_t)rl;
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (live && k < nq) raw = *reinterpret_cast<const uint4*>(bias + a0 + 4u * k);
+        if (kApp == FW_APP_METAPATH) {
+          x[s][0] = (int32_t)raw.x == want ? 1.0f : 0.0f;
+          x[s][1] = (int32_t)raw.y == want ? 1.0f : 0.0f;
+          x[s][2] = (int32_t)raw.z == want ? 1.0f : 0.0f;
+          x[s][3] = (int32_t)raw.w == want ? 1.0f : 0.0f;
+        } else {
+          x[s][0] = __uint_as_float(raw.x);
+          x[s][1] = __uint_as_float(raw.y);
+          x[s][2] = __uint_as_float(raw.z);
+          x[s][3] = __uint_as_float(raw.w);
+        }
+        const uint32_t li = a0 + 4u * k - task.off;  // wraps below 0 for the head quartet
+        x[s][0] = live && k < nq && li < task.deg ? x[s][0] : 0.0f;
+        x[s][1] = live && k < nq && li + 1u < task.deg ? x[s][1] : 0.0f;
+        x[s][2] = live && k < nq && li + 2u < task.deg ? x[s][2] : 0.0f;
+        x[s][3] = live && k < nq && li + 3u < task.deg ? x[s][3] : 0.0f;
+        q[s] = (((0.0f + x[s][0]) + x[s][1]) + x[s][2]) + x[s][3];  // the lane's other twelve biases are zeros
+      }
+      // prefixes of the 64 lanes of the group, put together as wave_scan does
+      float I[4];
+      I[0] = row_scan(q[0]);
+      const float p1 = row_scan(q[1]);
+      const float p2 = row_scan(q[2]);
+      const float p3 = row_scan(q[3]);
+      const float R0 = bperm_f(row_last, I[0]);
+      I[1] = p1 + R0;
+      const float C1 = bperm_f(row_last, I[1]);
+      const float R2 = bperm_f(row_last, p2);
+      I[2] = p2 + C1;
+      I[3] = (p3 + R2) + C1;
+      const float T = bperm_f(row_last, I[3]);
+      // running maximum of the positive lanes' prefixes, and the last positive lane
+      float M[4];
+      uint32_t carry = 0u;
+      int lastpos = 0;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const bool pos = q[s] > 0.0f;
+        float m = pos ? I[s] : 0.0f;
+        m = dpp_max<0x111, 0xF>(m);
+        m = dpp_max<0x112, 0xF>(m);
+        m = dpp_max<0x114, 0xF>(m);
+        m = dpp_max<0x118, 0xF>(m);
+        const uint32_t mi = __float_as_uint(m);
+        M[s] = __uint_as_float(mi > carry ? mi : carry);
+        carry = __float_as_uint(bperm_f(row_last, M[s]));
+        const uint32_t mrow = (uint32_t)(__ballot(pos) >> (16 * row)) & 0xFFFFu;
+        if (mrow != 0u) lastpos = 16 * s + 31 - __builtin_clz(mrow);
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        myM[16 * s + rl] = M[s];
+        myE[16 * s + rl] = I[s] - q[s];
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+      // per walker: one group, so the reservoir accepts it as soon as its total is positive (S * 1 > 0)
+      const bool acc = have && (T * 1.0f > 0.0f);
+      int32_t sel = -1;
+      {
+        LaneDraw dq;
+        float target = 0.0f;
+        if (acc) target = next_uniform_lane(dq, a, walker, step, trial << 8) * T;
+        const float p15 = myM[15], p31 = myM[31], p47 = myM[47];
+        const int quarter = p15 > target ? 0 : (p31 > target ? 1 : (p47 > target ? 2 : 3));
+        const float4* Mq = reinterpret_cast<const float4*>(myM + 16 * quarter);
+        const float4 m0 = Mq[0], m1 = Mq[1], m2 = Mq[2], m3 = Mq[3];
+        const float mm[16] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w, m2.x, m2.y, m2.z, m2.w, m3.x, m3.y, m3.z, m3.w};
+        int below = 0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) below += mm[i] <= target ? 1 : 0;
+        const int src = below < 16 ? 16 * quarter + below : lastpos;
+        float e = myE[src];
+        // the quartet of lane src: held by the row's lane src & 15 in its pass src >> 4
+        const int from = ((lane & 48) | (src & 15)) << 2;
+        const int pass = src >> 4;
+        float xs[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const float y0 = bperm_f(from, x[0][c]), y1 = bperm_f(from, x[1][c]);
+          const float y2 = bperm_f(from, x[2][c]), y3 = bperm_f(from, x[3][c]);
+          xs[c] = pass == 0 ? y0 : (pass == 1 ? y1 : (pass == 2 ? y2 : y3));
+        }
+        uint32_t cnt = 0u, pm = 0u;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          e = e + xs[c];
+          cnt += e <= target ? 1u : 0u;
+          pm |= (xs[c] > 0.0f ? 1u : 0u) << c;
+        }
+        cnt += e <= target ? 12u : 0u;  // the twelve zeros that follow leave the sum where it is
+        const uint32_t cand = pm >> cnt;
+        const int pick = cand != 0u ? (int)cnt + __builtin_ctz(cand) : 31 - __builtin_clz(pm | 1u);
+        if (acc) sel = (int32_t)(a0 + 4u * (uint32_t)src + (uint32_t)pick - task.off);
+      }
+      __builtin_amdgcn_wave_barrier();  // the rows are rewritten by the wave's next four tasks
+      batch_commit<kApp, true>(a, h, task.v, task.off, task.deg, task.rec_base + (uint32_t)rl, rec, trial, have, sel, walker,
+                               step, lane, n_steps, n_edges, n_out);
+    }
+  }
+
+  if (n_steps != 0ull) {
+    atomicAdd(&s_acc[0], n_steps);
+    atomicAdd(&s_acc[1], n_edges);
+  }
   if (n_out[0] != 0u) atomicAdd(&s_out[0], n_out[0]);
   if (n_out[1] != 0u) atomicAdd(&s_out[1], n_out[1]);
   __syncthreads();
@@ -1644,6 +1842,24 @@ int launch_hub_scan_app(const fw_kargs& a, const fw_hub_args& h, uint32_t tasks_
   uint32_t grid = (uint32_t)cus * 8u;  // one resident set
   if (tasks_hint != 0u && tasks_hint / 2u + 32u < grid) grid = tasks_hint / 2u + 32u;  // 4 waves a workgroup, room to grow
   hipLaunchKernelGGL((fw_hub_scan<kApp>), dim3(grid), dim3(256), 0, stream, a, h);
+  FW_HIP(hipGetLastError());
+  return FW_OK;
+}
+
+// quads_hint: about how many quad tasks to expect (the launch works through any number; 0 = no idea).  Four tasks per
+// wave and turn, about eight turns per wave, between one and eight resident sets (see launch_hub_one).
+template <int kApp>
+int launch_hub_quad_app(const fw_kargs& a, const fw_hub_args& h, uint32_t quads_hint, hipStream_t stream) {
+  int dev = 0, cus = 0;
+  FW_HIP(hipGetDevice(&dev));
+  FW_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  const uint32_t resident = (uint32_t)cus * 8u;  // workgroups of four waves, eight waves per SIMD
+  uint32_t grid = resident;
+  if (quads_hint != 0u) {
+    const uint32_t wanted = quads_hint / (4u * 4u * 8u) + 1u;
+    grid = wanted < 8u * resident ? wanted : 8u * resident;
+  }
+  hipLaunchKernelGGL((fw_hub_quad<kApp>), dim3(grid), dim3(256), 0, stream, a, h);
   FW_HIP(hipGetLastError());
   return FW_OK;
 }
@@ -1779,6 +1995,18 @@ int fw_launch_hub_scan(const fw_kargs& a, const fw_hub_args& h, int app, uint32_
     case FW_APP_PPR: return launch_hub_scan_app<FW_APP_PPR>(a, h, tasks_hint, stream);
     case FW_APP_NODE2VEC: return launch_hub_scan_app<FW_APP_DEEPWALK>(a, h, tasks_hint, stream);  // the same rows: plain weights
     case FW_APP_METAPATH: return launch_hub_scan_app<FW_APP_METAPATH>(a, h, tasks_hint, stream);
+    default:
+      fw_set_error("unknown app %d", app);
+      return FW_ERR_INVALID;
+  }
+}
+
+int fw_launch_hub_quad(const fw_kargs& a, const fw_hub_args& h, int app, uint32_t quads_hint, hipStream_t stream) {
+  switch (app) {
+    case FW_APP_DEEPWALK: return launch_hub_quad_app<FW_APP_DEEPWALK>(a, h, quads_hint, stream);
+    case FW_APP_PPR: return launch_hub_quad_app<FW_APP_PPR>(a, h, quads_hint, stream);
+    case FW_APP_NODE2VEC: return launch_hub_quad_app<FW_APP_NODE2VEC>(a, h, quads_hint, stream);
+    case FW_APP_METAPATH: return launch_hub_quad_app<FW_APP_METAPATH>(a, h, quads_hint, stream);
     default:
       fw_set_error("unknown app %d", app);
       return FW_ERR_INVALID;
