@@ -17,6 +17,7 @@ pipeline, host-side round trips included.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-configs]
 """
 import argparse
+import ctypes as C
 import importlib
 import json
 import os
@@ -47,7 +48,8 @@ CONFIG_OF = {"deepwalk_rmat22": "C2", "ppr_rmat22": "C3", "node2vec_rmat24_sym":
 # 1 GiB copy kernel; the file under profiles/ holds the command and the per-kernel figures.  Reported beside the
 # bytes this run counts itself (roofline.requested_bytes), never instead of them.
 PROFILED_TRAFFIC = {
-    "deepwalk_rmat24_sym": (5.73e11, "profiles/walk_pipeline_deepwalk_rmat24sym_pmc.txt"),
+    "deepwalk_rmat24_sym": (5.54e11, "profiles/walk_pipeline_deepwalk_rmat24sym_pmc.txt"),
+    "node2vec_rmat24_sym": (9.83e11, "profiles/walk_pipeline_node2vec_rmat24sym_pmc.txt"),
 }
 
 
@@ -181,6 +183,9 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run the plain copy kernel on 1 GiB (what rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE are "
                          "scaled against)")
+    ap.add_argument("--calibration-random", action="store_true",
+                    help="also measure the memory's rate of scattered accesses over 4 GiB (64-byte line reads, 4-byte "
+                         "and 16-byte stores) and report it as calibration.random_access")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -224,6 +229,17 @@ def main():
         src.free()
         dst.free()
 
+    random_access = None
+    if args.calibration_random:
+        buf = fw.DeviceBuffer(4 << 30)
+        fw.check(fw.lib().fw_dev_fill_i32(buf.ptr, 0, (4 << 30) // 4))
+        random_access = {"buffer_GiB": 4}
+        for name, mode in (("line_reads_per_s", 0), ("stores_4B_per_s", 1), ("stores_16B_per_s", 3)):
+            rate = C.c_double(0.0)
+            fw.check(fw.lib().fw_dev_random_access_rate(buf.ptr, 4 << 30, mode, C.byref(rate)))
+            random_access[name] = rate.value
+        buf.free()
+
     for _ in range(args.warmup):
         g.walk_device(params, d_starts, n, d_paths)
 
@@ -245,7 +261,7 @@ def main():
     avg_kernel_ms = float(np.mean(kernel_ms))
     roofline = roofline_of(wl["app"], last, n, avg_kernel_ms)
     roofline["kernel"] = ("fw_walk_ref" if args.sampler != "native" else
-                          "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_scan + fw_hub_batch pipeline")
+                          "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_scan + fw_hub_batch + fw_hub_quad pipeline")
     # the profiler's view of the same workload (library defaults only: any override makes it another run)
     prof = PROFILED_TRAFFIC.get(args.workload) if defaults and last.launches > 1 else None
     roofline["traffic"] = prof[0] if prof else None
@@ -256,7 +272,7 @@ def main():
         # per-kernel view of the last pass: each kernel's own HIP-event time and the steps it took
         roofline["kernels"] = [
             {"kernel": "fw_walk_zprs", "total_ms": last.walk_kernel_ms, "steps": int(last.steps - last.hub_steps)},
-            {"kernel": "fw_hub_scan + fw_hub_batch", "total_ms": last.hub_kernel_ms, "steps": int(last.hub_steps)},
+            {"kernel": "fw_hub_scan + fw_hub_batch + fw_hub_quad", "total_ms": last.hub_kernel_ms, "steps": int(last.hub_steps)},
         ]
 
     out = {
@@ -284,6 +300,10 @@ def main():
         },
         "roofline": roofline,
     }
+    if random_access is not None:
+        # requested bytes / 64 ~ the memory transactions of a pass (lists in 64-byte lines + one line per scattered access)
+        random_access["pipeline_lines_per_s"] = roofline["requested_bytes"] / 64.0 / (avg_kernel_ms * 1e-3)
+        out["calibration"] = {"random_access": random_access}
 
     if not args.no_configs and defaults and args.workload == HEADLINE:
         # after the timed region: the headline without hub parking (every walker reads its lists itself, one launch:

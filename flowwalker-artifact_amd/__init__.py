@@ -30,7 +30,7 @@ EXPORTED = [
     "fw_graph_download", "fw_walk_device", "fw_walk_batch", "fw_host_alloc_pinned", "fw_host_free_pinned",
     "fw_gen_rmat", "fw_csr_read_header", "fw_csr_load", "fw_csr_write", "fw_graph_load",
     "fw_graph_create_placed", "fw_graph_load_placed", "fw_walk_device_noalloc", "fw_csr_sort_neighbours",
-    "fw_sampler_baseline_run",
+    "fw_sampler_baseline_run", "fw_dev_random_access_rate",
 ]
 
 
@@ -119,6 +119,7 @@ def lib():
         L.fw_csr_sort_neighbours.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                              C.POINTER(C.c_int64)]
         L.fw_graph_load.argtypes = [C.c_char_p, C.c_int, C.c_int, C.POINTER(C.c_void_p)]
+        L.fw_dev_random_access_rate.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double)]
         L.fw_sampler_baseline_run.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_uint64, C.c_uint32, C.c_void_p, C.c_uint32,
                                               C.c_int, C.c_uint64, C.c_void_p, C.POINTER(C.c_double)]
         L.fw_graph_load_placed.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p)]

@@ -161,6 +161,70 @@ extern "C" int fw_dev_copy(void* d_dst, const void* d_src, size_t bytes) {
   FW_HIP(hipDeviceSynchronize());
   return FW_OK;
 }
+// Calibration: how many scattered accesses per second the memory delivers.  Every thread touches `per_thread`
+// pseudo-random 64-byte lines of a buffer: mode 0 reads 4 bytes of each, mode 1 / 2 / 3 store 4 / 8 / 16 bytes into
+// each (a store that does not cover its line costs the memory a read-modify-write).  The walk pipeline's kernels
+// are priced against these rates: what bounds them is the number of memory transactions, not their bytes.
+__device__ __forceinline__ uint64_t fw_probe_mix(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+template <int kMode>
+__global__ __launch_bounds__(256) void fw_random_access_kernel(uint32_t* arr, uint64_t n_lines, uint32_t per_thread,
+                                                               uint32_t* sink) {
+  const uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x;
+  uint32_t acc = 0u;
+  for (uint32_t i = 0; i < per_thread; i += 4u) {
+    uint64_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = (fw_probe_mix(tid * per_thread + i + (uint32_t)j) % n_lines) * 16u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (kMode == 0) acc += arr[w[j] + (tid & 15u)];
+      else if (kMode == 1) arr[w[j] + (tid & 15u)] = i;
+      else if (kMode == 2) *reinterpret_cast<uint2*>(arr + w[j] + (tid & 14u)) = make_uint2(i, 1u);
+      else *reinterpret_cast<uint4*>(arr + w[j] + (tid & 12u)) = make_uint4(i, 1u, 2u, 3u);
+    }
+  }
+  if (acc == 0x12345678u) *sink = acc;  // keeps the loads
+}
+extern "C" int fw_dev_random_access_rate(void* d_buf, size_t bytes, int mode, double* accesses_per_s) {
+  if (!d_buf || !accesses_per_s || bytes < ((size_t)1 << 20) || (bytes & 63u) || ((uintptr_t)d_buf & 63u) || mode < 0 ||
+      mode > 3) {
+    fw_set_error("fw_dev_random_access_rate: buffer of at least 1 MiB, 64-byte aligned and sized; mode 0..3");
+    return FW_ERR_INVALID;
+  }
+  const uint64_t n_lines = bytes / 64u;  // > 0: every index below stays inside the buffer
+  const uint32_t per_thread = 256u;
+  const unsigned grid = 8192u;
+  uint32_t* sink = nullptr;
+  FW_HIP(hipMalloc(reinterpret_cast<void**>(&sink), 64));
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  int rc = fw_check_hip(hipEventCreate(&e0), "hipEventCreate", __FILE__, __LINE__);
+  if (rc == FW_OK) rc = fw_check_hip(hipEventCreate(&e1), "hipEventCreate", __FILE__, __LINE__);
+  float best = 0.0f;
+  for (int rep = 0; rc == FW_OK && rep < 3; ++rep) {
+    (void)hipEventRecord(e0, nullptr);
+    uint32_t* arr = static_cast<uint32_t*>(d_buf);
+    if (mode == 0) hipLaunchKernelGGL(fw_random_access_kernel<0>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink);
+    else if (mode == 1) hipLaunchKernelGGL(fw_random_access_kernel<1>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink);
+    else if (mode == 2) hipLaunchKernelGGL(fw_random_access_kernel<2>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink);
+    else hipLaunchKernelGGL(fw_random_access_kernel<3>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink);
+    rc = fw_check_hip(hipGetLastError(), "fw_random_access_kernel", __FILE__, __LINE__);
+    (void)hipEventRecord(e1, nullptr);
+    if (rc == FW_OK) rc = fw_check_hip(hipEventSynchronize(e1), "hipEventSynchronize", __FILE__, __LINE__);
+    float ms = 0.0f;
+    if (rc == FW_OK) rc = fw_check_hip(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime", __FILE__, __LINE__);
+    if (rep > 0 && (best == 0.0f || ms < best)) best = ms;
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  (void)hipFree(sink);
+  if (rc == FW_OK) *accesses_per_s = (double)grid * 256.0 * (double)per_thread / ((double)best * 1e-3);
+  return rc;
+}
 extern "C" int fw_dev_sync(void) {
   FW_HIP(hipDeviceSynchronize());
   return FW_OK;

@@ -144,6 +144,13 @@ int fw_dev_fill_i32(int32_t* d_dst, int32_t value, size_t count);
  * counters are calibrated against. */
 int fw_dev_copy(void* d_dst, const void* d_src, size_t bytes);
 int fw_dev_sync(void);
+/*
+ * Calibration, no counterpart in the reference: scattered accesses per second over d_buf (at least 1 MiB, 64-byte
+ * aligned and sized).  mode 0: 4-byte reads of pseudo-random 64-byte lines; 1 / 2 / 3: 4- / 8- / 16-byte stores into
+ * them (a store that does not cover its line costs the memory a read-modify-write).  bench.py reports these next to
+ * the walk pipeline's own transaction rate.
+ */
+int fw_dev_random_access_rate(void* d_buf, size_t bytes, int mode, double* accesses_per_s);
 
 /* ---- graph ------------------------------------------------------------------------------------ */
 
