@@ -419,3 +419,21 @@ def test_one_walk_call_at_a_time_per_graph(gpu):
             b.free()
         g.destroy()
         g2.destroy()
+
+
+def test_random_access_calibration(gpu):
+    """fw_dev_random_access_rate: refuses buffers it could index out of, and reports a rate for reads and stores."""
+    import ctypes as C
+    buf = gpu.DeviceBuffer(64 << 20)
+    rate = C.c_double(0.0)
+    L = gpu.lib()
+    try:
+        assert L.fw_dev_random_access_rate(buf.ptr, 0, 0, C.byref(rate)) == 1          # empty
+        assert L.fw_dev_random_access_rate(buf.ptr, (64 << 20) + 4, 0, C.byref(rate)) == 1  # not a multiple of a line
+        assert L.fw_dev_random_access_rate(buf.ptr, 64 << 20, 7, C.byref(rate)) == 1    # unknown mode
+        assert L.fw_dev_random_access_rate(None, 64 << 20, 0, C.byref(rate)) == 1
+        for mode in (0, 1, 3):
+            gpu.check(L.fw_dev_random_access_rate(buf.ptr, 64 << 20, mode, C.byref(rate)))
+            assert 1e9 < rate.value < 1e13
+    finally:
+        buf.free()
