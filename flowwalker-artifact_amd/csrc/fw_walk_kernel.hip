@@ -1400,8 +1400,13 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
     int32_t* const at = a.paths + ((uint64_t)(uint32_t)rec.q * (uint64_t)a.max_depth + (uint64_t)rec.len);
     const bool upper = (reinterpret_cast<uintptr_t>(at) & 4u) != 0u;
     if (moved) {
-      if (upper) *reinterpret_cast<int2*>(at - 1) = make_int2(v, nv);
-      else if (!(go_on && park)) *at = nv;
+      // (non-temporal: nobody reads a path entry before the call ends, and the line is not worth an L2 slot)
+      if (upper) {
+        const unsigned long long both = ((unsigned long long)(uint32_t)nv << 32) | (unsigned long long)(uint32_t)v;
+        __builtin_nontemporal_store((long long)both, reinterpret_cast<long long*>(at - 1));
+      } else if (!(go_on && park)) {
+        __builtin_nontemporal_store(nv, at);
+      }
     } else if (upper) {
       at[-1] = v;
     }
