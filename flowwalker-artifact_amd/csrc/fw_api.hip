@@ -822,42 +822,65 @@ __global__ void fw_round_reset_kernel(uint32_t* ctrs, int n_ctrs, uint32_t* coun
   }
 }
 
+// A record read that is not worth an L2 slot: the lists of records are streamed once per round, and what the L2
+// should keep are the small tables the same kernels look up per record (bucket offsets, counters).
+typedef int fw_v4i __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ fw_walker_rec load_rec_streaming(const fw_walker_rec* p) {
+  const fw_v4i v = __builtin_nontemporal_load(reinterpret_cast<const fw_v4i*>(p));
+  fw_walker_rec r;
+  r.q = v.x; r.cur = v.y; r.prev = v.z; r.len = v.w;
+  return r;
+}
+
 // Counting-sort scatter of a round's parked walkers into `sorted`.  Two sources share a bucket's range:
 //  * the previous batch launch's output list, of which only the records tagged FW_REC_PARK are parked; they carry
 //    their bucket and their position inside it (taken when they were parked) and fill the range from its start;
 //  * the walk kernel's list, whose records were only counted; they take positions from the end of the range here.
 __global__ void fw_scatter_tagged_kernel(const fw_walker_rec* __restrict__ src, uint32_t m,
                                          const uint32_t* __restrict__ bucket_offset,
-                                         fw_walker_rec* __restrict__ sorted) {
+                                         fw_parked_rec* __restrict__ sorted) {
   const uint32_t stride = gridDim.x * blockDim.x;
   for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < m; i += stride) {
-    fw_walker_rec r = src[i];
+    const fw_walker_rec r = load_rec_streaming(src + i);
     if (r.q < 0 || (r.len & FW_REC_PARK) == 0) continue;
-    r.len &= ~FW_REC_PARK;
-    sorted[bucket_offset[r.cur] + (uint32_t)r.prev] = r;
+    fw_parked_rec p;
+    p.q = r.q;
+    p.len = r.len & ~FW_REC_PARK;
+    sorted[bucket_offset[r.cur] + (uint32_t)r.prev] = p;
   }
 }
 
 // tagged_only (node2vec, whose records carry the previous vertex instead of a position): src is a batch launch's
-// output list, of which only the records tagged FW_REC_PARK take part.
+// output list, of which only the records tagged FW_REC_PARK take part.  whole (node2vec): the sorted list holds
+// fw_walker_rec, otherwise fw_parked_rec.
 __global__ void fw_scatter_counted_kernel(const fw_walker_rec* __restrict__ src, uint32_t m,
                                           const uint32_t* __restrict__ bucket_count,
                                           const uint32_t* __restrict__ bucket_offset, uint32_t* bucket_fill,
-                                          fw_walker_rec* __restrict__ sorted, int tagged_only) {
+                                          void* __restrict__ sorted, int tagged_only, int whole) {
   const uint32_t stride = gridDim.x * blockDim.x;
   for (uint32_t i0 = blockIdx.x * blockDim.x; i0 < m; i0 += stride) {  // uniform in the wave: the ranks are taken together
     const uint32_t i = i0 + threadIdx.x;
     bool have = i < m;
     fw_walker_rec r;
     r.q = 0; r.cur = 0; r.prev = 0; r.len = 0;
-    if (have) r = src[i];
+    if (have) r = load_rec_streaming(src + i);
     if (tagged_only) {
       have = have && r.q >= 0 && (r.len & FW_REC_PARK) != 0;
       r.len &= ~FW_REC_PARK;
     }
     const uint32_t b = (uint32_t)r.cur;
     const uint32_t rank = fw_wave_count_keys<true>(bucket_fill, b, have);
-    if (have) sorted[bucket_offset[b] + bucket_count[b] - 1u - rank] = r;
+    if (have) {
+      const uint32_t at = bucket_offset[b] + bucket_count[b] - 1u - rank;
+      if (whole) {  // node2vec
+        static_cast<fw_walker_rec*>(sorted)[at] = r;
+      } else {
+        fw_parked_rec p;
+        p.q = r.q;
+        p.len = r.len;
+        static_cast<fw_parked_rec*>(sorted)[at] = p;
+      }
+    }
   }
 }
 
@@ -908,16 +931,35 @@ __global__ __launch_bounds__(1024) void fw_compact_resume_kernel(const fw_walker
   }
 }
 
-// Parked records name their bucket; the walk kernel wants the vertex (used when the last few walkers leave the
-// park / batch loop).  The batch kernel may have left the path entry of a walker it parked again to the walker's next
-// step there (entries are stored in pairs); these walkers take that step in the walk kernel, so the entry is stored here.
-__global__ void fw_bucket_to_vertex_kernel(fw_walker_rec* recs, uint32_t m, const fw_hub_info* __restrict__ hub_info,
-                                           int labels, int32_t* __restrict__ paths, int32_t max_depth, int n2v) {
+// When the last few walkers leave the park / batch loop they take their next steps in the walk kernel, which wants
+// whole records that name the vertex.  Sorted record i belongs to the last bucket whose offset is at most i (empty
+// buckets share their offset with the next one that is not); node2vec's records name their bucket themselves.  The
+// batch kernel may have left the path entry of a walker it parked again to the walker's next step there (entries are
+// stored in pairs), so the entry is stored here.
+__global__ void fw_bucket_to_vertex_kernel(const void* sorted, uint32_t m, const uint32_t* __restrict__ bucket_offset,
+                                           int n_buckets, const fw_hub_info* __restrict__ hub_info, int labels,
+                                           int32_t* __restrict__ paths, int32_t max_depth, int n2v,
+                                           fw_walker_rec* __restrict__ whole) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= m) return;
-  const fw_walker_rec r = recs[i];
-  const int32_t v = hub_info[(uint32_t)r.cur / (uint32_t)labels].v;
-  recs[i].cur = v;
+  fw_walker_rec r;
+  uint32_t bucket;
+  if (n2v != 0) {
+    r = static_cast<const fw_walker_rec*>(sorted)[i];
+    bucket = (uint32_t)r.cur;
+  } else {
+    const fw_parked_rec p = static_cast<const fw_parked_rec*>(sorted)[i];
+    uint32_t lo = 0u, hi = (uint32_t)n_buckets;  // first bucket whose offset is above i
+    while (lo < hi) {
+      const uint32_t mid = (lo + hi) >> 1;
+      if (bucket_offset[mid] > i) hi = mid; else lo = mid + 1u;
+    }
+    bucket = lo - 1u;  // lo >= 1: offset[0] = 0 <= i
+    r.q = p.q; r.prev = -1; r.len = p.len;
+  }
+  const int32_t v = hub_info[bucket / (uint32_t)labels].v;
+  r.cur = v;
+  whole[i] = r;
   const int32_t len = n2v != 0 ? (r.len & FW_REC_LEN_MASK) : r.len;
   if (r.q >= 0 && len >= 1) paths[(uint64_t)(uint32_t)r.q * (uint64_t)max_depth + (uint64_t)(len - 1)] = v;
 }
@@ -1217,14 +1259,15 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     if (n_out != 0u) {
       if (p->app == FW_APP_NODE2VEC)
         hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
-                           pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 1);
+                           pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 1, 1);
       else
         hipLaunchKernelGGL(fw_scatter_tagged_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
-                           pb->offset(), pb->sorted);
+                           pb->offset(), reinterpret_cast<fw_parked_rec*>(pb->sorted));
     }
     if (n_walked != 0u)
       hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_walked)), dim3(256), 0, stream, pb->walked,
-                         n_walked, pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 0);
+                         n_walked, pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 0,
+                         p->app == FW_APP_NODE2VEC ? 1 : 0);
     FW_HIP(hipGetLastError());
     hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs, pb->count(nxt),
                        pb->fill(), pb->n_buckets, a.dispenser);
@@ -1233,10 +1276,10 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
       // default rule only (an explicit threshold keeps every round in the loop): too few walkers are left to
       // meet anywhere, so they finish in one walk launch that does not park
       hipLaunchKernelGGL(fw_bucket_to_vertex_kernel, dim3(((unsigned)m + 255u) / 256u), dim3(256), 0, stream,
-                         pb->sorted, (uint32_t)m, g->hub_info, labels, a.paths, a.max_depth,
-                         p->app == FW_APP_NODE2VEC ? 1 : 0);
+                         pb->sorted, (uint32_t)m, pb->offset(), pb->n_buckets, g->hub_info, labels, a.paths,
+                         a.max_depth, p->app == FW_APP_NODE2VEC ? 1 : 0, pb->resume);
       FW_HIP(hipGetLastError());
-      a.resume = pb->sorted;
+      a.resume = pb->resume;
       a.n_dev = nullptr;
       a.n = (int32_t)m;
       a.park_threshold = INT_MAX;
@@ -1338,7 +1381,7 @@ static uint64_t requested_bytes_model(const fw_walk_params* p, int32_t n, bool p
     // hub launches: the lists, and per walker its record in and out, the selected neighbour, the path entry, the
     // parking index of the new vertex and that vertex's bucket counter
     b += 16 * t.hub_quartets;
-    b += (2 * kRec + 4 * kLine) * hub_steps;
+    b += ((n2v ? kRec : kRec / 2) + kRec + 4 * kLine) * hub_steps;
     b += 8 * kLine * t.table_walkers;                             // pivots, lane row, prefix, four quartets of one lane
     // counting sort, compaction, task list, reset, bucket scan
     b += (kRec + kLine + kLine) * t.sorted_records + 2 * kRec * t.sorted_records;

@@ -97,6 +97,14 @@ constexpr int FW_REC_TRIAL_SHIFT = 16;
 constexpr int32_t FW_REC_TRIAL_MASK = 0x3FFF;
 constexpr int32_t FW_REC_LEN_MASK = 0xFFFF;
 
+// A parked walker in the sorted list, for every application but node2vec: the bucket follows from the position and
+// the previous vertex is not needed, so 8 bytes are enough -- half the scattered bytes of the counting sort, whose
+// time follows the bytes it scatters (node2vec keeps whole records: its acceptance test needs the previous vertex).
+struct fw_parked_rec {
+  int32_t q;
+  int32_t len;
+};
+
 // One batch: up to 64 walkers parked on vertex v, records sorted[rec_base .. rec_base + count).  32 bytes.
 struct fw_batch_task {
   int32_t v;
@@ -112,7 +120,7 @@ struct fw_batch_task {
 // Arguments of the hub batch kernel: up to 64 walkers parked on one vertex are served with one scan of its list,
 // by a workgroup (degree above hub_threshold: workgroup-granularity sampling) or by a single wave.
 struct fw_hub_args {
-  const fw_walker_rec* sorted;       // parked records grouped by bucket
+  const void* sorted;                // parked records grouped by bucket: fw_parked_rec, node2vec fw_walker_rec
   const fw_batch_task* tasks;        // workgroup tasks, handed out through task_next to the last dynamic_wgs workgroups
   uint32_t* task_next;
   uint32_t dynamic_wgs;              // set by the launch: the workgroups of one resident set

@@ -1328,6 +1328,16 @@ __device__ __forceinline__ int32_t table_sample(const fw_kargs& a, const uint32_
 // bucket, the others are picked up from the same list by the next walk launch.
 // node2vec: `pick` is a proposal.  A walker whose proposal is rejected stays parked on v with one more trial on its
 // record; records carry the previous vertex instead of a position (the scatter kernel hands the positions out).
+// Record `at` of the sorted list of parked walkers (the walker stands on v, the vertex of its task).
+template <int kApp>
+__device__ __forceinline__ fw_walker_rec load_parked(const void* sorted, uint32_t at, int32_t v) {
+  if (kApp == FW_APP_NODE2VEC) return static_cast<const fw_walker_rec*>(sorted)[at];
+  const fw_parked_rec p = static_cast<const fw_parked_rec*>(sorted)[at];
+  fw_walker_rec r;
+  r.q = p.q; r.cur = v; r.prev = -1; r.len = p.len;
+  return r;
+}
+
 // v, off, deg: the list the lane's walker stands on (the same in every lane, or one list per 16-lane row with
 // kPerLane, where every lane then counts its own step); out_at: the walker's position in the output list.
 template <int kApp, bool kPerLane = false>
@@ -1488,7 +1498,7 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     const bool have = lane < count;
     fw_walker_rec rec;
     rec.q = 0; rec.cur = v; rec.prev = -1; rec.len = 1;
-    if (have) rec = h.sorted[rec_base + (uint32_t)lane];
+    if (have) rec = load_parked<kApp>(h.sorted, rec_base + (uint32_t)lane, v);
     uint32_t trial = 0u;
     if (kApp == FW_APP_NODE2VEC) {
       trial = (uint32_t)((rec.len >> FW_REC_TRIAL_SHIFT) & FW_REC_TRIAL_MASK);
@@ -1518,7 +1528,7 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     const bool have = lane < count;
     fw_walker_rec rec;
     rec.q = 0; rec.cur = v; rec.prev = -1; rec.len = 1;
-    if (have) rec = h.sorted[rec_base + (uint32_t)lane];
+    if (have) rec = load_parked<kApp>(h.sorted, rec_base + (uint32_t)lane, v);
     uint32_t trial = 0u;
     if (kApp == FW_APP_NODE2VEC) {
       trial = (uint32_t)((rec.len >> FW_REC_TRIAL_SHIFT) & FW_REC_TRIAL_MASK);
@@ -1554,7 +1564,7 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     const bool have = lane < task.count;
     fw_walker_rec rec;
     rec.q = 0; rec.cur = task.v; rec.prev = -1; rec.len = 1;
-    if (have) rec = h.sorted[task.rec_base + (uint32_t)lane];
+    if (have) rec = load_parked<kApp>(h.sorted, task.rec_base + (uint32_t)lane, task.v);
     uint32_t trial = 0u;
     if (kApp == FW_APP_NODE2VEC) {
       trial = (uint32_t)((rec.len >> FW_REC_TRIAL_SHIFT) & FW_REC_TRIAL_MASK);
@@ -1666,7 +1676,7 @@ __global__ __launch_bounds__(256, 8) void fw_hub_quad(const fw_kargs a, const fw
       const bool have = rl < task.count;
       fw_walker_rec rec;
       rec.q = 0; rec.cur = task.v; rec.prev = -1; rec.len = 1;
-      if (have) rec = h.sorted[task.rec_base + (uint32_t)rl];
+      if (have) rec = load_parked<kApp>(h.sorted, task.rec_base + (uint32_t)rl, task.v);
       uint32_t trial = 0u;
       if (kApp == FW_APP_NODE2VEC) {
         trial = (uint32_t)((rec.len >> FW_REC_TRIAL_SHIFT) & FW_REC_TRIAL_MASK);
