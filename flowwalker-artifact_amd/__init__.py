@@ -34,7 +34,7 @@ EXPORTED = [
 ]
 
 
-BASELINE_ITS, BASELINE_RJS = 0, 1
+BASELINE_ITS, BASELINE_RJS, BASELINE_ALS = 0, 1, 2
 
 
 class WalkParams(C.Structure):

@@ -11,11 +11,12 @@
 // --type picks the algorithm, as TestSampler's --type does (src/sampler_test.cu:789-895): `native` = this engine's
 // one-pass group reservoir; `zprs` / `dprs` = the reference's own samplers restated for 64-lane waves
 // (include/sampler.cuh:46-127 and :129-200, FW_SAMPLER_REF_ZPRS / _DPRS: TestSampler types 1 / 2 and 3 / 4), run
-// on the same lists so that the columns can be compared; `its` / `rjs` = inverse transform and rejection sampling on
-// the same slices of the weight array (TestSampler types 5 / 6 and its RJS kernels, fw_sampler_baseline_run).
+// on the same lists so that the columns can be compared; `its` / `rjs` / `als` = inverse transform sampling,
+// rejection sampling and the alias method on the same slices of the weight array (TestSampler types 5 / 6, its RJS
+// kernels and types 7 / 8; fw_sampler_baseline_run).
 //
 //   fw_sampler_bench [--elements 268435456] [--gran 16,64,256,1024,4096,16384,65536] [--samples 4194304]
-//                    [--granularity wave|workgroup|both] [--type native,zprs,dprs,its,rjs] [--wg_threads 512] [--reps 3]
+//                    [--granularity wave|workgroup|both] [--type native,zprs,dprs,its,rjs,als] [--wg_threads 512] [--reps 3]
 //                    [--seed 1]
 // Output: one line per (gran, type, granularity): samples/s and GB/s of weights (4 bytes per element and sample;
 // the two-pass ZPRS reads them twice, which is not counted).
@@ -90,7 +91,8 @@ int main(int argc, char** argv) {
     else if (t == "dprs") run_types.push_back({"dprs", FW_SAMPLER_REF_DPRS});
     else if (t == "its") run_types.push_back({"its", -1 - FW_BASELINE_ITS});
     else if (t == "rjs") run_types.push_back({"rjs", -1 - FW_BASELINE_RJS});
-    else { fprintf(stderr, "fw_sampler_bench: --type takes native, zprs, dprs, its, rjs (got %s)\n", t.c_str()); return 2; }
+    else if (t == "als") run_types.push_back({"als", -1 - FW_BASELINE_ALS});
+    else { fprintf(stderr, "fw_sampler_bench: --type takes native, zprs, dprs, its, rjs, als (got %s)\n", t.c_str()); return 2; }
   }
   void* d_w = nullptr;  // the baselines read the weight array itself, not a graph
   for (const Type& type : run_types)

@@ -290,16 +290,16 @@ int fw_gen_rmat(const fw_rmat_params* rp, fw_graph** out);
 /* ---- sampler micro-benchmark baselines ----------------------------------------------------------- */
 
 /*
- * The two textbook samplers that the reference's sampler test compares its reservoir samplers with
+ * The three textbook samplers that the reference's sampler test compares its reservoir samplers with
  * (src/sampler_test.cu:290-410 and :561-712; include/sampler.cuh:850-884, :934-968 inverse transform sampling,
- * :970-1100 rejection sampling), for 64-lane waves.  They are a measuring stick, not part of the walk path.
+ * :970-1100 rejection sampling, :559-790 the alias method), for 64-lane waves.  They are a measuring stick, not part of the walk path.
  * d_weights: float[elements]; task position i draws ONE index from the list_len weights that start at
  * d_tasks[i] * list_len (d_tasks NULL: at i * list_len; every slice must lie inside the array) and writes it to
  * d_out[i] (-1 when no weight of the slice is positive).  workgroup = 0: one wave per task; 1: one workgroup of
  * wg_threads (256, 512 or 1024) per task.  Inverse transform sampling allocates its prefix-sum scratch
- * (list_len floats per resident worker) for the call.  kernel_ms (may be NULL): duration of the one launch.
+ * (list_len floats per resident worker) for the call, the alias method six times as much.  kernel_ms (may be NULL): duration of the one launch.
  */
-typedef enum { FW_BASELINE_ITS = 0, FW_BASELINE_RJS = 1 } fw_baseline_sampler;
+typedef enum { FW_BASELINE_ITS = 0, FW_BASELINE_RJS = 1, FW_BASELINE_ALS = 2 } fw_baseline_sampler;
 int fw_sampler_baseline_run(int type, int workgroup, const float* d_weights, uint64_t elements, uint32_t list_len,
                             const uint32_t* d_tasks, uint32_t n_tasks, int wg_threads, uint64_t seed, int32_t* d_out,
                             double* kernel_ms);

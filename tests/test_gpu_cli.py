@@ -84,17 +84,17 @@ def test_metapath_and_ppr(gpu, graph_files, tmp_path):
 
 
 def test_sampler_micro_benchmark_and_converter(gpu, tmp_path):
-    """fw_sampler_bench (one sampling step at fixed list lengths, five algorithms, both granularities) runs and reports every sample;
+    """fw_sampler_bench (one sampling step at fixed list lengths, six algorithms, both granularities) runs and reports every sample;
     a graph written by fw_convert loads and walks."""
     tool = os.path.join(ROOT, "flowwalker-artifact_amd", "bin", "fw_sampler_bench")
     r = subprocess.run([tool, "--elements", "1048576", "--samples", "20000", "--gran", "16,1024", "--reps", "1",
-                        "--type", "native,zprs,dprs,its,rjs"],
+                        "--type", "native,zprs,dprs,its,rjs,als"],
                        stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
     assert r.returncode == 0, r.stderr
     rows = [ln.split() for ln in r.stdout.splitlines()[1:]]
-    # per list length: this engine's sampler, the reference's ZPRS and DPRS on 64-lane waves, then inverse transform and
-    # rejection sampling, each at both granularities
-    want = [(g, t, s) for g in ("16", "1024") for t in ("native", "zprs", "dprs", "its", "rjs") for s in ("wave", "workgroup")]
+    # per list length: this engine's sampler, the reference's ZPRS and DPRS on 64-lane waves, then inverse transform sampling,
+    # rejection sampling and the alias method, each at both granularities
+    want = [(g, t, s) for g in ("16", "1024") for t in ("native", "zprs", "dprs", "its", "rjs", "als") for s in ("wave", "workgroup")]
     assert [(row[0], row[1], row[2]) for row in rows] == want
     assert all(int(row[3]) == 20000 and float(row[4]) > 0 for row in rows)
 

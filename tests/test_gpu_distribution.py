@@ -105,10 +105,10 @@ def test_node2vec_second_step_frequencies(gpu):
         g.destroy()
 
 
-@pytest.mark.parametrize("kind", ["its", "rjs"])
+@pytest.mark.parametrize("kind", ["its", "rjs", "als"])
 @pytest.mark.parametrize("workgroup,list_len", [(False, 40), (False, 700), (True, 700), (True, 5000)])
 def test_baseline_sampler_frequencies(gpu, kind, workgroup, list_len):
-    """fw_sampler_baseline_run: both textbook samplers draw index i with probability w_i / sum(w); zero weights
+    """fw_sampler_baseline_run: the three textbook samplers draw index i with probability w_i / sum(w); zero weights
     are never drawn, an all-zero slice and a slice beyond the array answer -1."""
     rng = np.random.RandomState(list_len)
     w = np.stack([rng.uniform(0.5, 20.0, list_len), np.zeros(list_len), rng.uniform(1.0, 2.0, list_len)]).astype(np.float32)
@@ -117,7 +117,7 @@ def test_baseline_sampler_frequencies(gpu, kind, workgroup, list_len):
     n = 2_000_000
     tasks = np.zeros(n, dtype=np.uint32)
     tasks[-3:] = (1, 2, 3)                                       # slice 1 is all zero, slice 3 does not exist
-    k = gpu.BASELINE_ITS if kind == "its" else gpu.BASELINE_RJS
+    k = {"its": gpu.BASELINE_ITS, "rjs": gpu.BASELINE_RJS, "als": gpu.BASELINE_ALS}[kind]
     out, ms = gpu.sampler_baseline(k, w.reshape(-1), list_len, tasks=tasks, workgroup=workgroup, seed=77)
     assert ms > 0 and out[-3] == -1 and out[-1] == -1 and 0 <= out[-2] < list_len
     draws = out[:-3]
