@@ -4,6 +4,7 @@ import ctypes as C
 import os
 import re
 import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -209,3 +210,23 @@ def test_sort_neighbours_moves_weights_and_labels_with_their_edges(fw):
     assert fw.csr_sort_neighbours(xadj, a2, w2, l2) == shuffled
     assert (a2 == adj).all() and (w2 == w).all() and (l2 == lab).all()   # uniform_graph's lists ascend, no duplicates
     assert fw.csr_sort_neighbours(xadj, a2, w2, l2) == 0
+
+
+def test_bench_measures_one_gpu_only():
+    """bench.py --gpus N with N above 1 exits with a message that says so (no figure at several GPUs is produced)."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE,
+                       stderr=subprocess.PIPE, text=True, timeout=120)
+    assert r.returncode != 0 and r.stdout.strip() == ""
+    assert "one GPU" in r.stderr and "--gpus 1" in r.stderr
+
+
+def test_bench_byte_formulas():
+    """The algorithmic bytes of a pass: 4*D + 16*S + 16*Q, for node2vec 8*D + 24*S + 16*Q (src/main.cu:93-104 counts D and S)."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_module", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    assert bench.algorithmic_bytes("deepwalk", 10, 1000, 3) == 4 * 1000 + 16 * 10 + 16 * 3
+    assert bench.algorithmic_bytes("metapath", 10, 1000, 3) == bench.algorithmic_bytes("ppr", 10, 1000, 3)
+    assert bench.algorithmic_bytes("node2vec", 10, 1000, 3) == 8 * 1000 + 24 * 10 + 16 * 3
+    assert bench.HBM_PEAK_GBS == 8000.0
