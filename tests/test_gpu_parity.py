@@ -186,6 +186,16 @@ def test_hub_parking_through_the_batch_driver(gpu, hub):
         p_off = gpu.default_params(max_depth=31, hub_threshold=1000, park_threshold=-1, seed=3)
         paths, st = g.walk(p_off, starts)
         assert (paths == ref).all() and st.launches == 1
+        # the other applications through the same driver, parked from a low degree on (short lists four to a wave,
+        # path entries stored in pairs, node2vec's rejected walkers waiting in their buckets)
+        for kw in (dict(app=gpu.APP_PPR, tp=0.1), dict(app=gpu.APP_NODE2VEC, p=2.0, q=0.5),
+                   dict(app=gpu.APP_METAPATH, schema=[1, 0, 2])):
+            p = gpu.default_params(max_depth=24, hub_threshold=1000, park_threshold=20, seed=11, **kw)
+            ref, steps, edges = _oracle.walk(og, _oracle.from_walk_params(p), starts)
+            for bs in (9000, 3001):
+                paths, st = g.walk_batch(p, starts, batch_size=bs, sync=False)
+                assert (paths == ref).all(), (kw, bs)
+                assert (st.steps, st.sampled_edges) == (steps, edges)
     finally:
         g.destroy()
 
