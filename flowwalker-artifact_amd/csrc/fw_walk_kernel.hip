@@ -872,7 +872,8 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
             if ((uint32_t)sp < (uint32_t)a.V && ln < a.max_depth) {
               const uint32_t o = a.xadj[sp];
               const uint32_t e = a.xadj[sp + 1];
-              if (parking) hidx = a.hub_index[sp];
+              // (a walker that resumes stands on a vertex nobody is parked on: the batch kernel looked it up)
+              hidx = parking && a.resume == nullptr ? a.hub_index[sp] : -1;
               deg = (int32_t)(e - o);
               if (deg > 0) {
                 tt.walker[tid] = wq;
