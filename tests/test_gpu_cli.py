@@ -239,3 +239,26 @@ def test_readme_node2vec_command_on_the_shipped_graph(gpu, tmp_path):
     ref, _, _ = orc.walk(orc.Graph(xadj, adj, w), orc.make_params(app=2, max_depth=81, seed=3, hub_threshold=(1 << 31) - 1),
                          np.arange(100, dtype=np.int32))
     assert (np.fromfile(out, dtype=np.int32).reshape(100, 81) == ref).all()
+
+
+def test_bench_line_contract(gpu):
+    """bench.py prints ONE JSON line with the agreed fields; the roofline fraction is a fraction (small graph, no CPU leg)."""
+    import json
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--scale", "16", "--steps", "2", "--warmup", "1",
+                        "--no-cpu"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr
+    lines = [ln for ln in r.stdout.splitlines() if ln.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 2 and d["warmup"] == 1 and d["unit"] == "steps/s" and d["vs_baseline"] is None
+    assert d["higher_is_better"] is True and d["data"] == "synthetic" and "workload" in d["config"]
+    rf = d["roofline"]
+    for key in ("bound", "achieved", "peak", "unit", "frac", "traffic"):
+        assert key in rf, key
+    assert rf["bound"] == "hbm" and rf["peak"] == 8000.0 and 0.0 < rf["frac"] <= 1.0
+    assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-9
+    assert d["value"] > 0 and abs(d["value"] - d["config"]["walk_steps_per_pass"] / (d["ms_per_step"] * 1e-3)) < 1e-6 * d["value"]
