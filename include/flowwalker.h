@@ -233,6 +233,9 @@ int fw_graph_load_placed(const char* prefix, int want_weight, int want_label, in
  * d_starts: int32[n]; d_paths: int32[n][max_depth], written completely (-1 padded; the caller does
  * not have to pre-fill it, unlike src/walk.cu:536).  stream: hipStream_t or NULL.  Synchronous:
  * returns after the kernel has finished; stats may be NULL.
+ * One walk call at a time per graph: the graph keeps the parking lists, the table of parked-on vertices and the
+ * launch record between calls, so a second fw_walk_device / fw_walk_batch on the same fw_graph while one is running
+ * (another host thread, whatever the stream) returns FW_ERR_INVALID.  Different graphs are independent.
  */
 int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const int32_t* d_starts, int32_t n,
                    int32_t* d_paths, void* stream, fw_walk_stats* stats);
