@@ -93,8 +93,8 @@ typedef struct {
   int32_t grid;           /* workgroups per launch actually used */
   /* per-kernel breakdown of kernel_ms / steps / sampled_edges (hub parking splits a pass over two kernels) */
   double walk_kernel_ms;      /* sum over fw_walk_zprs launches */
-  double hub_kernel_ms;       /* sum over fw_hub_batch launches (and the fw_hub_scan launches in front of them) */
-  uint64_t hub_steps;         /* steps taken in fw_hub_batch (included in steps) */
+  double hub_kernel_ms;       /* sum over the hub launches of every round: fw_hub_scan, fw_hub_batch, fw_hub_quad */
+  uint64_t hub_steps;         /* steps taken in the hub launches (included in steps) */
   uint64_t hub_sampled_edges; /* their source degrees (included in sampled_edges) */
   /* Bytes the call's kernels requested from the memory system, from the run's own counters: every list pass in
    * 16-byte quartets (a list is read once per walker step by the walk kernel, once per batch of up to 64 walkers
