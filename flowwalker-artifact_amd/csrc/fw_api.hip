@@ -993,6 +993,8 @@ struct ParkBuffers {
   void* tmp = nullptr;                // scan temporary storage
   size_t scan_bytes = 0;
   hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};  // timing events of the walk and the hub launches
+  hipStream_t side = nullptr;          // the quad launch of a round runs beside the batch launch
+  hipEvent_t fork = nullptr, join = nullptr;
 
   uint32_t* count(int parity) const { return buckets + (size_t)parity * n_buckets; }
   uint32_t* offset() const { return buckets + (size_t)2 * n_buckets; }
@@ -1014,6 +1016,9 @@ struct ParkBuffers {
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), kParkCtrs * sizeof(uint32_t)));
     FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), kParkCtrs * sizeof(uint32_t), hipHostMallocDefault));
     for (hipEvent_t& e : ev) FW_HIP(hipEventCreate(&e));
+    FW_HIP(hipStreamCreateWithFlags(&side, hipStreamNonBlocking));
+    FW_HIP(hipEventCreateWithFlags(&fork, hipEventDisableTiming));
+    FW_HIP(hipEventCreateWithFlags(&join, hipEventDisableTiming));
     // the rows are an extra: without room for them every bucket is served by batch tasks
     if (rows_wanted != 0u) {
       // scan tasks: a list of G groups is cut into at most G / kScanRun + 1 runs, and no more lists are scanned in
@@ -1052,6 +1057,11 @@ struct ParkBuffers {
       if (e) (void)hipEventDestroy(e);
       e = nullptr;
     }
+    if (side) (void)hipStreamDestroy(side);
+    if (fork) (void)hipEventDestroy(fork);
+    if (join) (void)hipEventDestroy(join);
+    side = nullptr;
+    fork = join = nullptr;
     walked = sorted = out = resume = nullptr;
     buckets = ctrs = h_ctrs = nullptr;
     tasks = wtasks = qtasks = nullptr;
@@ -1314,11 +1324,16 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     // work: an oversized grid puts them behind all wave tasks, and they are better spread among those.
     uint32_t tasks_hint = n_out != 0u ? (uint32_t)((uint64_t)batch_tasks * m / n_out) + 1u : 0u;
     if ((uint64_t)wg_task_waves * 16u > batch_tasks) tasks_hint = 0u;
+    // the short lists with few walkers, four to a wave (about as many as a round ago, scaled by the walkers): beside
+    // the batch launch on a stream of their own -- the two work on different tasks and meet only in counters
+    FW_HIP(hipEventRecord(pb->fork, stream));
+    FW_HIP(hipStreamWaitEvent(pb->side, pb->fork, 0));
+    rc = fw_launch_hub_quad(a, h, p->app, n_out != 0u ? (uint32_t)((uint64_t)quad_tasks * m / n_out) + 1u : 0u, pb->side);
+    if (rc != FW_OK) return rc;
+    FW_HIP(hipEventRecord(pb->join, pb->side));
     rc = fw_launch_hub_batch(a, h, p->app, p->wg_threads, tasks_hint, stream);
     if (rc != FW_OK) return rc;
-    // the short lists with few walkers, four to a wave (about as many as a round ago, scaled by the walkers)
-    rc = fw_launch_hub_quad(a, h, p->app, n_out != 0u ? (uint32_t)((uint64_t)quad_tasks * m / n_out) + 1u : 0u, stream);
-    if (rc != FW_OK) return rc;
+    FW_HIP(hipStreamWaitEvent(stream, pb->join, 0));
     if ((rc = th.end(stream)) != FW_OK) return rc;
     ++*launches;
     {
