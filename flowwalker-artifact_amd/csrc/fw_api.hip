@@ -559,16 +559,20 @@ __global__ void fw_hub_count_kernel(const uint32_t* __restrict__ xadj, int32_t V
   if (local) atomicAdd(count, local);
 }
 
+// Hub numbers are spread: hub k of the order in which the vertices come up gets number k * spread mod n_hubs (spread is a
+// prime that does not divide n_hubs, so this is a permutation).  Vertices that come up together are often busy together
+// (in an R-MAT graph the busiest vertices have the lowest ids), and the counters of buckets whose numbers are neighbours
+// share a 64-byte line, on which atomic updates queue behind each other.
 // next[0]: the next hub number; next[1]: the next free row.  A hub of at least rows_degree elements gets rows for its
 // groups (1024 elements each, from the list's first aligned quartet on) while fewer than rows_limit are taken.
 __global__ void fw_hub_index_kernel(const uint32_t* __restrict__ xadj, int32_t V, int32_t threshold, unsigned* next,
                                     int32_t* hub_index, fw_hub_info* hub_info, uint32_t rows_degree,
-                                    uint32_t rows_limit) {
+                                    uint32_t rows_limit, uint32_t n_hubs, uint32_t spread) {
   const int stride = gridDim.x * blockDim.x;
   for (int v = blockIdx.x * blockDim.x + threadIdx.x; v < V; v += stride) {
     int32_t idx = -1;
     if ((int32_t)(xadj[v + 1] - xadj[v]) > threshold) {
-      idx = (int32_t)atomicAdd(next, 1u);
+      idx = (int32_t)(((unsigned long long)atomicAdd(next, 1u) * spread) % n_hubs);  // a permutation: spread is coprime with n_hubs
       fw_hub_info hi;
       hi.v = v;
       hi.off = xadj[v];
@@ -601,9 +605,11 @@ static int ensure_hub_index(fw_graph* g, int32_t threshold) {
   int rc = fw_check_hip(hipMemcpy(&n_hubs, d_cnt, sizeof(unsigned), hipMemcpyDeviceToHost), "hipMemcpy(hub count)", __FILE__, __LINE__);
   if (rc == FW_OK) rc = fw_check_hip(hipMalloc(reinterpret_cast<void**>(&g->hub_index), (size_t)g->V * sizeof(int32_t)), "hipMalloc(hub_index)", __FILE__, __LINE__);
   if (rc == FW_OK) rc = fw_check_hip(hipMalloc(reinterpret_cast<void**>(&g->hub_info), (size_t)(n_hubs ? n_hubs : 1) * sizeof(fw_hub_info)), "hipMalloc(hub_info)", __FILE__, __LINE__);
+  uint32_t spread = 1u;
+  for (uint32_t prime : {1000003u, 999983u, 999979u}) if (n_hubs > 64u && n_hubs % prime != 0u) { spread = prime; break; }
   if (rc == FW_OK) {
     hipLaunchKernelGGL(fw_hub_index_kernel, dim3(1024), dim3(256), 0, 0, g->xadj, g->V, threshold, d_cnt + 1,
-                       g->hub_index, g->hub_info, kTwoPassDegree, kMaxHubRows);
+                       g->hub_index, g->hub_info, kTwoPassDegree, kMaxHubRows, n_hubs ? n_hubs : 1u, spread);
     rc = fw_check_hip(hipDeviceSynchronize(), "hub index", __FILE__, __LINE__);
   }
   unsigned rows_taken = 0;
