@@ -870,8 +870,9 @@ __global__ void fw_scatter_counted_kernel(const fw_walker_rec* __restrict__ src,
     fw_walker_rec r;
     r.q = 0; r.cur = 0; r.prev = 0; r.len = 0;
     if (have) r = load_rec_streaming(src + i);
+    have = have && r.q >= 0;  // both lists have holes
     if (tagged_only) {
-      have = have && r.q >= 0 && (r.len & FW_REC_PARK) != 0;
+      have = have && (r.len & FW_REC_PARK) != 0;
       r.len &= ~FW_REC_PARK;
     }
     const uint32_t b = (uint32_t)r.cur;
@@ -1250,6 +1251,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   tw.collect(&times->walk_ms);
   times->parked_records += pb->h_ctrs[0];
   uint32_t n_out = 0;  // records in `out` (the previous batch launch's input size)
+  uint32_t walk_entries = (uint32_t)a.n;  // entries of the last walk launch's input = positions of its list of parked walkers
   uint32_t fullest = 0;  // walkers in the fullest bucket of the previous round
   uint32_t scan_tasks = 0;  // and its scan tasks
   uint32_t quad_tasks = 0;  // and its quad tasks
@@ -1280,9 +1282,9 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
         hipLaunchKernelGGL(fw_scatter_tagged_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
                            pb->offset(), reinterpret_cast<fw_parked_rec*>(pb->sorted));
     }
-    if (n_walked != 0u)
-      hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_walked)), dim3(256), 0, stream, pb->walked,
-                         n_walked, pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 0,
+    if (n_walked != 0u)  // the walk launch's list has one position per entry of its input: parked walkers and holes
+      hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(walk_entries)), dim3(256), 0, stream, pb->walked,
+                         walk_entries, pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 0,
                          p->app == FW_APP_NODE2VEC ? 1 : 0);
     FW_HIP(hipGetLastError());
     hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs, pb->count(nxt),
@@ -1369,6 +1371,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     n_out = (uint32_t)m;
     fullest = pb->h_ctrs[12];
     resumed = pb->h_ctrs[6];
+    walk_entries = resumed;
     wg_task_waves = pb->h_ctrs[3] * (uint32_t)(p->wg_threads / 64);
     batch_tasks = pb->h_ctrs[5] + pb->h_ctrs[7] + wg_task_waves;
     quad_tasks = pb->h_ctrs[9];

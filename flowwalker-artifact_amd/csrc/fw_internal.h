@@ -79,8 +79,8 @@ struct fw_kargs {
   int32_t park_threshold;            // a walker that arrives on a vertex of larger degree is parked
   int32_t n_labels_per_hub;          // buckets per hub: 1, or schema_len for metapath (walkers wanting one label share a scan)
   const int32_t* hub_index;          // int32[V]: index of the vertex among the parked-on ones, -1, or -2 = degree 0
-  fw_walker_rec* parked;             // out: parked walkers
-  uint32_t* parked_count;
+  fw_walker_rec* parked;             // out: parked[i] = the walker of entry i of the launch's input if it was parked, else a hole (q = -1)
+  uint32_t* parked_count;            // += walkers parked (one update per workgroup)
   uint32_t* bucket_count;            // [n_hubs * n_labels_per_hub]
   const fw_walker_rec* resume;       // in: walkers to continue instead of fresh queries (NULL: use starts)
   const uint32_t* n_dev;             // in: when not NULL, the number of entries is read here (n is an upper bound

@@ -352,6 +352,8 @@ struct TaskTable {
   int32_t claim[2];
   int32_t exhausted;
   uint32_t cursor;            // resume lists: entries of this workgroup's share handed out so far
+  uint32_t entry[kWGT];       // parking: the slot's walker came in as entry number ... of the launch's input
+  uint32_t n_parked;          // walkers this workgroup has parked
   unsigned long long acc[2];  // steps, sum of source degrees of this workgroup
   // wave partials of the hub chunk in flight
   float hub_w[kHubChunk][16];
@@ -603,6 +605,7 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   unsigned long long n_steps = 0ull, n_edges = 0ull;
+  uint32_t my_parked = 0u;  // walkers parked, counted by the leading lanes of the parking waves
   // entries of this launch and the slots a workgroup fills: from the host, or (a launch queued before its input's
   // size was known to the host) from the device, with the same rule: small inputs are spread over the grid
   uint32_t n_entries = (uint32_t)a.n;
@@ -630,6 +633,7 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
     tt.claim[0] = tt.claim[1] = 0;
     tt.exhausted = 0;
     tt.cursor = 0u;
+    tt.n_parked = 0u;
     tt.acc[0] = tt.acc[1] = 0ull;
   }
   __syncthreads();
@@ -808,10 +812,12 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
         // park first: the record leaves the slot, which then asks for the next walker
         const uint64_t pm = __ballot(park);
         if (pm != 0ull) {
-          uint32_t pbase = 0;
-          const int pleader = __builtin_ctzll(pm);
-          if (lane == pleader) pbase = atomicAdd(a.parked_count, (uint32_t)__builtin_popcountll(pm));
-          pbase = (uint32_t)__builtin_amdgcn_readlane((int)pbase, pleader);
+          // The record goes to the position of the walker's entry in the launch's input (every entry is parked at most
+          // once), not to the end of a list: appending would take an update of one list counter per wave and round, and
+          // updates of one address complete one after the other -- with some 2,800 waves per launch that chain was as
+          // long as the rounds themselves.  The positions of walkers that are not parked hold holes (q = -1, written
+          // when the entry is taken).
+          if (lane == __builtin_ctzll(pm)) my_parked += (uint32_t)__builtin_popcountll(pm);
           const uint32_t label_slot =
               kApp == FW_APP_METAPATH ? (uint32_t)(len - 1) % (uint32_t)a.n_labels_per_hub : 0u;
           const uint32_t bucket = (uint32_t)hidx * (uint32_t)a.n_labels_per_hub + label_slot;
@@ -819,7 +825,7 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
           // vertices are contended); the counting sort hands the positions out later
           fw_wave_count_keys<false>(a.bucket_count, bucket, park);
           if (park) {
-            const uint32_t at = pbase + (uint32_t)__builtin_popcountll(pm & ((1ull << lane) - 1ull));
+            const uint32_t at = tt.entry[tid];
             fw_walker_rec rec;
             rec.q = tt.walker[tid];
             rec.cur = (int32_t)bucket;  // the vertex follows from the bucket
@@ -855,6 +861,10 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
             q = pos < (uint64_t)n_entries ? (uint32_t)pos : 0xFFFFFFFFu;
           }
           if (q < n_entries) {
+            if (parking) {  // the entry's place in the list of parked walkers: a hole until its walker is parked
+              a.parked[q].q = -1;
+              tt.entry[tid] = q;
+            }
             int32_t wq, sp, pv, ln, tr = 0;
             if (a.resume != nullptr) {  // a walker coming back from its batch step
               const fw_walker_rec rec = a.resume[q];
@@ -939,11 +949,13 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
     atomicAdd(&tt.acc[0], n_steps);
     atomicAdd(&tt.acc[1], n_edges);
   }
+  if (my_parked != 0u) atomicAdd(&tt.n_parked, my_parked);
   __syncthreads();
   if (tid == 0 && tt.acc[0] != 0ull) {
     atomicAdd(&a.counters[0], tt.acc[0]);
     atomicAdd(&a.counters[1], tt.acc[1]);
   }
+  if (tid == 0 && tt.n_parked != 0u) atomicAdd(a.parked_count, tt.n_parked);
 }
 
 // ---- hub batch kernel -----------------------------------------------------------------------------
