@@ -738,7 +738,7 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
     }
     __syncthreads();
     if (threadIdx.x == kKinds && s_cmax != 0u) {  // one update of the global maximum per workgroup
-      atomicMax(&ctrs[12], s_cmax);
+      atomicMax(&ctrs[12 * FW_CTR_STRIDE], s_cmax);
       s_cmax = 0u;
     }
     if (threadIdx.x < kKinds) {
@@ -749,7 +749,7 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
         total += v;
       }
       const int ctr = threadIdx.x == 0 ? 3 : (threadIdx.x == 1 ? 5 : (threadIdx.x == 2 ? 7 : (threadIdx.x == 3 ? 8 : 9)));
-      s_base[threadIdx.x] = total != 0u ? atomicAdd(&ctrs[ctr], total) : 0u;
+      s_base[threadIdx.x] = total != 0u ? atomicAdd(&ctrs[ctr * FW_CTR_STRIDE], total) : 0u;
     }
     __syncthreads();
     const int kind = two_pass ? 2 : (wg ? 0 : (quad ? 4 : 1));
@@ -809,8 +809,8 @@ __global__ __launch_bounds__(1024) void fw_bucket_tasks_kernel(const uint32_t* _
       q += s_q[w];
       tw += s_tot[2][w];
     }
-    if (q != 0ull) atomicAdd(reinterpret_cast<unsigned long long*>(ctrs + 14), q);
-    if (tw != 0u) atomicAdd(&ctrs[13], tw);
+    if (q != 0ull) atomicAdd(reinterpret_cast<unsigned long long*>(ctrs + 14 * FW_CTR_STRIDE), q);
+    if (tw != 0u) atomicAdd(&ctrs[13 * FW_CTR_STRIDE], tw);
   }
 }
 
@@ -1020,8 +1020,8 @@ struct ParkBuffers {
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&tasks), ntask * sizeof(fw_batch_task)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&wtasks), ntask * sizeof(fw_batch_task)));
     FW_HIP(hipMalloc(reinterpret_cast<void**>(&qtasks), (cap / 16 + (size_t)n + 1) * sizeof(fw_batch_task)));
-    FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), kParkCtrs * sizeof(uint32_t)));
-    FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), kParkCtrs * sizeof(uint32_t), hipHostMallocDefault));
+    FW_HIP(hipMalloc(reinterpret_cast<void**>(&ctrs), kParkCtrs * FW_CTR_STRIDE * sizeof(uint32_t)));
+    FW_HIP(hipHostMalloc(reinterpret_cast<void**>(&h_ctrs), kParkCtrs * FW_CTR_STRIDE * sizeof(uint32_t), hipHostMallocDefault));
     for (hipEvent_t& e : ev) FW_HIP(hipEventCreate(&e));
     FW_HIP(hipStreamCreateWithFlags(&side, hipStreamNonBlocking));
     FW_HIP(hipEventCreateWithFlags(&fork, hipEventDisableTiming));
@@ -1173,23 +1173,23 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   a.n_labels_per_hub = labels;
   a.hub_index = g->hub_index;
   a.parked = pb->walked;
-  a.parked_count = &pb->ctrs[0];
+  a.parked_count = &pb->ctrs[0 * FW_CTR_STRIDE];
   fw_hub_args h;
   h.sorted = pb->sorted;
   h.tasks = pb->tasks;
-  h.ntasks = &pb->ctrs[3];
-  h.task_next = &pb->ctrs[4];
+  h.ntasks = &pb->ctrs[3 * FW_CTR_STRIDE];
+  h.task_next = &pb->ctrs[4 * FW_CTR_STRIDE];
   h.dynamic_wgs = 0u;
   h.wtasks = pb->wtasks;
-  h.nwtasks = &pb->ctrs[5];
+  h.nwtasks = &pb->ctrs[5 * FW_CTR_STRIDE];
   h.out = pb->out;
-  h.out_counts = &pb->ctrs[1];
+  h.out_counts = &pb->ctrs[1 * FW_CTR_STRIDE];
   h.stasks = pb->stasks;
-  h.nstasks = &pb->ctrs[8];
+  h.nstasks = &pb->ctrs[8 * FW_CTR_STRIDE];
   h.ttasks = pb->ttasks;
-  h.nttasks = &pb->ctrs[7];
+  h.nttasks = &pb->ctrs[7 * FW_CTR_STRIDE];
   h.qtasks = pb->qtasks;
-  h.nqtasks = &pb->ctrs[9];
+  h.nqtasks = &pb->ctrs[9 * FW_CTR_STRIDE];
   h.totals = pb->totals;
   h.rows = pb->rows;
   h.lastpos = pb->lastpos;
@@ -1223,7 +1223,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     return FW_OK;
   };
   auto read_back = [&]() -> int {
-    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, kParkCtrs * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, kParkCtrs * FW_CTR_STRIDE * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     FW_HIP(hipStreamSynchronize(stream));
     return FW_OK;
   };
@@ -1238,7 +1238,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   }
   // first walk launch: fresh queries; the walkers it parks are counted in bucket array 0
   int cur = 0;
-  hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs, pb->count(0),
+  hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs * FW_CTR_STRIDE, pb->count(0),
                      pb->fill(), pb->n_buckets, a.dispenser);
   FW_HIP(hipGetLastError());
   a.resume = nullptr;
@@ -1249,7 +1249,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   if (rc != FW_OK) return rc;
   if ((rc = read_back()) != FW_OK) return rc;
   tw.collect(&times->walk_ms);
-  times->parked_records += pb->h_ctrs[0];
+  times->parked_records += pb->h_ctrs[0 * FW_CTR_STRIDE];
   uint32_t n_out = 0;  // records in `out` (the previous batch launch's input size)
   uint32_t walk_entries = (uint32_t)a.n;  // entries of the last walk launch's input = positions of its list of parked walkers
   uint32_t fullest = 0;  // walkers in the fullest bucket of the previous round
@@ -1262,8 +1262,8 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     // one round: the walkers parked by the last walk launch and by the last batch launch are grouped by bucket, the
     // batch launch moves each of them one step, and the walk launch queued right behind it takes those that are
     // not parked again as far as their next parking.  The host looks at the counters once per round.
-    const uint32_t n_walked = pb->h_ctrs[0];                 // parked by the walk launch
-    const uint32_t n_again = n_out ? pb->h_ctrs[2] : 0u;     // parked again by the previous batch launch
+    const uint32_t n_walked = pb->h_ctrs[0 * FW_CTR_STRIDE];                 // parked by the walk launch
+    const uint32_t n_again = n_out ? pb->h_ctrs[2 * FW_CTR_STRIDE] : 0u;     // parked again by the previous batch launch
     const uint64_t m = (uint64_t)n_walked + n_again;
     if (m == 0u) break;
     if (m > pb->cap) { fw_set_error("internal: %llu walkers parked, capacity %zu", (unsigned long long)m, pb->cap); return FW_ERR_INVALID; }
@@ -1287,7 +1287,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
                          walk_entries, pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 0,
                          p->app == FW_APP_NODE2VEC ? 1 : 0);
     FW_HIP(hipGetLastError());
-    hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs, pb->count(nxt),
+    hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs * FW_CTR_STRIDE, pb->count(nxt),
                        pb->fill(), pb->n_buckets, a.dispenser);
     FW_HIP(hipGetLastError());
     if (p->park_threshold == 0 && m < kParkTail) {
@@ -1348,13 +1348,13 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
       unsigned cblocks = ((unsigned)m + 4095u) / 4096u;
       if (cblocks > 1024u) cblocks = 1024u;
       hipLaunchKernelGGL(fw_compact_resume_kernel, dim3(cblocks), dim3(1024), 0, stream, pb->out, (uint32_t)m,
-                         pb->resume, pb->ctrs + 6);
+                         pb->resume, pb->ctrs + 6 * FW_CTR_STRIDE);
       FW_HIP(hipGetLastError());
     }
     // the walkers on vertices below the threshold continue in the walk kernel, which counts the walkers it parks in
     // the same bucket array as the batch launch did; how many they are is only known on the device yet
     a.resume = pb->resume;
-    a.n_dev = pb->ctrs + 6;
+    a.n_dev = pb->ctrs + 6 * FW_CTR_STRIDE;
     a.n = (int32_t)m;
     a.bucket_count = pb->count(nxt);
     entries_hint = hint_for(n_out != 0u ? (uint64_t)resumed + 1u : m / 4u + 1u);  // about as many as a round ago
@@ -1362,20 +1362,20 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     if ((rc = read_back()) != FW_OK) return rc;
     th.collect(&times->hub_ms);
     tw.collect(&times->walk_ms);
-    times->hub_quartets += *reinterpret_cast<const uint64_t*>(pb->h_ctrs + 14);
-    times->table_walkers += pb->h_ctrs[13];
-    times->parked_records += pb->h_ctrs[0];
-    times->resume_entries += pb->h_ctrs[6];
+    times->hub_quartets += *reinterpret_cast<const uint64_t*>(pb->h_ctrs + 14 * FW_CTR_STRIDE);
+    times->table_walkers += pb->h_ctrs[13 * FW_CTR_STRIDE];
+    times->parked_records += pb->h_ctrs[0 * FW_CTR_STRIDE];
+    times->resume_entries += pb->h_ctrs[6 * FW_CTR_STRIDE];
     times->sorted_records += m;
     times->bucket_passes += (uint64_t)pb->n_buckets;
     n_out = (uint32_t)m;
-    fullest = pb->h_ctrs[12];
-    resumed = pb->h_ctrs[6];
+    fullest = pb->h_ctrs[12 * FW_CTR_STRIDE];
+    resumed = pb->h_ctrs[6 * FW_CTR_STRIDE];
     walk_entries = resumed;
-    wg_task_waves = pb->h_ctrs[3] * (uint32_t)(p->wg_threads / 64);
-    batch_tasks = pb->h_ctrs[5] + pb->h_ctrs[7] + wg_task_waves;
-    quad_tasks = pb->h_ctrs[9];
-    scan_tasks = pb->h_ctrs[8];
+    wg_task_waves = pb->h_ctrs[3 * FW_CTR_STRIDE] * (uint32_t)(p->wg_threads / 64);
+    batch_tasks = pb->h_ctrs[5 * FW_CTR_STRIDE] + pb->h_ctrs[7 * FW_CTR_STRIDE] + wg_task_waves;
+    quad_tasks = pb->h_ctrs[9 * FW_CTR_STRIDE];
+    scan_tasks = pb->h_ctrs[8 * FW_CTR_STRIDE];
     cur = nxt;
   }
   return FW_OK;

@@ -105,6 +105,10 @@ struct fw_parked_rec {
   int32_t len;
 };
 
+// The counters of a parking round sit one to a 64-byte line (counter k at word k * FW_CTR_STRIDE): atomic updates of
+// one line complete one after the other wherever they come from, and several kernels update several of them at once.
+constexpr int FW_CTR_STRIDE = 16;
+
 // One batch: up to 64 walkers parked on vertex v, records sorted[rec_base .. rec_base + count).  32 bytes.
 struct fw_batch_task {
   int32_t v;
@@ -132,7 +136,7 @@ struct fw_hub_args {
   // bucket), untagged otherwise
   fw_walker_rec* out;
   uint32_t* bucket_out;
-  uint32_t* out_counts;              // [0] += records that resume, [1] += records parked again
+  uint32_t* out_counts;              // [0] += records that resume, [FW_CTR_STRIDE] += records parked again
   // Two-pass steps of crowded hubs.  The scan launch works through stasks (rec_base = first group of the run,
   // count = one past its last, row = the list's first row) and fills, per group of a list, totals[row],
   // rows[row * 128 ..] (64 running maxima, 64 prefixes) and lastpos[row]; the batch launch then serves ttasks

@@ -1636,7 +1636,7 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
       atomicAdd(&a.counters[3], s_acc[1]);
     }
     if (s_out[0] != 0u) atomicAdd(&h.out_counts[0], s_out[0]);
-    if (s_out[1] != 0u) atomicAdd(&h.out_counts[1], s_out[1]);
+    if (s_out[1] != 0u) atomicAdd(&h.out_counts[FW_CTR_STRIDE], s_out[1]);
   }
 }
 
@@ -1823,7 +1823,7 @@ __global__ __launch_bounds__(256, 8) void fw_hub_quad(const fw_kargs a, const fw
       atomicAdd(&a.counters[3], s_acc[1]);
     }
     if (s_out[0] != 0u) atomicAdd(&h.out_counts[0], s_out[0]);
-    if (s_out[1] != 0u) atomicAdd(&h.out_counts[1], s_out[1]);
+    if (s_out[1] != 0u) atomicAdd(&h.out_counts[FW_CTR_STRIDE], s_out[1]);
   }
 }
 
