@@ -1969,7 +1969,7 @@ int launch_hub_app(const fw_kargs& a, const fw_hub_args& h, int wg_threads, uint
 // walkers are short-lived (a step or two until they are parked again), so a launch is a few rounds of refills plus
 // a tail of sparse rounds that every workgroup pays; fewer workgroups with kEntriesPerWorkgroup entries each
 // (but at least one per compute unit) spend less on that tail than a full resident set with a few refills each.
-constexpr int kEntriesPerWorkgroup = 4864;
+constexpr int kEntriesPerWorkgroup = 2432;
 
 template <int kApp, int kWGT>
 int launch_one(fw_kargs a, int grid, uint32_t entries_hint, hipStream_t stream, int* grid_used) {
