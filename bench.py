@@ -48,8 +48,8 @@ CONFIG_OF = {"deepwalk_rmat22": "C2", "ppr_rmat22": "C3", "node2vec_rmat24_sym":
 # 1 GiB copy kernel; the file under profiles/ holds the command and the per-kernel figures.  Reported beside the
 # bytes this run counts itself (roofline.requested_bytes), never instead of them.
 PROFILED_TRAFFIC = {
-    "deepwalk_rmat24_sym": (5.41e11, "profiles/walk_pipeline_deepwalk_rmat24sym_pmc.txt"),
-    "node2vec_rmat24_sym": (9.63e11, "profiles/walk_pipeline_node2vec_rmat24sym_pmc.txt"),
+    "deepwalk_rmat24_sym": (5.48e11, "profiles/walk_pipeline_deepwalk_rmat24sym_pmc.txt"),
+    "node2vec_rmat24_sym": (9.86e11, "profiles/walk_pipeline_node2vec_rmat24sym_pmc.txt"),
 }
 
 
