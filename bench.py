@@ -5,12 +5,13 @@ Default workload = the headline configuration: DeepWalk, length 80, one query pe
 symmetrised R-MAT scale-24 graph (edge factor 16, a/b/c/d = .57/.19/.19/.05, weights U[1,100)).
 Inputs (CSR, start vertices, path matrix) are resident in HBM before the timed region starts.
 
-Prints ONE JSON line with the walk-steps/s of the whole job, the HBM roofline of the walk path
-(bytes the kernels of one pass requested from memory, counted by the library in the run / device time
-of that pass, measured with HIP events on the launch stream; the algorithmic bytes every walker would
-read alone are reported beside it), one line per benchmark configuration measured after the timed
-region (`configs`) and the CPU oracle timed on the host cores of the same box over a bounded prefix
-of the same queries.  With hub parking (the default for large batches) one pass is a short pipeline of launches --
+Prints ONE JSON line with the walk-steps/s of the whole job, the HBM roofline of the walk path on three
+stated bases (what the kernels of one pass ask of the memory, modelled from the run's counters; the
+useful part of it; the algorithmic bytes every walker would read alone -- all over the device time of
+that pass, measured with HIP events on the launch stream), the profiler's measured traffic for the same
+workload when the summary under profiles/ was taken on these sources, one line per benchmark
+configuration measured after the timed region (`configs`) and the CPU oracle timed on the host cores
+of the same box over a bounded prefix of the same queries.  With hub parking (the default for large batches) one pass is a short pipeline of launches --
 fw_walk_zprs, then per round fw_hub_scan + fw_hub_batch + fw_walk_zprs -- and the HIP events bracket the whole
 pipeline, host-side round trips included.
 
@@ -43,14 +44,33 @@ HEADLINE = "deepwalk_rmat24_sym"
 CONFIG_OF = {"deepwalk_rmat22": "C2", "ppr_rmat22": "C3", "node2vec_rmat24_sym": "C4", "metapath_rmat26": "C5",
              "deepwalk_rmat24_sym": "C4 graph, DeepWalk (headline)"}
 
-# HBM-side bytes of one pass (all launches of the walk pipeline) as rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE saw them
-# on an earlier run of the same workload with the library defaults, each counter scaled by what it reads for the
-# 1 GiB copy kernel; the file under profiles/ holds the command and the per-kernel figures.  Reported beside the
-# bytes this run counts itself (roofline.requested_bytes), never instead of them.
-PROFILED_TRAFFIC = {
-    "deepwalk_rmat24_sym": (5.48e11, "profiles/walk_pipeline_deepwalk_rmat24sym_pmc.txt"),
-    "node2vec_rmat24_sym": (9.86e11, "profiles/walk_pipeline_node2vec_rmat24sym_pmc.txt"),
+# The profiler's view of a pass (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read for
+# the 1 GiB copy kernel) lives in the summary under profiles/, in a line
+#   traffic_bytes_per_pass workload=<name> fetched=<B> written=<B> total=<B> sources=<sha of the kernel sources>
+# which is read at run time; the line says on which sources it was taken, and the JSON says whether those are the
+# sources of this run.
+PROFILE_OF = {
+    "deepwalk_rmat24_sym": "profiles/walk_pipeline_deepwalk_rmat24sym_pmc.txt",
+    "node2vec_rmat24_sym": "profiles/walk_pipeline_node2vec_rmat24sym_pmc.txt",
 }
+
+
+def profiled_traffic(workload, sources_sha):
+    """(total bytes, fields) of the traffic line for `workload` in its profile summary, or None."""
+    path = PROFILE_OF.get(workload)
+    if not path or not os.path.exists(os.path.join(ROOT, path)):
+        return None
+    for line in open(os.path.join(ROOT, path)):
+        parts = line.split()
+        if parts[:1] != ["traffic_bytes_per_pass"]:
+            continue
+        kv = dict(x.split("=", 1) for x in parts[1:] if "=" in x)
+        if kv.get("workload") != workload:
+            continue
+        return {"traffic": float(kv["total"]), "traffic_fetched": float(kv["fetched"]),
+                "traffic_written": float(kv["written"]), "traffic_source": path,
+                "traffic_sources_sha": kv.get("sources"), "traffic_taken_on_these_sources": kv.get("sources") == sources_sha}
+    return None
 
 
 def algorithmic_bytes(app, steps, sampled_edges, queries):
@@ -63,24 +83,31 @@ def algorithmic_bytes(app, steps, sampled_edges, queries):
 
 
 def roofline_of(app, st, n, kernel_ms):
-    """HBM roofline of one pass from the run's own counters.  `achieved` is the rate of the bytes the kernels
-    requested from the memory system (lists as often as they were actually streamed + 64 bytes per scattered access,
-    counted by the library: fw_walk_stats.requested_bytes) over the device time of the pass, so `frac` is a fraction
-    of what the memory can deliver.  `algorithmic_rate` divides the bytes every walker would read alone
-    (4*D + 16*S + 16*Q) by the same time: with hub parking a list is read once per batch of walkers, so this figure
-    exceeds the peak and `reuse_factor` = algorithmic / requested says by how much lists were shared.  node2vec's
-    algorithmic bytes are those of evaluating every neighbour's bias (8*D + 24*S + 16*Q); its two-stage step reads the
-    weights only, shares the passes, and makes one binary search per trial (counted as 16 lines per step)."""
+    """HBM roofline of one pass on three bases, all over the same device time.
+    * `achieved` / `frac`: what the kernels asked of the memory, MODELLED from the run's own counters
+      (fw_walk_stats: lists as often as they were actually streamed + 128 bytes per scattered read + 32 bytes per
+      scattered store + the records streamed; `breakdown` has the parts).  Bounded by 1.
+    * `useful_frac`: the part of it an implementation cannot avoid once lists are shared: the list bytes streamed
+      + 16 bytes per step + 16 bytes per query.
+    * `algorithmic_rate` / `algorithmic_frac`: the bytes every walker would read on its own (4*D + 16*S + 16*Q; node2vec
+      as the reference evaluates it, 8*D + 24*S + 16*Q) over the same time.  With hub parking a list is read once per
+      batch of walkers, so this exceeds the peak; `reuse_factor` = algorithmic / modelled says by how much lists were
+      shared.  Without parking (roofline.no_parking) it is the fraction of the roofline the walk kernel reaches."""
     alg = algorithmic_bytes(app, st.steps, st.sampled_edges, n)
     req = int(st.requested_bytes)
-    hbm = alg if req == 0 else req
     sec = kernel_ms * 1e-3
+    useful = int(st.list_bytes) + 16 * int(st.steps) + 16 * n
     return {
-        "bound": "hbm", "achieved": hbm / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": hbm / sec / 1e9 / HBM_PEAK_GBS, "kernel_ms": kernel_ms,
-        "bytes_basis": "algorithmic" if hbm == alg else "requested (counted by the library in this run)",
-        "requested_bytes": req, "algorithmic_bytes": int(alg), "algorithmic_rate": alg / sec / 1e9,
-        "reuse_factor": alg / hbm,
+        "bound": "hbm", "achieved": req / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": req / sec / 1e9 / HBM_PEAK_GBS, "kernel_ms": kernel_ms,
+        "bytes_basis": "modelled from the run's counters (lists as streamed + 128 B per scattered read + 32 B per "
+                       "scattered store + records)",
+        "requested_bytes": req,
+        "breakdown": {"list_bytes": int(st.list_bytes), "scattered_read_bytes": 128 * int(st.scattered_reads),
+                      "scattered_write_bytes": 32 * int(st.scattered_writes), "record_bytes": int(st.record_bytes)},
+        "useful_bytes": useful, "useful_frac": useful / sec / 1e9 / HBM_PEAK_GBS,
+        "algorithmic_bytes": int(alg), "algorithmic_rate": alg / sec / 1e9,
+        "algorithmic_frac": alg / sec / 1e9 / HBM_PEAK_GBS, "reuse_factor": alg / req if req else None,
     }
 
 
@@ -124,6 +151,7 @@ def one_config(fw, g, name, wl, passes, warmup, **overrides):
         "queries": n, "walk_steps_per_pass": int(st.steps), "passes": passes, "device_ms_per_pass": kernel_ms,
         "steps_per_s": st.steps / (kernel_ms * 1e-3), "launches_per_pass": st.launches,
         "frac": r["frac"], "achieved_GBs": r["achieved"], "bytes_basis": r["bytes_basis"],
+        "useful_frac": r["useful_frac"], "algorithmic_frac": r["algorithmic_frac"],
         "algorithmic_rate_GBs": r["algorithmic_rate"], "reuse_factor": r["reuse_factor"],
     }
 
@@ -157,6 +185,7 @@ def config1(fw):
                 "queries": 100, "walk_steps_per_pass": int(st.steps), "passes": 5, "device_ms_per_pass": kernel_ms,
                 "steps_per_s": st.steps / (kernel_ms * 1e-3), "launches_per_pass": st.launches, "frac": r["frac"],
                 "achieved_GBs": r["achieved"], "bytes_basis": r["bytes_basis"],
+                "useful_frac": r["useful_frac"], "algorithmic_frac": r["algorithmic_frac"],
                 "algorithmic_rate_GBs": r["algorithmic_rate"], "reuse_factor": r["reuse_factor"],
                 "note": "100 walks of 80 dependent steps: a latency measurement, not a bandwidth one"}
     finally:
@@ -234,7 +263,8 @@ def main():
         buf = fw.DeviceBuffer(4 << 30)
         fw.check(fw.lib().fw_dev_fill_i32(buf.ptr, 0, (4 << 30) // 4))
         random_access = {"buffer_GiB": 4}
-        for name, mode in (("line_reads_per_s", 0), ("stores_4B_per_s", 1), ("stores_16B_per_s", 3)):
+        for name, mode in (("line_reads_per_s", 0), ("stores_4B_per_s", 1), ("stores_16B_per_s", 3),
+                           ("loads_per_s_two_halves_of_one_128B_block", 4), ("loads_per_s_two_128B_blocks", 5)):
             rate = C.c_double(0.0)
             fw.check(fw.lib().fw_dev_random_access_rate(buf.ptr, 4 << 30, mode, C.byref(rate)))
             random_access[name] = rate.value
@@ -263,11 +293,12 @@ def main():
     roofline["kernel"] = ("fw_walk_ref" if args.sampler != "native" else
                           "fw_walk_zprs" if last.launches == 1 else "fw_walk_zprs + fw_hub_scan + fw_hub_batch + fw_hub_quad pipeline")
     # the profiler's view of the same workload (library defaults only: any override makes it another run)
-    prof = PROFILED_TRAFFIC.get(args.workload) if defaults and last.launches > 1 else None
-    roofline["traffic"] = prof[0] if prof else None
+    sources_sha = fw.sources_sha()
+    prof = profiled_traffic(args.workload, sources_sha) if defaults and last.launches > 1 else None
+    roofline["traffic"] = None
     if prof:
-        roofline["traffic_source"] = prof[1]
-        roofline["traffic_frac"] = prof[0] / (avg_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+        roofline.update(prof)
+        roofline["traffic_frac"] = prof["traffic"] / (avg_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
     if last.launches > 1:
         # per-kernel view of the last pass: each kernel's own HIP-event time and the steps it took
         roofline["kernels"] = [
@@ -296,19 +327,27 @@ def main():
             "wg_threads": params.wg_threads, "hub_threshold": params.hub_threshold,
             "park_threshold": params.park_threshold, "sampler": args.sampler, "launches_per_pass": last.launches,
             "grid": last.grid,
-            "graph_gen_s": round(gen_s, 2),
+            "graph_gen_s": round(gen_s, 2), "sources_sha": sources_sha,
         },
         "roofline": roofline,
     }
     if random_access is not None:
-        # requested bytes / 64 ~ the memory transactions of a pass (lists in 64-byte lines + one line per scattered access)
-        random_access["pipeline_lines_per_s"] = roofline["requested_bytes"] / 64.0 / (avg_kernel_ms * 1e-3)
+        # the modelled requests of a pass: lists in 128-byte blocks, one request per scattered read or store
+        random_access["pipeline_requests_per_s"] = (
+            (last.list_bytes + last.record_bytes) / 128.0 + last.scattered_reads + last.scattered_writes) / (avg_kernel_ms * 1e-3)
         out["calibration"] = {"random_access": random_access}
 
     if not args.no_configs and defaults and args.workload == HEADLINE:
         # after the timed region: the headline without hub parking (every walker reads its lists itself, one launch:
         # the walk kernel against the roofline on the bytes it touches) and one line per benchmark configuration
-        out["roofline"]["no_parking"] = one_config(fw, g, HEADLINE, wl, passes=1, warmup=0, park_threshold=-1)
+        nop = one_config(fw, g, HEADLINE, wl, passes=1, warmup=0, park_threshold=-1)
+        # one launch in which every walker reads its own lists: the walk kernel against the roofline on the algorithmic
+        # bytes 4*D + 16*S + 16*Q
+        nop["modelled_frac"] = nop["frac"]
+        nop["frac"] = nop["algorithmic_frac"]
+        nop["achieved_GBs"] = nop["algorithmic_rate_GBs"]
+        nop["bytes_basis"] = "algorithmic (4*D + 16*S + 16*Q)"
+        out["roofline"]["no_parking"] = nop
         configs = [config1(fw)]
         configs.append(one_config(fw, g, "node2vec_rmat24_sym", WORKLOADS["node2vec_rmat24_sym"], passes=3, warmup=1))
         cpu = None if args.no_cpu else cpu_baseline(fw, g, params, starts, args.cpu_seconds)
@@ -329,7 +368,8 @@ def main():
             "csr_entries": out["config"]["csr_entries"], "queries": n, "walk_steps_per_pass": int(last.steps),
             "passes": args.steps, "device_ms_per_pass": avg_kernel_ms, "steps_per_s": last.steps / (avg_kernel_ms * 1e-3),
             "launches_per_pass": last.launches, "frac": roofline["frac"], "achieved_GBs": roofline["achieved"],
-            "bytes_basis": roofline["bytes_basis"], "algorithmic_rate_GBs": roofline["algorithmic_rate"],
+            "bytes_basis": roofline["bytes_basis"], "useful_frac": roofline["useful_frac"],
+            "algorithmic_frac": roofline["algorithmic_frac"], "algorithmic_rate_GBs": roofline["algorithmic_rate"],
             "reuse_factor": roofline["reuse_factor"]})
         out["configs"] = configs
         if cpu is not None:
@@ -342,7 +382,9 @@ def main():
 
 
 def cpu_baseline(fw, g, params, starts, target_s):
-    """Times the CPU oracle (the checker, used here only as the reported baseline) on a prefix of the queries."""
+    """Times the CPU oracle (the checker, used here only as the reported baseline) on a prefix of the queries: one
+    warm-up run, then the best of three timed runs, wall clock around the walk only (the graph is in host memory);
+    the prefix is sized so that the three runs together take about target_s."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import fw_oracle_binding as orc
 
@@ -351,19 +393,22 @@ def cpu_baseline(fw, g, params, starts, target_s):
     og = orc.Graph(xadj, adj, w, lab)
     op = orc.from_walk_params(params)
     cores = orc.lib().fw_oracle_num_threads()
-    # pilot to size the sample so that the timed run takes about target_s
+    # warm-up, which also sizes the sample
     pilot = min(len(starts), 4096)
     t = time.perf_counter()
-    _, s0, _ = orc.walk(og, op, starts[:pilot])
+    orc.walk(og, op, starts[:pilot])
     dt = max(time.perf_counter() - t, 1e-4)
-    m = int(min(len(starts), max(pilot, pilot * target_s / dt)))
-    t = time.perf_counter()
-    _, steps, _ = orc.walk(og, op, starts[:m])
-    dt = time.perf_counter() - t
+    m = int(min(len(starts), max(pilot, pilot * (target_s / 3.0) / dt)))
+    best, steps = None, 0
+    for _ in range(3):
+        t = time.perf_counter()
+        _, steps, _ = orc.walk(og, op, starts[:m])
+        dt = time.perf_counter() - t
+        best = dt if best is None or dt < best else best
     return {
-        "value": steps / dt, "unit": "steps/s", "cores": int(cores), "kind": "port",
-        "sample": "first %d of %d queries of the same workload, %d steps in %.1f s, OpenMP schedule(dynamic)" % (
-            m, len(starts), steps, dt),
+        "value": steps / best, "unit": "steps/s", "cores": int(cores), "kind": "port",
+        "sample": "first %d of %d queries of the same workload, %d steps: one warm-up, best of 3 runs %.2f s, OpenMP "
+                  "schedule(dynamic)" % (m, len(starts), steps, best),
     }
 
 

@@ -19,6 +19,7 @@ LIB_PATH = os.environ.get("FLOWWALKER_LIB") or os.path.join(_PKG, "lib", "libflo
 FW_MAX_SCHEMA = 64
 APP_DEEPWALK, APP_PPR, APP_NODE2VEC, APP_METAPATH = 0, 1, 2, 3
 SAMPLER_ZPRS, SAMPLER_DPRS, SAMPLER_REF_ZPRS, SAMPLER_REF_DPRS, SAMPLER_REF_STATIC = 0, 1, 2, 3, 0x100
+SAMPLER_REF_RNG_LDS, SAMPLER_REF_RNG_GLOBAL = 0x200, 0x400
 FW_OK = 0
 GRAPH_DEVICE, GRAPH_HOST_PINNED = 0, 1
 
@@ -51,7 +52,8 @@ class WalkStats(C.Structure):
         ("kernel_ms", C.c_double), ("total_ms", C.c_double), ("steps", C.c_uint64),
         ("sampled_edges", C.c_uint64), ("launches", C.c_int32), ("grid", C.c_int32),
         ("walk_kernel_ms", C.c_double), ("hub_kernel_ms", C.c_double), ("hub_steps", C.c_uint64),
-        ("hub_sampled_edges", C.c_uint64), ("requested_bytes", C.c_uint64),
+        ("hub_sampled_edges", C.c_uint64), ("requested_bytes", C.c_uint64), ("list_bytes", C.c_uint64),
+        ("scattered_reads", C.c_uint64), ("scattered_writes", C.c_uint64), ("record_bytes", C.c_uint64),
     ]
 
 
@@ -61,6 +63,20 @@ class RmatParams(C.Structure):
         ("symmetrise", C.c_int32), ("w_lo", C.c_float), ("w_hi", C.c_float), ("n_labels", C.c_int32),
         ("make_weights", C.c_int32), ("seed", C.c_uint64),
     ]
+
+
+def sources_sha():
+    """Short hash of the kernel sources (csrc/*.hip, *.h and the public header): names the build a measurement was
+    taken on."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(_PKG, "csrc")
+    files = sorted(os.path.join(csrc, f) for f in os.listdir(csrc) if f.endswith((".hip", ".h")))
+    files.append(os.path.join(os.path.dirname(_PKG), "include", "flowwalker.h"))
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        h.update(open(f, "rb").read())
+    return h.hexdigest()[:12]
 
 
 class FlowWalkerError(RuntimeError):

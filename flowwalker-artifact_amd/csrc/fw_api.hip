@@ -163,8 +163,11 @@ extern "C" int fw_dev_copy(void* d_dst, const void* d_src, size_t bytes) {
 }
 // Calibration: how many scattered accesses per second the memory delivers.  Every thread touches `per_thread`
 // pseudo-random 64-byte lines of a buffer: mode 0 reads 4 bytes of each, mode 1 / 2 / 3 store 4 / 8 / 16 bytes into
-// each (a store that does not cover its line costs the memory a read-modify-write).  The walk pipeline's kernels
-// are priced against these rates: what bounds them is the number of memory transactions, not their bytes.
+// each (a store that does not cover its line costs the memory a read-modify-write).  Modes 4 and 5 settle the size of
+// a read request: both read two words per access, mode 4 from the two 64-byte halves of one random 128-byte block,
+// mode 5 from two different random blocks.  If the memory is asked for 128 bytes at a time, mode 4 costs one request
+// per pair and runs at about twice mode 5's rate of loads; if for 64, both cost two.  The walk pipeline's kernels are
+// priced against these rates.
 __device__ __forceinline__ uint64_t fw_probe_mix(uint64_t z) {
   z += 0x9E3779B97F4A7C15ull;
   z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
@@ -177,23 +180,33 @@ __global__ __launch_bounds__(256) void fw_random_access_kernel(uint32_t* arr, ui
   const uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x;
   uint32_t acc = 0u;
   for (uint32_t i = 0; i < per_thread; i += 4u) {
-    uint64_t w[4];
+    uint64_t w[4], w2[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) w[j] = (fw_probe_mix(tid * per_thread + i + (uint32_t)j) % n_lines) * 16u;
+    for (int j = 0; j < 4; ++j) {
+      const uint64_t r = fw_probe_mix(tid * per_thread + i + (uint32_t)j);
+      if (kMode >= 4) {  // n_lines counts 64-byte lines: blocks of 128 bytes are pairs of them
+        w[j] = (r % (n_lines >> 1)) * 32u;
+        w2[j] = kMode == 4 ? w[j] + 16u : (fw_probe_mix(r) % (n_lines >> 1)) * 32u;
+      } else {
+        w[j] = (r % n_lines) * 16u;
+        w2[j] = 0u;
+      }
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if (kMode == 0) acc += arr[w[j] + (tid & 15u)];
       else if (kMode == 1) arr[w[j] + (tid & 15u)] = i;
       else if (kMode == 2) *reinterpret_cast<uint2*>(arr + w[j] + (tid & 14u)) = make_uint2(i, 1u);
-      else *reinterpret_cast<uint4*>(arr + w[j] + (tid & 12u)) = make_uint4(i, 1u, 2u, 3u);
+      else if (kMode == 3) *reinterpret_cast<uint4*>(arr + w[j] + (tid & 12u)) = make_uint4(i, 1u, 2u, 3u);
+      else acc += arr[w[j] + (tid & 15u)] + arr[w2[j] + (tid & 15u)];
     }
   }
   if (acc == 0x12345678u) *sink = acc;  // keeps the loads
 }
 extern "C" int fw_dev_random_access_rate(void* d_buf, size_t bytes, int mode, double* accesses_per_s) {
-  if (!d_buf || !accesses_per_s || bytes < ((size_t)1 << 20) || (bytes & 63u) || ((uintptr_t)d_buf & 63u) || mode < 0 ||
-      mode > 3) {
-    fw_set_error("fw_dev_random_access_rate: buffer of at least 1 MiB, 64-byte aligned and sized; mode 0..3");
+  if (!d_buf || !accesses_per_s || bytes < ((size_t)1 << 20) || (bytes & 127u) || ((uintptr_t)d_buf & 127u) || mode < 0 ||
+      mode > 5) {
+    fw_set_error("fw_dev_random_access_rate: buffer of at least 1 MiB, 128-byte aligned and sized; mode 0..5");
     return FW_ERR_INVALID;
   }
   const uint64_t n_lines = bytes / 64u;  // > 0: every index below stays inside the buffer
@@ -208,10 +221,14 @@ extern "C" int fw_dev_random_access_rate(void* d_buf, size_t bytes, int mode, do
   for (int rep = 0; rc == FW_OK && rep < 3; ++rep) {
     (void)hipEventRecord(e0, nullptr);
     uint32_t* arr = static_cast<uint32_t*>(d_buf);
-    if (mode == 0) hipLaunchKernelGGL(fw_random_access_kernel<0>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink);
-    else if (mode == 1) hipLaunchKernelGGL(fw_random_access_kernel<1>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink);
-    else if (mode == 2) hipLaunchKernelGGL(fw_random_access_kernel<2>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink);
-    else hipLaunchKernelGGL(fw_random_access_kernel<3>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink);
+    switch (mode) {
+      case 0: hipLaunchKernelGGL(fw_random_access_kernel<0>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink); break;
+      case 1: hipLaunchKernelGGL(fw_random_access_kernel<1>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink); break;
+      case 2: hipLaunchKernelGGL(fw_random_access_kernel<2>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink); break;
+      case 3: hipLaunchKernelGGL(fw_random_access_kernel<3>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink); break;
+      case 4: hipLaunchKernelGGL(fw_random_access_kernel<4>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink); break;
+      default: hipLaunchKernelGGL(fw_random_access_kernel<5>, dim3(grid), dim3(256), 0, nullptr, arr, n_lines, per_thread, sink); break;
+    }
     rc = fw_check_hip(hipGetLastError(), "fw_random_access_kernel", __FILE__, __LINE__);
     (void)hipEventRecord(e1, nullptr);
     if (rc == FW_OK) rc = fw_check_hip(hipEventSynchronize(e1), "hipEventSynchronize", __FILE__, __LINE__);
@@ -222,7 +239,8 @@ extern "C" int fw_dev_random_access_rate(void* d_buf, size_t bytes, int mode, do
   if (e0) (void)hipEventDestroy(e0);
   if (e1) (void)hipEventDestroy(e1);
   (void)hipFree(sink);
-  if (rc == FW_OK) *accesses_per_s = (double)grid * 256.0 * (double)per_thread / ((double)best * 1e-3);
+  // modes 4 and 5 make two loads per access: the rate counts loads
+  if (rc == FW_OK) *accesses_per_s = (double)grid * 256.0 * (double)per_thread * (mode >= 4 ? 2.0 : 1.0) / ((double)best * 1e-3);
   return rc;
 }
 extern "C" int fw_dev_sync(void) {
@@ -392,7 +410,7 @@ __global__ void fw_sorted_kernel(const uint32_t* __restrict__ xadj, const int32_
   for (int v = blockIdx.x * blockDim.x + threadIdx.x; v < V; v += stride) {
     const uint32_t b = xadj[v], e = xadj[v + 1];
     for (uint32_t i = b + 1; i < e; ++i) {
-      if (adjncy[i] <= adjncy[i - 1]) { *unsorted = 1; break; }
+      if (adjncy[i] < adjncy[i - 1]) { *unsorted = 1; break; }  // equal neighbours (a multigraph) are in order
     }
   }
 }
@@ -502,7 +520,7 @@ static int check_walk_args(const fw_graph* g, const fw_walk_params* p, const voi
     const int rc = graph_sorted(g, &sorted, d_flag);  // one pass over the adjacency the first time, then cached
     if (rc != FW_OK) return rc;
     if (!sorted) {
-      fw_set_error("walk: node2vec needs strictly ascending neighbour lists and this graph has others "
+      fw_set_error("walk: node2vec needs ascending neighbour lists and this graph has others "
                    "(fw_csr_sort_neighbours sorts a host CSR before the upload)");
       return FW_ERR_INVALID;
     }
@@ -1381,37 +1399,53 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   return FW_OK;
 }
 
-// Bytes a call's kernels request from the memory system, from the counters of the run: lists are streamed in
-// 16-byte quartets, every scattered access (a path entry, a CSR offset pair, a parking index, a counter, the selected
-// neighbour) is one 64-byte line, records are 16 bytes.  See fw_walk_stats::requested_bytes.
-static uint64_t requested_bytes_model(const fw_walk_params* p, int32_t n, bool parked, int32_t park_threshold,
-                                      uint64_t walk_steps, uint64_t walk_edges, uint64_t hub_steps,
-                                      const KernelTimes& t) {
-  constexpr uint64_t kLine = 64, kRec = 16;
+// What a call's kernels ask of the memory, modelled from the run's own counters (steps, records, list quartets, table
+// walkers): the lists as often as they were actually streamed, the scattered reads (one 128-byte block each: that is
+// what the L2 asks the memory for, a pair of reads from the two halves of a block costs what one read costs), the
+// scattered stores (one 32-byte write request each: a path entry or pair, a record) and the records and tasks that are
+// streamed.  Tables that stay in the L2s (bucket counters, bucket offsets: 4 bytes per parked-on vertex) are not
+// priced.  A model, not a measurement: the profiler's FETCH_SIZE / WRITE_SIZE are the measurement.
+struct TrafficModel {
+  uint64_t list_bytes = 0;
+  uint64_t scattered_reads = 0;
+  uint64_t scattered_writes = 0;
+  uint64_t record_bytes = 0;
+  uint64_t total() const { return list_bytes + 128u * scattered_reads + 32u * scattered_writes + record_bytes; }
+};
+
+static TrafficModel traffic_model(const fw_walk_params* p, int32_t n, bool parked, int32_t park_threshold,
+                                  uint64_t walk_steps, uint64_t walk_edges, uint64_t hub_steps, const KernelTimes& t) {
+  constexpr uint64_t kRec = 16;
   const bool n2v = p->app == FW_APP_NODE2VEC;
-  uint64_t b = 0;
+  TrafficModel m;
   // walk launches.  A list is read from its first aligned quartet on (about 12 bytes of padding per step); lists of
   // up to 64 quartets bring their neighbours along with the biases, longer ones fetch the selected neighbour alone.
   const bool short_lists = parked && park_threshold <= 252;
-  const uint64_t per_entry_array = short_lists ? 2 : 1;
-  b += per_entry_array * (4 * walk_edges + 12 * walk_steps);
-  if (!short_lists) b += kLine * walk_steps;                      // adjncy[off + sel]
-  b += (kLine + kLine + (parked ? kLine : 0)) * walk_steps;       // path entry, xadj pair, parking index
-  if (n2v) b += 16 * kLine * (walk_steps + hub_steps);            // about one binary search in N(prev) per step
-  b += (4 + kLine + kLine + (parked ? kLine : 0)) * (uint64_t)n;  // start vertex, path[0], xadj pair, parking index
+  m.list_bytes += (short_lists ? 2u : 1u) * (4 * walk_edges + 12 * walk_steps);
+  if (!short_lists) m.scattered_reads += walk_steps;             // adjncy[off + sel]
+  m.scattered_reads += (parked ? 2u : 1u) * walk_steps;          // xadj pair, parking index
+  m.scattered_writes += walk_steps;                              // path entry
+  if (n2v) m.scattered_reads += 8 * (walk_steps + hub_steps);    // about one search in N(prev) per step
+  m.record_bytes += 4 * (uint64_t)n;                             // start vertices
+  m.scattered_reads += (parked ? 2u : 1u) * (uint64_t)n;         // xadj pair, parking index
+  m.scattered_writes += (uint64_t)n;                             // path[0]
   if (parked) {
-    b += (kRec + kLine) * t.parked_records;                       // record out, bucket counter
-    b += (kRec + kLine + kLine) * t.resume_entries;               // record in, xadj pair, parking index
-    // hub launches: the lists, and per walker its record in and out, the selected neighbour, the path entry, the
-    // parking index of the new vertex and that vertex's bucket counter
-    b += 16 * t.hub_quartets;
-    b += ((n2v ? kRec : kRec / 2) + kRec + 4 * kLine) * hub_steps;
-    b += 8 * kLine * t.table_walkers;                             // pivots, lane row, prefix, four quartets of one lane
-    // counting sort, compaction, task list, reset, bucket scan
-    b += (kRec + kLine + kLine) * t.sorted_records + 2 * kRec * t.sorted_records;
-    b += (12 + 8 + 8) * t.bucket_passes;
+    m.scattered_writes += t.parked_records;                      // record out (the bucket counter stays in the L2)
+    m.record_bytes += kRec * t.resume_entries;                   // record in
+    m.scattered_reads += t.resume_entries;                       // xadj pair
+    // hub launches: the lists, and per walker its record in and out, the selected neighbour, the parking index of
+    // the new vertex and the path entry
+    m.list_bytes += 16 * t.hub_quartets;
+    m.record_bytes += ((n2v ? kRec : kRec / 2) + kRec) * hub_steps;
+    m.scattered_reads += 2 * hub_steps;
+    m.scattered_writes += hub_steps;
+    m.scattered_reads += 7 * t.table_walkers;                    // pivots, lane row, prefix, four quartets of one lane
+    // counting sort (record in, scattered record out), compaction (in, out), task list, reset, bucket scan
+    m.record_bytes += 3 * kRec * t.sorted_records;
+    m.scattered_writes += t.sorted_records;
+    m.record_bytes += (12 + 8 + 8) * t.bucket_passes;
   }
-  return b;
+  return m;
 }
 
 struct Scratch {  // dispenser word + workload counters of the two kernels, 48 bytes per launch slot
@@ -1430,7 +1464,7 @@ struct BusyGuard {
     int expected = 0;
     held = g->busy.compare_exchange_strong(expected, 1);
     if (!held) fw_set_error("walk: another walk call is running on this fw_graph (one call at a time per graph; "
-                            "make a second fw_graph, or use fw_walk_device_noalloc, to walk concurrently)");
+                            "make a second fw_graph to walk concurrently)");
   }
   bool ok() const { return held; }
   ~BusyGuard() { if (held) g->busy.store(0); }
@@ -1511,8 +1545,13 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
     stats->hub_kernel_ms = times.hub_ms;
     stats->hub_steps = h.counters[2];
     stats->hub_sampled_edges = h.counters[3];
-    stats->requested_bytes = requested_bytes_model(p, n, launches > 1, park_threshold, h.counters[0], h.counters[1],
-                                                   h.counters[2], times);
+    const TrafficModel tm = traffic_model(p, n, launches > 1, park_threshold, h.counters[0], h.counters[1],
+                                          h.counters[2], times);
+    stats->requested_bytes = tm.total();
+    stats->list_bytes = tm.list_bytes;
+    stats->scattered_reads = tm.scattered_reads;
+    stats->scattered_writes = tm.scattered_writes;
+    stats->record_bytes = tm.record_bytes;
   }
   return FW_OK;
 }
@@ -1523,7 +1562,9 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
 // This variant keeps that scratch in a file-scope device array and creates its events once per device, so a call
 // makes no hipMalloc / hipFree / hipEventCreate.  Every device holds its own copy of the array at its own address;
 // the address is looked up once per device (the array's name is only a host-side handle, never a kernel argument).
-// All calls on a device share the array: calls that overlap on one device race on it.
+// All calls on a device share the array, so a call that starts while another one is running on the same device is
+// refused.  The call is synchronous like fw_walk_device (it waits for its launch and reads the counters back), so it is
+// not a call to make while a stream is being captured into a graph.
 
 static __device__ __align__(256) unsigned char scratch[256];
 static_assert(sizeof(Scratch) <= 128 && sizeof(scratch) >= 128 + sizeof(int), "launch record in the first half, flag behind it");
@@ -1533,6 +1574,20 @@ constexpr int kNoAllocMaxDevices = 64;
 struct NoAllocDevice {
   Scratch* ptr = nullptr;  // device address of `scratch` on this device
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  std::atomic<int> busy{0};  // a call is using this device's array
+};
+// One call at a time per device: the array is shared by every call on the device.
+struct NoAllocGuard {
+  NoAllocDevice* d;
+  bool held;
+  explicit NoAllocGuard(NoAllocDevice* dev) : d(dev), held(false) {
+    int expected = 0;
+    held = d->busy.compare_exchange_strong(expected, 1);
+    if (!held) fw_set_error("fw_walk_device_noalloc: another call is running on this device (all calls on a device share "
+                            "one launch record inside the library; run them one after the other)");
+  }
+  bool ok() const { return held; }
+  ~NoAllocGuard() { if (held) d->busy.store(0); }
 };
 NoAllocDevice g_noalloc[kNoAllocMaxDevices];
 std::mutex g_noalloc_lock;
@@ -1571,6 +1626,8 @@ extern "C" int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p
   NoAllocDevice* d = nullptr;
   int rc = noalloc_device(&d);
   if (rc != FW_OK) return rc;
+  NoAllocGuard guard(d);
+  if (!guard.ok()) return FW_ERR_INVALID;
   // (the neighbour-order check of a graph's first node2vec call keeps its flag behind the launch record)
   rc = check_walk_args(g, p, d_starts, n, d_paths, reinterpret_cast<int*>(reinterpret_cast<unsigned char*>(d->ptr) + 128));
   if (rc != FW_OK) return rc;
@@ -1583,8 +1640,7 @@ extern "C" int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p
   const double t0 = now_ms();
   Scratch* const scr = d->ptr;  // the device address; never the array's name
 
-  // the array keeps the last call's contents: the dispenser word and the counters start at zero (fill kernels, not
-  // memset nodes, so that a caller may capture the call's launches)
+  // the array keeps the last call's contents: the dispenser word and the counters start at zero
   hipLaunchKernelGGL(fw_fill_i32_kernel, dim3(1), dim3(64), 0, stream, reinterpret_cast<int32_t*>(scr), 0,
                      sizeof(Scratch) / sizeof(int32_t));
   FW_HIP(hipGetLastError());
@@ -1623,7 +1679,12 @@ extern "C" int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p
     stats->hub_kernel_ms = 0.0;
     stats->hub_steps = 0;
     stats->hub_sampled_edges = 0;
-    stats->requested_bytes = requested_bytes_model(p, n, false, INT_MAX, h.counters[0], h.counters[1], 0, KernelTimes());
+    const TrafficModel tm = traffic_model(p, n, false, INT_MAX, h.counters[0], h.counters[1], 0, KernelTimes());
+    stats->requested_bytes = tm.total();
+    stats->list_bytes = tm.list_bytes;
+    stats->scattered_reads = tm.scattered_reads;
+    stats->scattered_writes = tm.scattered_writes;
+    stats->record_bytes = tm.record_bytes;
   }
   return FW_OK;
 }
@@ -1755,9 +1816,13 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     stats->grid = grid_used;
     stats->walk_kernel_ms = times.hub_ms == 0.0 && times.walk_ms == 0.0 ? kernel_ms : times.walk_ms;
     stats->hub_kernel_ms = times.hub_ms;
-    stats->requested_bytes = requested_bytes_model(p, n, times.hub_ms != 0.0, park_threshold,
-                                                   stats->steps - stats->hub_steps,
-                                                   stats->sampled_edges - stats->hub_sampled_edges, stats->hub_steps, times);
+    const TrafficModel tm = traffic_model(p, n, times.hub_ms != 0.0, park_threshold, stats->steps - stats->hub_steps,
+                                          stats->sampled_edges - stats->hub_sampled_edges, stats->hub_steps, times);
+    stats->requested_bytes = tm.total();
+    stats->list_bytes = tm.list_bytes;
+    stats->scattered_reads = tm.scattered_reads;
+    stats->scattered_writes = tm.scattered_writes;
+    stats->record_bytes = tm.record_bytes;
   }
   return FW_OK;
 }

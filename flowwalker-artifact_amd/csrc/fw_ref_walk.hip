@@ -18,6 +18,18 @@
 // group of W lanes at (walker, step) is word j & 3 of block (j >> 2) * W + t of stream kStreamRef, t = i % W,
 // j = i / W, mapped to (0, 1] as cuRAND's uniforms are (include/myrand.cuh:213-215).  Walks are therefore a function
 // of (seed, walker id, graph, parameters) and can be compared bit for bit with a CPU restatement.
+//
+// Thread-owned generators (FW_SAMPLER_REF_RNG_LDS / _GLOBAL, static assignment only).  The reference's ablation
+// (README.md:152-163) starts from generators that belong to the threads: cuRAND states in device memory, read and
+// written around every draw (walker_wb_dprs_curand, include/walker.cuh:1584-1696, `state + gid`), then its own
+// generator with the states of a block in shared memory, structure of arrays (include/myrand.cuh:83-86, :174-186;
+// walker_wb_dprs, include/walker.cuh:1813).  Both are restated here with one generator: thread `gid` (global thread id,
+// the reference's sequence number, include/myrand.cuh:271-292) draws word n & 3 of Philox block n >> 2 of its own
+// stream (counter (gid, n >> 2, kStreamThread, 0)) as its n-th uniform, whatever list it is working on; the state (the
+// current block and n) lives in LDS or in device memory.  With static assignment every step of the launch is a
+// function of (seed, grid, wg_threads, queries): slots take their queries in slot order, deferred lists are stepped in
+// slot order, so the CPU restatement replays a workgroup thread by thread and the walks compare bit for bit.  Both
+// placements give the same walks; they differ in what a draw costs.
 
 #include "fw_internal.h"
 #include "fw_device_util.h"
@@ -25,6 +37,7 @@
 namespace {
 
 constexpr uint32_t kStreamRef = 0x20000000u;
+constexpr uint32_t kStreamThread = 0x08000000u;   // thread-owned generators: counter (gid, block, kStreamThread, 0)
 constexpr uint32_t kStreamStopRef = 0x80000000u;  // PPR stop draw: the same stream the walk kernel uses
 constexpr int kRefTasks = 64;                      // TASK_NUM, include/walker.cuh:28
 
@@ -90,32 +103,78 @@ __device__ __forceinline__ float ref_bias(const fw_kargs& a, const RefStep& s, u
   return w;
 }
 
-// The uniforms of one lane of a group of W lanes: its j-th element takes word j & 3 of block (j >> 2) * W + t.
+// State of a thread-owned generator in device memory (the place of cuRAND's `state + gid`).
+struct RefThreadState {
+  uint32_t w[4];
+  uint32_t n;
+  uint32_t pad[3];
+};
+
+// Where the calling thread's generator lives (kRng 1: LDS, structure of arrays; 2: device memory).
+struct RefRng {
+  uint32_t* lds_w;  // [4][blockDim.x]
+  uint32_t* lds_n;  // [blockDim.x]
+  RefThreadState* dev;  // this thread's state
+  uint32_t tid, threads, gid;
+};
+
+// kRng 0: the uniforms of one lane of a group of W lanes, its j-th element takes word j & 3 of block (j >> 2) * W + t.
+// kRng 1 / 2: the thread's own generator, its draws one after the other.
+template <int kRng>
 struct RefDraws {
   uint4 blk;
-  __device__ __forceinline__ float next(const fw_kargs& a, const RefStep& s, uint32_t W, uint32_t t, uint32_t j) {
-    if ((j & 3u) == 0u) blk = philox4x32_10(s.walker, s.step, kStreamRef, (j >> 2) * W + t, a.seed_lo, a.seed_hi);
-    const uint32_t k = j & 3u;
-    const uint32_t bits = k == 0u ? blk.x : (k == 1u ? blk.y : (k == 2u ? blk.z : blk.w));
+  __device__ __forceinline__ float next(const fw_kargs& a, const RefStep& s, const RefRng& r, uint32_t W, uint32_t t,
+                                        uint32_t j) {
+    if (kRng == 0) {
+      if ((j & 3u) == 0u) blk = philox4x32_10(s.walker, s.step, kStreamRef, (j >> 2) * W + t, a.seed_lo, a.seed_hi);
+      const uint32_t k = j & 3u;
+      const uint32_t bits = k == 0u ? blk.x : (k == 1u ? blk.y : (k == 2u ? blk.z : blk.w));
+      return ref_u(bits);
+    }
+    uint32_t bits;
+    if (kRng == 1) {
+      const uint32_t n = r.lds_n[r.tid];
+      if ((n & 3u) == 0u) {
+        const uint4 b = philox4x32_10(r.gid, n >> 2, kStreamThread, 0u, a.seed_lo, a.seed_hi);
+        r.lds_w[0u * r.threads + r.tid] = b.x;
+        r.lds_w[1u * r.threads + r.tid] = b.y;
+        r.lds_w[2u * r.threads + r.tid] = b.z;
+        r.lds_w[3u * r.threads + r.tid] = b.w;
+      }
+      bits = r.lds_w[(n & 3u) * r.threads + r.tid];
+      r.lds_n[r.tid] = n + 1u;
+    } else {
+      volatile RefThreadState* st = r.dev;  // every draw goes to memory and back, as a cuRAND state does
+      const uint32_t n = st->n;
+      if ((n & 3u) == 0u) {
+        const uint4 b = philox4x32_10(r.gid, n >> 2, kStreamThread, 0u, a.seed_lo, a.seed_hi);
+        st->w[0] = b.x;
+        st->w[1] = b.y;
+        st->w[2] = b.z;
+        st->w[3] = b.w;
+      }
+      bits = st->w[n & 3u];
+      st->n = n + 1u;
+    }
     return ref_u(bits);
   }
 };
 
 // sampler_warp (include/sampler.cuh:46-85) for a 64-lane wave
-template <int kApp>
-__device__ __forceinline__ int32_t ref_zprs_wave(const fw_kargs& a, const RefStep& s, const int lane) {
+template <int kApp, int kRng>
+__device__ __forceinline__ int32_t ref_zprs_wave(const fw_kargs& a, const RefStep& s, const RefRng& r, const int lane) {
   const uint32_t deg = (uint32_t)s.deg;
   float L = 0.0f;
   for (uint32_t i = (uint32_t)lane; i < deg; i += 64u) L += ref_bias<kApp>(a, s, i);  // :56-59
   const float I = wave_scan(L);                                                       // :62-66
   float S = I - L;                                                                    // :68
   long long key = -1;
-  RefDraws d;
+  RefDraws<kRng> d;
   uint32_t j = 0u;
   for (uint32_t i = (uint32_t)lane; i < deg; i += 64u, ++j) {  // :70-80
     const float w = ref_bias<kApp>(a, s, i);
     S += w;
-    const float u = d.next(a, s, 64u, (uint32_t)lane, j);
+    const float u = d.next(a, s, r, 64u, (uint32_t)lane, j);
     if (w > 0.0f) {
       if (key == -1) key = 0;
       if (u < w / S) key = (long long)i + (long long)deg * (long long)lane;
@@ -126,13 +185,13 @@ __device__ __forceinline__ int32_t ref_zprs_wave(const fw_kargs& a, const RefSte
 }
 
 // sampler_warp_oneloop (include/sampler.cuh:129-155) for a 64-lane wave
-template <int kApp>
-__device__ __forceinline__ int32_t ref_dprs_wave(const fw_kargs& a, const RefStep& s, const int lane) {
+template <int kApp, int kRng>
+__device__ __forceinline__ int32_t ref_dprs_wave(const fw_kargs& a, const RefStep& s, const RefRng& r, const int lane) {
   const uint32_t deg = (uint32_t)s.deg;
   if (deg == 0u) return -1;
   float carry = 0.0f;
   int32_t sel = -1;
-  RefDraws d;
+  RefDraws<kRng> d;
   const uint64_t bound = (uint64_t)deg + 64u - deg % 64u;  // :138
   uint32_t j = 0u;
   for (uint64_t base = 0; base < bound; base += 64u, ++j) {
@@ -140,7 +199,7 @@ __device__ __forceinline__ int32_t ref_dprs_wave(const fw_kargs& a, const RefSte
     const float x = i < deg ? ref_bias<kApp>(a, s, (uint32_t)i) : 0.0f;
     if (x > 0.0f && sel == -1) sel = 0;                        // :142
     const float Sl = carry + wave_scan(x);                     // :143-149
-    const float u = d.next(a, s, 64u, (uint32_t)lane, j);
+    const float u = d.next(a, s, r, 64u, (uint32_t)lane, j);
     if (i < deg && x > 0.0f && u < x / Sl) sel = (int32_t)i;   // :150
     carry = readlane_f(Sl, 63);                                // :151
     sel = wave_max_i32(sel);                                   // :152
@@ -157,9 +216,9 @@ struct RefBlockScratch {
 // sampler_block (include/sampler.cuh:87-127) for a workgroup of W = blockDim.x threads.  The exclusive prefix over the
 // threads' totals is: wave scan inside each wave, the waves' totals added up one after the other, minus the thread's
 // own total (the reference's cub::BlockScan has no documented association).
-template <int kApp>
-__device__ __forceinline__ int32_t ref_zprs_block(const fw_kargs& a, const RefStep& s, RefBlockScratch& scr, const int tid,
-                                                  const int lane, const int wave, const int nw) {
+template <int kApp, int kRng>
+__device__ __forceinline__ int32_t ref_zprs_block(const fw_kargs& a, const RefStep& s, const RefRng& r, RefBlockScratch& scr,
+                                                  const int tid, const int lane, const int wave, const int nw) {
   const uint32_t deg = (uint32_t)s.deg;
   const uint32_t W = (uint32_t)nw * 64u;
   float L = 0.0f;
@@ -171,12 +230,12 @@ __device__ __forceinline__ int32_t ref_zprs_block(const fw_kargs& a, const RefSt
   for (int v = 0; v < wave; ++v) off = off + scr.tot[v];
   float S = (off + I) - L;  // :102-104
   long long key = -1;
-  RefDraws d;
+  RefDraws<kRng> d;
   uint32_t j = 0u;
   for (uint32_t i = (uint32_t)tid; i < deg; i += W, ++j) {  // :106-116
     const float w = ref_bias<kApp>(a, s, i);
     S += w;
-    const float u = d.next(a, s, W, (uint32_t)tid, j);
+    const float u = d.next(a, s, r, W, (uint32_t)tid, j);
     if (w > 0.0f) {
       if (key == -1) key = 0;
       if (u < w / S) key = (long long)i + (long long)deg * (long long)tid;
@@ -192,15 +251,15 @@ __device__ __forceinline__ int32_t ref_zprs_block(const fw_kargs& a, const RefSt
 }
 
 // sampler_block_oneloop (include/sampler.cuh:157-200) for a workgroup of W = blockDim.x threads
-template <int kApp>
-__device__ __forceinline__ int32_t ref_dprs_block(const fw_kargs& a, const RefStep& s, RefBlockScratch& scr, const int tid,
-                                                  const int lane, const int wave, const int nw) {
+template <int kApp, int kRng>
+__device__ __forceinline__ int32_t ref_dprs_block(const fw_kargs& a, const RefStep& s, const RefRng& r, RefBlockScratch& scr,
+                                                  const int tid, const int lane, const int wave, const int nw) {
   const uint32_t deg = (uint32_t)s.deg;
   if (deg == 0u) return -1;
   const uint32_t W = (uint32_t)nw * 64u;
   float carry = 0.0f;  // prefix_sum, :163-164
   int32_t sel = -1;
-  RefDraws d;
+  RefDraws<kRng> d;
   const uint64_t bound = (uint64_t)deg + W - deg % W;  // :167
   uint32_t j = 0u;
   for (uint64_t base = 0; base < bound; base += W, ++j) {
@@ -215,7 +274,7 @@ __device__ __forceinline__ int32_t ref_dprs_block(const fw_kargs& a, const RefSt
     for (int v = 0; v < nw; ++v) next_carry = next_carry + scr.tot[v];  // :194-196
     const float Sl = off + I;
     int32_t local = -1;
-    const float u = d.next(a, s, W, (uint32_t)tid, j);
+    const float u = d.next(a, s, r, W, (uint32_t)tid, j);
     if (x > 0.0f && i < deg) {  // :181-184
       local = 0;
       if (u < x / Sl) local = (int32_t)i;
@@ -233,17 +292,22 @@ __device__ __forceinline__ int32_t ref_dprs_block(const fw_kargs& a, const RefSt
 }
 
 // walker_wb_dynamic_zprs / _dprs (include/walker.cuh:1307-1580) and their statically assigned forms.
-template <int kApp, bool kDprs>
-__global__ __launch_bounds__(1024) void fw_walk_ref(const fw_kargs a, const int static_assignment) {
+// kRng: 0 = every draw addressed by (walker, step, element); 1 / 2 = thread-owned generators with their state in LDS /
+// in device memory (rng_dev, one RefThreadState per thread of the grid), static assignment only.
+template <int kApp, bool kDprs, int kRng>
+__global__ __launch_bounds__(1024) void fw_walk_ref(const fw_kargs a, const int static_assignment, RefThreadState* rng_dev) {
+  static_assert(kRefTasks == 64, "the task slots are claimed and refilled by the lanes of wave 0");
   __shared__ int32_t t_walker[kRefTasks], t_cur[kRefTasks], t_prev[kRefTasks], t_len[kRefTasks], t_deg[kRefTasks];
   __shared__ int32_t t_prev_deg[kRefTasks], t_moved[kRefTasks];
   __shared__ uint32_t t_off[kRefTasks], t_prev_off[kRefTasks];
-  __shared__ int32_t large_tasks[kRefTasks];
-  __shared__ int32_t num_active, block_task_count;
+  __shared__ int32_t is_large[kRefTasks];
+  __shared__ int32_t num_active;
   __shared__ uint32_t s_cursor;
   __shared__ int32_t s_schema[kApp == FW_APP_METAPATH ? FW_MAX_SCHEMA : 1];
   __shared__ RefBlockScratch scr;
   __shared__ unsigned long long s_acc[2];
+  __shared__ uint32_t s_rng_w[kRng == 1 ? 4 * 1024 : 1];  // include/myrand.cuh:83-86: the block's states, structure of arrays
+  __shared__ uint32_t s_rng_n[kRng == 1 ? 1024 : 1];
 
   const int tid = (int)threadIdx.x;
   const int lane = lane_id();
@@ -255,11 +319,24 @@ __global__ __launch_bounds__(1024) void fw_walk_ref(const fw_kargs a, const int 
   const uint32_t lo = blockIdx.x * per < n ? blockIdx.x * per : n;
   const uint32_t hi = lo + per < n ? lo + per : n;
 
+  RefRng rng;
+  rng.lds_w = s_rng_w;
+  rng.lds_n = s_rng_n;
+  rng.tid = (uint32_t)tid;
+  rng.threads = blockDim.x;
+  rng.gid = blockIdx.x * blockDim.x + (uint32_t)tid;
+  rng.dev = kRng == 2 ? rng_dev + rng.gid : nullptr;
+  if (kRng == 1) s_rng_n[tid] = 0u;  // myrand_init (include/myrand.cuh:271-292): sequence = global thread id
+  if (kRng == 2) rng.dev->n = 0u;    // curand_init(1337, gid, 0, state + gid), include/walker.cuh:1597
+
   if (tid == 0) {
     num_active = kRefTasks;
-    block_task_count = 0;
     s_cursor = 0u;
     s_acc[0] = s_acc[1] = 0ull;
+  }
+  if (tid < kRefTasks) {
+    t_len[tid] = -1;
+    is_large[tid] = 0;
   }
   if (kApp == FW_APP_METAPATH && tid == 0) {
 #pragma unroll
@@ -267,19 +344,26 @@ __global__ __launch_bounds__(1024) void fw_walk_ref(const fw_kargs a, const int 
   }
   __syncthreads();
 
-  // next query of this workgroup, or 0xFFFFFFFF (include/walker.cuh:1339, :1423)
-  auto claim = [&]() -> uint32_t {
+  // Wave 0, all lanes: the slots with `want` take the next queries (include/walker.cuh:1339, :1423), in slot order --
+  // the lowest slot gets the lowest query, so that a statically assigned launch is the same every time it runs.
+  // Task::init (include/gpu_task.cuh:52-68), include/walker.cuh:1340-1349.
+  auto refill = [&](bool want) {
+    const uint64_t m = __ballot(want);
+    if (m == 0ull) return;
+    const uint32_t rank = (uint32_t)__builtin_popcountll(m & ((1ull << lane) - 1ull));
+    const uint32_t cnt = (uint32_t)__builtin_popcountll(m);
+    uint32_t base = 0u;
     if (static_assignment) {
-      const uint32_t q = lo + atomicAdd(&s_cursor, 1u);
-      return q < hi ? q : 0xFFFFFFFFu;
+      base = s_cursor;  // only wave 0 touches it
+      if (lane == 0) s_cursor = base + cnt;
+    } else {
+      if (lane == __builtin_ctzll(m)) base = atomicAdd(a.dispenser, cnt);
+      base = (uint32_t)__builtin_amdgcn_readlane((int)base, __builtin_ctzll(m));
     }
-    const uint32_t q = atomicAdd(a.dispenser, 1u);
-    return q < n ? q : 0xFFFFFFFFu;
-  };
-  // Task::init (include/gpu_task.cuh:52-68), include/walker.cuh:1340-1349
-  auto init_slot = [&](int slot) {
-    const uint32_t q = claim();
-    if (q == 0xFFFFFFFFu) {
+    if (!want) return;
+    const uint32_t q = static_assignment ? lo + base + rank : base + rank;
+    const int slot = tid;
+    if (q >= (static_assignment ? hi : n)) {
       t_len[slot] = -1;
       atomicSub(&num_active, 1);
       return;
@@ -303,7 +387,7 @@ __global__ __launch_bounds__(1024) void fw_walk_ref(const fw_kargs a, const int 
       t_len[slot] = a.max_depth;
     }
   };
-  if (tid < kRefTasks) init_slot(tid);
+  if (wave == 0) refill(true);
   __syncthreads();
 
   unsigned long long n_steps = 0ull, n_edges = 0ull;
@@ -347,36 +431,37 @@ __global__ __launch_bounds__(1024) void fw_walk_ref(const fw_kargs a, const int 
       if (t_len[slot] < 0 || t_len[slot] >= a.max_depth) continue;
       const RefStep s = load_step(slot);
       if (s.deg <= a.hub_threshold) {  // :1362
-        const int32_t sel = kDprs ? ref_dprs_wave<kApp>(a, s, lane) : ref_zprs_wave<kApp>(a, s, lane);
+        const int32_t sel = kDprs ? ref_dprs_wave<kApp, kRng>(a, s, rng, lane) : ref_zprs_wave<kApp, kRng>(a, s, rng, lane);
         if (lane == 0) commit(slot, s, sel);
       } else if (lane == 0) {
-        large_tasks[atomicAdd(&block_task_count, 1)] = slot;  // :1386-1391
+        is_large[slot] = 1;  // :1386-1391 (a flag per slot instead of a list: the deferred lists are stepped in slot order)
       }
     }
     __syncthreads();  // :1395
-    const int nl = block_task_count;
-    for (int k = 0; k < nl; ++k) {  // :1397-1419
-      const int slot = large_tasks[k];
+    for (int slot = 0; slot < kRefTasks; ++slot) {  // :1397-1419
+      if (is_large[slot] == 0) continue;  // uniform in the workgroup
       const RefStep s = load_step(slot);
-      const int32_t sel = kDprs ? ref_dprs_block<kApp>(a, s, scr, tid, lane, wave, nw)
-                                : ref_zprs_block<kApp>(a, s, scr, tid, lane, wave, nw);
+      const int32_t sel = kDprs ? ref_dprs_block<kApp, kRng>(a, s, rng, scr, tid, lane, wave, nw)
+                                : ref_zprs_block<kApp, kRng>(a, s, rng, scr, tid, lane, wave, nw);
       if (tid == 0) commit(slot, s, sel);
     }
     __syncthreads();
-    if (tid < kRefTasks && t_len[tid] >= 0) {  // :1422-1432, on live slots only
-      const int32_t len = t_len[tid];
-      bool stop = len >= a.max_depth || t_deg[tid] == 0;
-      if (kApp == FW_APP_PPR && !stop && t_moved[tid]) {  // include/app.cuh:88-94: one draw per completed step
-        const uint32_t w = a.walker_base + (uint32_t)t_walker[tid];
-        const uint32_t bits = philox4x32_10(w, (uint32_t)(len - 2), kStreamStopRef, 0u, a.seed_lo, a.seed_hi).x;
-        stop = u24(bits) < a.tp;
+    if (wave == 0) {  // :1422-1432, on live slots only
+      bool stop = false;
+      if (t_len[tid] >= 0) {
+        const int32_t len = t_len[tid];
+        stop = len >= a.max_depth || t_deg[tid] == 0;
+        if (kApp == FW_APP_PPR && !stop && t_moved[tid]) {  // include/app.cuh:88-94: one draw per completed step
+          const uint32_t w = a.walker_base + (uint32_t)t_walker[tid];
+          const uint32_t bits = philox4x32_10(w, (uint32_t)(len - 2), kStreamStopRef, 0u, a.seed_lo, a.seed_hi).x;
+          stop = u24(bits) < a.tp;
+        }
+        t_moved[tid] = 0;
       }
-      t_moved[tid] = 0;
-      if (stop) init_slot(tid);
+      is_large[tid] = 0;
+      refill(stop);
     }
     __syncthreads();  // :1433-1437
-    if (tid == 0) block_task_count = 0;
-    __syncthreads();
   }
 
   if (n_steps != 0ull) {
@@ -390,7 +475,9 @@ __global__ __launch_bounds__(1024) void fw_walk_ref(const fw_kargs a, const int 
   }
 }
 
-template <int kApp, bool kDprs>
+// Workgroups of a launch of the reference's engine: `grid` when given, else twice the resident set (src/walk.cu:84-92),
+// never more than there are groups of kRefTasks queries.
+template <int kApp, bool kDprs, int kRng>
 int launch_ref(const fw_kargs& a, int wg_threads, int grid, int static_assignment, hipStream_t stream, int* grid_used) {
   if (wg_threads != 256 && wg_threads != 512 && wg_threads != 1024) {
     fw_set_error("wg_threads must be 256, 512 or 1024 (got %d)", wg_threads);
@@ -400,22 +487,39 @@ int launch_ref(const fw_kargs& a, int wg_threads, int grid, int static_assignmen
     int dev = 0, cus = 0, per_cu = 0;
     FW_HIP(hipGetDevice(&dev));
     FW_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    FW_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fw_walk_ref<kApp, kDprs>, wg_threads, 0));
-    grid = cus * (per_cu > 0 ? per_cu : 1) * 2;  // twice the resident set, as src/walk.cu:84-92 launches it
+    FW_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fw_walk_ref<kApp, kDprs, kRng>, wg_threads, 0));
+    grid = cus * (per_cu > 0 ? per_cu : 1) * 2;
   }
   const int needed = (a.n + kRefTasks - 1) / kRefTasks;
   if (grid > needed) grid = needed;
-  hipLaunchKernelGGL((fw_walk_ref<kApp, kDprs>), dim3(grid), dim3(wg_threads), 0, stream, a, static_assignment);
-  FW_HIP(hipGetLastError());
+  RefThreadState* rng_dev = nullptr;
+  if (kRng == 2) FW_HIP(hipMalloc(reinterpret_cast<void**>(&rng_dev), (size_t)grid * (size_t)wg_threads * sizeof(RefThreadState)));
+  hipLaunchKernelGGL((fw_walk_ref<kApp, kDprs, kRng>), dim3(grid), dim3(wg_threads), 0, stream, a, static_assignment, rng_dev);
+  int rc = fw_check_hip(hipGetLastError(), "fw_walk_ref", __FILE__, __LINE__);
+  if (kRng == 2) {  // the states are the launch's own: wait for it and give them back
+    if (rc == FW_OK) rc = fw_check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize", __FILE__, __LINE__);
+    (void)hipFree(rng_dev);
+  }
+  if (rc != FW_OK) return rc;
   if (grid_used) *grid_used = grid;
   return FW_OK;
 }
 
-template <int kApp>
-int launch_ref_app(const fw_kargs& a, bool dprs, int wg_threads, int grid, int static_assignment, hipStream_t stream,
+template <int kApp, int kRng>
+int launch_ref_rng(const fw_kargs& a, bool dprs, int wg_threads, int grid, int static_assignment, hipStream_t stream,
                    int* grid_used) {
-  return dprs ? launch_ref<kApp, true>(a, wg_threads, grid, static_assignment, stream, grid_used)
-              : launch_ref<kApp, false>(a, wg_threads, grid, static_assignment, stream, grid_used);
+  return dprs ? launch_ref<kApp, true, kRng>(a, wg_threads, grid, static_assignment, stream, grid_used)
+              : launch_ref<kApp, false, kRng>(a, wg_threads, grid, static_assignment, stream, grid_used);
+}
+
+template <int kApp>
+int launch_ref_app(const fw_kargs& a, bool dprs, int rng, int wg_threads, int grid, int static_assignment, hipStream_t stream,
+                   int* grid_used) {
+  switch (rng) {
+    case 0: return launch_ref_rng<kApp, 0>(a, dprs, wg_threads, grid, static_assignment, stream, grid_used);
+    case 1: return launch_ref_rng<kApp, 1>(a, dprs, wg_threads, grid, static_assignment, stream, grid_used);
+    default: return launch_ref_rng<kApp, 2>(a, dprs, wg_threads, grid, static_assignment, stream, grid_used);
+  }
 }
 
 }  // namespace
@@ -424,11 +528,21 @@ int fw_launch_ref_walk(const fw_kargs& a, int app, int sampler, int wg_threads, 
                        int* grid_used) {
   const bool dprs = (sampler & 0xFF) == FW_SAMPLER_REF_DPRS;
   const int static_assignment = (sampler & FW_SAMPLER_REF_STATIC) ? 1 : 0;
+  const int rng = (sampler & FW_SAMPLER_REF_RNG_LDS) ? 1 : ((sampler & FW_SAMPLER_REF_RNG_GLOBAL) ? 2 : 0);
+  if ((sampler & FW_SAMPLER_REF_RNG_LDS) && (sampler & FW_SAMPLER_REF_RNG_GLOBAL)) {
+    fw_set_error("FW_SAMPLER_REF_RNG_LDS and FW_SAMPLER_REF_RNG_GLOBAL exclude each other");
+    return FW_ERR_INVALID;
+  }
+  if (rng != 0 && !static_assignment) {
+    fw_set_error("thread-owned generators (FW_SAMPLER_REF_RNG_*) need FW_SAMPLER_REF_STATIC: with the global query "
+                 "dispenser the thread that serves a query changes from run to run");
+    return FW_ERR_INVALID;
+  }
   switch (app) {
-    case FW_APP_DEEPWALK: return launch_ref_app<FW_APP_DEEPWALK>(a, dprs, wg_threads, grid, static_assignment, stream, grid_used);
-    case FW_APP_PPR: return launch_ref_app<FW_APP_PPR>(a, dprs, wg_threads, grid, static_assignment, stream, grid_used);
-    case FW_APP_NODE2VEC: return launch_ref_app<FW_APP_NODE2VEC>(a, dprs, wg_threads, grid, static_assignment, stream, grid_used);
-    case FW_APP_METAPATH: return launch_ref_app<FW_APP_METAPATH>(a, dprs, wg_threads, grid, static_assignment, stream, grid_used);
+    case FW_APP_DEEPWALK: return launch_ref_app<FW_APP_DEEPWALK>(a, dprs, rng, wg_threads, grid, static_assignment, stream, grid_used);
+    case FW_APP_PPR: return launch_ref_app<FW_APP_PPR>(a, dprs, rng, wg_threads, grid, static_assignment, stream, grid_used);
+    case FW_APP_NODE2VEC: return launch_ref_app<FW_APP_NODE2VEC>(a, dprs, rng, wg_threads, grid, static_assignment, stream, grid_used);
+    case FW_APP_METAPATH: return launch_ref_app<FW_APP_METAPATH>(a, dprs, rng, wg_threads, grid, static_assignment, stream, grid_used);
     default:
       fw_set_error("unknown app %d", app);
       return FW_ERR_INVALID;

@@ -2058,7 +2058,8 @@ int fw_launch_walk(const fw_kargs& a, int app, int sampler, int wg_threads, int 
                    hipStream_t stream, int* grid_used) {
   // FW_SAMPLER_DPRS is an alias: the one sampler already evaluates every bias exactly once, which is
   // what the reference's DPRS kernel (include/walker.cuh:1444) exists for.
-  if ((sampler & ~FW_SAMPLER_REF_STATIC) == FW_SAMPLER_REF_ZPRS || (sampler & ~FW_SAMPLER_REF_STATIC) == FW_SAMPLER_REF_DPRS)
+  constexpr int kRefFlags = FW_SAMPLER_REF_STATIC | FW_SAMPLER_REF_RNG_LDS | FW_SAMPLER_REF_RNG_GLOBAL;
+  if ((sampler & ~kRefFlags) == FW_SAMPLER_REF_ZPRS || (sampler & ~kRefFlags) == FW_SAMPLER_REF_DPRS)
     return fw_launch_ref_walk(a, app, sampler, wg_threads, grid, stream, grid_used);
   if (sampler != FW_SAMPLER_ZPRS && sampler != FW_SAMPLER_DPRS) {
     fw_set_error("unknown sampler %d", sampler);

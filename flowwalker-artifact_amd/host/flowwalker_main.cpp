@@ -16,10 +16,14 @@
 // include/gpu_graph.cuh:46-54).  --walkmode keeps the reference's ablation levels (README.md:152-163), run by the
 // reference's own algorithms restated for 64-lane waves (FW_SAMPLER_REF_*: two-pass ZPRS / chunked DPRS, 64 task
 // slots per workgroup), and adds this engine's own levels:
-//   --walkmode=9 / 10  "FW" / "FW + RNG": the reference's DPRS samplers, static query assignment (the counter-based
-//                      RNG has one form, so 9 and 10 are the same)
-//   --walkmode=1       "FW + ZPRS": the reference's ZPRS samplers, static query assignment
-//   --walkmode=6       "FW + DS": the reference's ZPRS samplers with the global query dispenser (its default kernel)
+//   --walkmode=9       "FW": the reference's DPRS samplers, static query assignment, generators that belong to the threads
+//                      with their state in device memory (cuRAND's place: walker_wb_dprs_curand, include/walker.cuh:1584)
+//   --walkmode=10      "FW + RNG": the same with the generators' state in LDS, structure of arrays (include/myrand.cuh:83-86;
+//                      walker_wb_dprs, include/walker.cuh:1813): the same walks as 9, cheaper draws
+//   --walkmode=1       "FW + ZPRS": the reference's ZPRS samplers, static query assignment, generators in LDS (walker_wb, :172)
+//   --walkmode=6       "FW + DS": the reference's ZPRS samplers with the global query dispenser (its default kernel, :1307);
+//                      draws addressed by (walker, step, element), because a generator owned by a thread gives other
+//                      walks on every run once the queries are handed out dynamically
 //   --walkmode=20      this engine's walk kernel alone, every list sampled by one wave (no workgroup sampler, no parking)
 //   --walkmode=21      + the workgroup sampler for lists above --hub_threshold
 //   --walkmode=22      + parking: walkers waiting on the same vertex share one scan of its list (the default)
@@ -332,10 +336,14 @@ int main(int argc, char** argv) {
   } else if (F.walkmode >= 0) {  // the reference's levels (README.md:152-163), its algorithms on 64-lane waves
     const bool dprs = F.walkmode == 9 || F.walkmode == 10;
     const bool is_static = F.walkmode != 6;
-    P.sampler = (dprs ? FW_SAMPLER_REF_DPRS : FW_SAMPLER_REF_ZPRS) | (is_static ? FW_SAMPLER_REF_STATIC : 0);
+    const int rng = F.walkmode == 9 ? FW_SAMPLER_REF_RNG_GLOBAL : (is_static ? FW_SAMPLER_REF_RNG_LDS : 0);
+    P.sampler = (dprs ? FW_SAMPLER_REF_DPRS : FW_SAMPLER_REF_ZPRS) | (is_static ? FW_SAMPLER_REF_STATIC : 0) | rng;
     if (F.hub_threshold < 0) P.hub_threshold = 1024;  // THRESHOLD, include/walker.cuh:29
-    printf("ablation level %d: the reference's %s samplers on 64-lane waves, %s\n", F.walkmode, dprs ? "DPRS" : "ZPRS",
-           is_static ? "static query assignment" : "global query dispenser");
+    printf("ablation level %d: the reference's %s samplers on 64-lane waves, %s, %s\n", F.walkmode, dprs ? "DPRS" : "ZPRS",
+           is_static ? "static query assignment" : "global query dispenser",
+           rng == FW_SAMPLER_REF_RNG_GLOBAL ? "thread-owned generators in device memory"
+           : rng == FW_SAMPLER_REF_RNG_LDS  ? "thread-owned generators in LDS"
+                                            : "draws addressed by walker, step and element");
   }
 
   // ---- walk (src/main.cu:346-357) ----

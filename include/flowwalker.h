@@ -48,13 +48,23 @@ typedef enum { FW_APP_DEEPWALK = 0, FW_APP_PPR = 1, FW_APP_NODE2VEC = 2, FW_APP_
  * README.md:152-163 and the columns of the sampler micro-benchmark; same sampling law, their own random streams, no
  * parking.  OR FW_SAMPLER_REF_STATIC into either for the reference's static query assignment (src/walk.cu:46-61)
  * instead of the global dispenser.
+ * With FW_SAMPLER_REF_STATIC, OR in FW_SAMPLER_REF_RNG_GLOBAL or FW_SAMPLER_REF_RNG_LDS for generators that belong to
+ * the threads, as the reference's do, instead of draws addressed by (walker, step, element): thread `gid` takes its
+ * uniforms one after the other from its own stream, with the generator's state in device memory, read and written
+ * around every draw (cuRAND states, walker_wb_dprs_curand, include/walker.cuh:1584-1696: the "FW" level of
+ * README.md:152-163), or in LDS as a structure of arrays (include/myrand.cuh:83-86, :174-186: the "+ RNG" level).  The
+ * walks are then a function of (seed, queries, grid, wg_threads) -- the same for both placements -- and the law is
+ * unchanged.  FW_ERR_INVALID without FW_SAMPLER_REF_STATIC (with the dispenser the thread that serves a query changes
+ * from run to run).
  */
 typedef enum {
   FW_SAMPLER_ZPRS = 0,
   FW_SAMPLER_DPRS = 1,
   FW_SAMPLER_REF_ZPRS = 2,
   FW_SAMPLER_REF_DPRS = 3,
-  FW_SAMPLER_REF_STATIC = 0x100
+  FW_SAMPLER_REF_STATIC = 0x100,
+  FW_SAMPLER_REF_RNG_LDS = 0x200,
+  FW_SAMPLER_REF_RNG_GLOBAL = 0x400
 } fw_sampler;
 
 /*
@@ -96,13 +106,20 @@ typedef struct {
   double hub_kernel_ms;       /* sum over the hub launches of every round: fw_hub_scan, fw_hub_batch, fw_hub_quad */
   uint64_t hub_steps;         /* steps taken in the hub launches (included in steps) */
   uint64_t hub_sampled_edges; /* their source degrees (included in sampled_edges) */
-  /* Bytes the call's kernels requested from the memory system, from the run's own counters: every list pass in
-   * 16-byte quartets (a list is read once per walker step by the walk kernel, once per batch of up to 64 walkers
-   * or once per round by the hub kernels), 64 bytes for every scattered access (path entry, xadj pair, parking
-   * index, bucket counter, selected neighbour), 16 bytes per walker record moved, node2vec: 16 lines per step for
-   * the binary search of its acceptance test.  What sits between the algorithmic bytes of src/main.cu:93-111
-   * (4 * sampled_edges + ...) and what the HBM counters of a profiler see. */
+  /* What the call's kernels asked of the memory, MODELLED from the run's own counters (steps, records moved, list
+   * quartets streamed): requested_bytes = list_bytes + 128 * scattered_reads + 32 * scattered_writes + record_bytes.
+   * list_bytes: every list pass in 16-byte quartets (a list is read once per walker step by the walk kernel, once per
+   * batch of up to 64 walkers or once per call by the hub kernels); scattered_reads: reads of one 128-byte block each
+   * (CSR offset pair, parking index, selected neighbour; node2vec: 8 per step for the search of its acceptance test);
+   * scattered_writes: stores of one 32-byte write request each (path entry, scattered record); record_bytes: walker
+   * records, tasks and bucket tables that are streamed.  Tables that stay in the L2 are not priced.  This sits
+   * between the algorithmic bytes of src/main.cu:93-111 (4 * sampled_edges + ...) and what a profiler's HBM counters
+   * see; it is an estimate, the counters are the measurement. */
   uint64_t requested_bytes;
+  uint64_t list_bytes;
+  uint64_t scattered_reads;
+  uint64_t scattered_writes;
+  uint64_t record_bytes;
 } fw_walk_stats;
 
 typedef struct fw_graph fw_graph; /* device CSR mirror: include/gpu_graph.cuh:28-78 */
@@ -145,10 +162,12 @@ int fw_dev_fill_i32(int32_t* d_dst, int32_t value, size_t count);
 int fw_dev_copy(void* d_dst, const void* d_src, size_t bytes);
 int fw_dev_sync(void);
 /*
- * Calibration, no counterpart in the reference: scattered accesses per second over d_buf (at least 1 MiB, 64-byte
+ * Calibration, no counterpart in the reference: scattered accesses per second over d_buf (at least 1 MiB, 128-byte
  * aligned and sized).  mode 0: 4-byte reads of pseudo-random 64-byte lines; 1 / 2 / 3: 4- / 8- / 16-byte stores into
- * them (a store that does not cover its line costs the memory a read-modify-write).  bench.py reports these next to
- * the walk pipeline's own transaction rate.
+ * them (a store that does not cover its line costs the memory a read-modify-write); 4 / 5: pairs of 4-byte reads, from
+ * the two 64-byte halves of one random 128-byte block / from two random blocks, loads per second (the two rates tell
+ * whether the memory is asked for 64 or for 128 bytes at a time).  bench.py reports these next to the walk pipeline's
+ * own transaction rate.
  */
 int fw_dev_random_access_rate(void* d_buf, size_t bytes, int mode, double* accesses_per_s);
 
@@ -189,7 +208,7 @@ int fw_graph_destroy(fw_graph* g);
 /* V, E and the maximum degree / its vertex (graph::print_max_degree, include/graph.cuh:209-220). */
 int fw_graph_info(const fw_graph* g, int32_t* V, uint64_t* E, int32_t* max_degree, int32_t* max_degree_vertex);
 
-/* 1 when every neighbour list is strictly ascending (needed by node2vec: include/gpu_graph.cuh:97-118; the walk
+/* 1 when every neighbour list is ascending (equal neighbours allowed; needed by node2vec: include/gpu_graph.cuh:97-118; the walk
  * entry points return FW_ERR_INVALID for FW_APP_NODE2VEC on a graph where this is 0). */
 int fw_graph_is_sorted(const fw_graph* g, int* sorted);
 
@@ -241,17 +260,19 @@ int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const int32_t* d_
                    int32_t* d_paths, void* stream, fw_walk_stats* stats);
 
 /*
- * fw_walk_device for callers that cannot allocate device memory: code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (walk_test allocates on every
+ * fw_walk_device for callers that cannot allocate device memory: tight serving loops that must not touch the allocator,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference (walk_test allocates on every
  * call, src/walk.cu:535-536).  Same arguments, same walks and same counters as fw_walk_device with
  * park_threshold < 0 (one launch, walkers run their whole walks; parking never changes results, so the paths also
  * equal fw_walk_device's under any park_threshold).  The launch scratch (query dispenser word and workload
  * counters, 48 bytes) lives in a 256-byte array inside the library's device image, one copy per device, held
  * until the process ends; the call makes no hipMalloc / hipFree / event creation after its first call on a
- * device.  n is limited to FW_WALK_NOALLOC_MAX_QUERIES, the largest batch fw_walk_device itself serves with a
- * single launch under its default rule (larger batches are what its parking pipeline and the lists it allocates
- * are for): FW_ERR_INVALID beyond it.  All calls on one device share the array, so calls that overlap on one
- * device (two host threads, two streams) race; calls one after the other are independent.
+ * device.  Like fw_walk_device it is synchronous (it waits for its launch and copies the counters back), so it cannot
+ * be recorded into a HIP graph.  n is limited to FW_WALK_NOALLOC_MAX_QUERIES, the largest batch fw_walk_device itself
+ * serves with a single launch under its default rule (larger batches are what its parking pipeline and the lists it
+ * allocates are for): FW_ERR_INVALID beyond it.  All calls on one device share the array: a call made while another
+ * one is running on the same device (two host threads) returns FW_ERR_INVALID; calls one after the other are
+ * independent.
  */
 #define FW_WALK_NOALLOC_MAX_QUERIES 65535
 int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p, const int32_t* d_starts, int32_t n,

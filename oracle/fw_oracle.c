@@ -472,6 +472,176 @@ int fw_oracle_num_threads(void) {
 #endif
 }
 
+/* ---- the reference's engine with thread-owned generators, replayed thread by thread -------------------------------
+ *
+ * FW_SAMPLER_REF_ZPRS / _DPRS with static query assignment and FW_SAMPLER_REF_RNG_LDS / _GLOBAL (the "FW" and "+ RNG"
+ * levels of the reference's ablation, README.md:152-163): the generators belong to the threads, as the reference's do
+ * (include/myrand.cuh:271-292: sequence = global thread id; walker_wb_dprs_curand, include/walker.cuh:1584-1696), so a
+ * walk is no longer a function of the walker alone.  With static assignment it is still a function of the launch:
+ *   - workgroup b of `grid` owns queries [b * per, (b + 1) * per), per = ceil(n / grid) (src/walk.cu:46-61), and
+ *     grid is cut to ceil(n / 64) workgroups; it has 64 task slots (TASK_NUM, include/walker.cuh:28) and
+ *     W = wg_threads threads in W / 64 waves;
+ *   - slots take the next queries in slot order (at the start, and after a round for the slots whose walk ended);
+ *   - a round (include/walker.cuh:1357-1438): wave v steps slots v, v + W/64, ... whose degree is at most
+ *     hub_threshold with the wave sampler (its 64 threads draw), then the deferred slots are stepped in slot order by
+ *     the workgroup sampler (all W threads draw), then the stop rule (PPR's stop draw is addressed by the walker:
+ *     stream FW_STREAM_STOP);
+ *   - thread gid = b * W + t takes as its k-th uniform word k & 3 of Philox block (gid, k >> 2, 0x08000000, 0),
+ *     mapped to (0, 1]; a DPRS step costs every thread of the group one draw per chunk (also the lanes past the end
+ *     of the list, include/sampler.cuh:139-152), a ZPRS step one draw per element the thread owns.
+ * The samplers themselves are fw_ref64_zprs / fw_ref64_dprs, fed with these uniforms.
+ */
+typedef struct {
+  uint64_t seed;
+  uint32_t gid0;     /* global id of the workgroup's thread 0 */
+  uint32_t* count;   /* [W] draws taken so far by each thread */
+} thread_rngs;
+
+static float thread_draw(thread_rngs* r, uint32_t t) {
+  const uint32_t k = r->count[t]++;
+  const uint32_t ctr[4] = {r->gid0 + t, k >> 2, 0x08000000u, 0u};
+  const uint32_t key[2] = {(uint32_t)r->seed, (uint32_t)(r->seed >> 32)};
+  uint32_t out[4];
+  fw_oracle_philox4x32_10(ctr, key, out);
+  return (float)((out[k & 3] >> 8) + 1u) * 0x1p-24f;
+}
+
+/* One step of slot state (cur, prev) at `step` by the threads t0 .. t0 + W - 1 of the workgroup. */
+static int32_t thread_rng_step(const fw_oracle_graph* g, const fw_oracle_params* p, int32_t cur, int32_t prev,
+                               uint32_t step, thread_rngs* r, uint32_t t0, int32_t W) {
+  bias_ctx c;
+  c.g = g; c.p = p; c.prev = prev;
+  c.prev_off = 0; c.prev_deg = 0;
+  c.force = 0; c.cache = NULL; c.cache_groups = 0;
+  c.n2v_full = 1; c.stream_base = 0;
+  if (prev >= 0) { c.prev_off = g->xadj[prev]; c.prev_deg = (int32_t)(g->xadj[prev + 1] - g->xadj[prev]); }
+  c.want_label = (p->app == FW_APP_METAPATH && p->schema_len > 0) ? p->schema[step % (uint32_t)p->schema_len] : 0;
+  const uint32_t off = g->xadj[cur];
+  const int32_t deg = (int32_t)(g->xadj[cur + 1] - off);
+  if (deg <= 0) return -1;
+  float* w = (float*)malloc(sizeof(float) * (size_t)deg);
+  float* u = (float*)malloc(sizeof(float) * (size_t)deg);
+  for (int32_t i = 0; i < deg; ++i) w[i] = bias_at(&c, (uint64_t)off + (uint32_t)i);
+  int32_t sel;
+  if ((p->sampler & 0xFF) == FW_SAMPLER_REF_DPRS) {
+    const int64_t bound = (int64_t)deg + W - deg % W; /* include/sampler.cuh:138, :167 */
+    for (int64_t base = 0; base < bound; base += W)
+      for (int32_t l = 0; l < W; ++l) {
+        const float d = thread_draw(r, t0 + (uint32_t)l);
+        if (base + l < deg) u[base + l] = d;
+      }
+    sel = fw_ref64_dprs(w, deg, W, u);
+  } else {
+    for (int32_t l = 0; l < W; ++l)
+      for (int64_t i = l; i < deg; i += W) u[i] = thread_draw(r, t0 + (uint32_t)l);
+    sel = fw_ref64_zprs(w, deg, W, u);
+  }
+  free(w);
+  free(u);
+  return sel;
+}
+
+int fw_oracle_walk_ref_threads(const fw_oracle_graph* g, const fw_oracle_params* p, const int32_t* starts, int64_t n,
+                               int32_t grid, int32_t* paths, uint64_t* steps_out, uint64_t* edges_out) {
+  enum { SLOTS = 64 };
+  const int32_t W = p->wg_threads;
+  const int kind = p->sampler & 0xFF;
+  if (W % FW_WAVE != 0 || W > FW_MAX_GROUP || W < FW_WAVE || grid < 1 || n < 1) return -1;
+  if (kind != FW_SAMPLER_REF_ZPRS && kind != FW_SAMPLER_REF_DPRS) return -1;
+  const int64_t needed = (n + SLOTS - 1) / SLOTS;
+  if (grid > needed) grid = (int32_t)needed;
+  const int md = p->max_depth;
+  const int nw = W / FW_WAVE;
+  const int64_t per = (n + grid - 1) / grid;
+  uint64_t steps = 0, edges = 0;
+  for (int64_t i = 0; i < n * (int64_t)md; ++i) paths[i] = -1;
+#pragma omp parallel for schedule(dynamic, 1) reduction(+ : steps, edges)
+  for (int32_t b = 0; b < grid; ++b) {
+    const int64_t lo = (int64_t)b * per < n ? (int64_t)b * per : n;
+    const int64_t hi = lo + per < n ? lo + per : n;
+    int64_t cursor = lo;
+    thread_rngs r;
+    r.seed = p->seed;
+    r.gid0 = (uint32_t)b * (uint32_t)W;
+    r.count = (uint32_t*)calloc((size_t)W, sizeof(uint32_t));
+    int64_t q_of[SLOTS];
+    int32_t cur[SLOTS], prev[SLOTS], len[SLOTS], moved[SLOTS];
+    int large[SLOTS];
+    int active = 0;
+    for (int s = 0; s < SLOTS; ++s) { len[s] = -1; large[s] = 0; }
+    /* Task::init (include/gpu_task.cuh:52-68) */
+#define FW_TAKE_QUERY(s)                                                   \
+    do {                                                                   \
+      if (cursor < hi) {                                                   \
+        const int64_t q = cursor++;                                        \
+        q_of[s] = q;                                                       \
+        cur[s] = starts[q];                                                \
+        prev[s] = -1;                                                      \
+        moved[s] = 0;                                                      \
+        paths[q * md] = starts[q];                                         \
+        len[s] = (starts[q] >= 0 && starts[q] < g->V) ? 1 : md;            \
+        ++active;                                                          \
+      } else {                                                             \
+        len[s] = -1;                                                       \
+      }                                                                    \
+    } while (0)
+    for (int s = 0; s < SLOTS; ++s) FW_TAKE_QUERY(s);
+    while (active > 0) {
+      for (int pass = 0; pass < 2; ++pass) {
+        /* pass 0: the waves step their slots (wave v: slots v, v + nw, ... in this order; the waves do not share
+         * threads, so their order among each other does not matter); pass 1: the deferred slots, by the workgroup */
+        for (int v = 0; v < (pass == 0 ? nw : 1); ++v)
+          for (int s = (pass == 0 ? v : 0); s < SLOTS; s += (pass == 0 ? nw : 1)) {
+            if (pass == 0) {
+              if (len[s] < 0 || len[s] >= md) continue;
+              const int32_t deg = (int32_t)(g->xadj[cur[s] + 1] - g->xadj[cur[s]]);
+              if (deg > p->hub_threshold) { large[s] = 1; continue; }
+            } else {
+              if (!large[s]) continue;
+            }
+            const uint32_t off = g->xadj[cur[s]];
+            const int32_t deg = (int32_t)(g->xadj[cur[s] + 1] - off);
+            const int32_t sel = pass == 0
+                ? thread_rng_step(g, p, cur[s], prev[s], (uint32_t)(len[s] - 1), &r, (uint32_t)v * FW_WAVE, FW_WAVE)
+                : thread_rng_step(g, p, cur[s], prev[s], (uint32_t)(len[s] - 1), &r, 0u, W);
+            if (sel < 0) { /* include/walker.cuh:1373-1374 */
+              len[s] = md;
+              moved[s] = 0;
+              continue;
+            }
+            const int32_t nv = g->adjncy[(uint64_t)off + (uint32_t)sel];
+            paths[q_of[s] * md + len[s]] = nv;
+            prev[s] = cur[s];
+            cur[s] = nv;
+            len[s] += 1;
+            moved[s] = 1;
+            steps += 1;
+            edges += (uint64_t)deg;
+          }
+      }
+      for (int s = 0; s < SLOTS; ++s) { /* include/walker.cuh:1422-1432, on live slots only */
+        large[s] = 0;
+        if (len[s] < 0) continue;
+        int stop = len[s] >= md || g->xadj[cur[s] + 1] == g->xadj[cur[s]];
+        if (p->app == FW_APP_PPR && !stop && moved[s]) { /* include/app.cuh:88-94 */
+          const uint32_t walker = p->walker_base + (uint32_t)q_of[s];
+          stop = u24(draw_bits(p->seed, walker, (uint32_t)(len[s] - 2), FW_STREAM_STOP, 0u)) < p->tp;
+        }
+        moved[s] = 0;
+        if (stop) {
+          --active;
+          FW_TAKE_QUERY(s);
+        }
+      }
+    }
+#undef FW_TAKE_QUERY
+    free(r.count);
+  }
+  if (steps_out) *steps_out = steps;
+  if (edges_out) *edges_out = edges;
+  return 0;
+}
+
 /* ---- sequential ground truth (include/sampler.cuh:26-44), for brute-force equivalence tests -- */
 
 /*

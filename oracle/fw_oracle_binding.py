@@ -50,6 +50,9 @@ def lib():
                                      C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.c_int]
         L.fw_oracle_walk.restype = C.c_int
         L.fw_oracle_num_threads.restype = C.c_int
+        L.fw_oracle_walk_ref_threads.argtypes = [C.POINTER(OracleGraph), C.POINTER(OracleParams), C.c_void_p, C.c_int64,
+                                                 C.c_int32, C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
+        L.fw_oracle_walk_ref_threads.restype = C.c_int
         L.fw_oracle_enumerate_draw.argtypes = [C.c_void_p, C.c_int32, C.c_uint32, C.c_int32, C.c_uint32, C.c_uint32,
                                                C.c_uint64, C.c_uint32, C.c_uint32, C.c_void_p]
         L.fw_oracle_sample_forced.argtypes = [C.c_void_p, C.c_int32, C.c_uint32, C.c_int32, C.c_uint32, C.c_uint32,
@@ -140,6 +143,20 @@ def walk(graph, params, starts, nthreads=0):
     steps, edges = C.c_uint64(), C.c_uint64()
     rc = lib().fw_oracle_walk(C.byref(graph.c), C.byref(params), starts.ctypes.data_as(C.c_void_p), n,
                               paths.ctypes.data_as(C.c_void_p), C.byref(steps), C.byref(edges), nthreads)
+    assert rc == 0, "oracle rejected the parameters"
+    return paths, steps.value, edges.value
+
+
+def walk_ref_threads(graph, params, starts, grid):
+    """The reference's engine with thread-owned generators and static assignment (FW_SAMPLER_REF_ZPRS / _DPRS |
+    FW_SAMPLER_REF_STATIC | FW_SAMPLER_REF_RNG_LDS or _GLOBAL), replayed thread by thread for a launch of `grid`
+    workgroups of params.wg_threads."""
+    starts = np.ascontiguousarray(starts, dtype=np.int32)
+    n = len(starts)
+    paths = np.empty((n, params.max_depth), dtype=np.int32)
+    steps, edges = C.c_uint64(), C.c_uint64()
+    rc = lib().fw_oracle_walk_ref_threads(C.byref(graph.c), C.byref(params), starts.ctypes.data_as(C.c_void_p), n,
+                                          int(grid), paths.ctypes.data_as(C.c_void_p), C.byref(steps), C.byref(edges))
     assert rc == 0, "oracle rejected the parameters"
     return paths, steps.value, edges.value
 

@@ -87,7 +87,7 @@ def test_sampler_micro_benchmark_and_converter(gpu, tmp_path):
     """fw_sampler_bench (one sampling step at fixed list lengths, six algorithms, both granularities) runs and reports every sample;
     a graph written by fw_convert loads and walks."""
     tool = os.path.join(ROOT, "flowwalker-artifact_amd", "bin", "fw_sampler_bench")
-    r = subprocess.run([tool, "--elements", "1048576", "--samples", "20000", "--gran", "16,1024", "--reps", "1",
+    r = subprocess.run([tool, "--elements", "1048576", "--samples", "20000", "--lengths", "16,1024", "--reps", "1",
                         "--type", "native,zprs,dprs,its,rjs,als"],
                        stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
     assert r.returncode == 0, r.stderr
@@ -111,6 +111,35 @@ def test_sampler_micro_benchmark_and_converter(gpu, tmp_path):
     ref, _, _ = orc.walk(orc.Graph(xadj, adj, w, lab), orc.make_params(app=2, max_depth=11, seed=9, p=2.0, q=0.5),
                          np.arange(200, dtype=np.int32))
     assert (paths == ref).all()
+
+
+def test_sampler_micro_benchmark_takes_the_reference_command_lines(gpu):
+    """The commands of the reference's README for Figure 6a / 6b (README.md:128-149: `--groupsize=$SAMPLING_SIZE --gran=32
+    --type=1` ...) and the same measurements spelled as the flags' own descriptions have them (src/sampler_test.cu:33-35:
+    --groupsize = threads of a sampler, --gran = elements per sampler) run, sample every list once and end with the
+    reference's "Elapsed time" line (src/sampler_test.cu:915).  --elements shrinks the 512 Mi-element array for the test."""
+    tool = os.path.join(ROOT, "flowwalker-artifact_amd", "bin", "fw_sampler_bench")
+    size = 1 << 20
+    readme = [(1, 32), (2, 512), (5, 32), (6, 512), (7, 32), (8, 512), (3, 32), (4, 512)]
+    names = {1: "zprs", 2: "zprs", 3: "dprs", 4: "dprs", 5: "its", 6: "its", 7: "als", 8: "als"}
+    for sampling_size in (128, 2048):
+        for typ, gran in (readme if sampling_size == 128 else readme[:2]):
+            for args in (["--groupsize=%d" % sampling_size, "--gran=%d" % gran, "--type=%d" % typ],       # README.md
+                         ["--groupsize=%d" % gran, "--gran=%d" % sampling_size, "--type=%d" % typ]):      # the source's flags
+                r = subprocess.run([tool, "--elements=%d" % size] + args, stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                                   text=True, timeout=300)
+                assert r.returncode == 0, (args, r.stderr)
+                cfg = re.search(r"Number of Threads in a Sampler: (\d+), Sampler Type: (\d+) \((\w+)\), Number of Elements "
+                                r"Processed by a Sampler: (\d+), Number of tasks: (\d+)", r.stdout)
+                assert cfg, r.stdout
+                assert int(cfg.group(1)) == (64 if typ % 2 else 512) and int(cfg.group(2)) == typ
+                assert cfg.group(3) == names[typ]
+                assert int(cfg.group(4)) == sampling_size and int(cfg.group(5)) == size // sampling_size
+                assert int(re.search(r"Samples: (\d+),", r.stdout).group(1)) == size // sampling_size
+                assert float(re.search(r"Elapsed time: ([0-9.]+) ms", r.stdout).group(1)) > 0.0
+    # a size flag without a numeric type is refused instead of being read as this tool's own list-length flag
+    r = subprocess.run([tool, "--gran=32", "--type", "native"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    assert r.returncode == 2 and "--lengths" in r.stderr
 
 
 def test_save_degree_and_lognorm(gpu, graph_files, tmp_path):
@@ -143,11 +172,12 @@ def test_save_degree_and_lognorm(gpu, graph_files, tmp_path):
 
 
 def test_ablation_levels_and_park_threshold(gpu, graph_files, tmp_path):
-    """--walkmode 9 / 10 / 1 / 6 are the reference's ablation levels (README.md:152-163: DPRS static, ZPRS static, ZPRS
-    with the dispenser), run by its own samplers restated for 64-lane waves; 20 / 21 / 22 are this engine's levels
-    (wave sampler alone, + workgroup sampler, + parking).  Parking and the way queries are assigned never change a
-    path; the sampler and its granularity are part of the sampling definition: every level equals the oracle run
-    with its settings."""
+    """--walkmode 9 / 10 / 1 / 6 are the reference's ablation levels (README.md:152-163), run by its own samplers restated
+    for 64-lane waves: DPRS, static assignment, thread-owned generators in device memory; the same with the generators
+    in LDS (same walks); ZPRS instead of DPRS; ZPRS with the dispenser (draws addressed by walker, step and element).
+    20 / 21 / 22 are this engine's levels (wave sampler alone, + workgroup sampler, + parking).  Every level equals the
+    oracle run with its settings -- the statically assigned levels the oracle's thread-by-thread replay of the launch
+    the tool reports (grid and block)."""
     prefix, csr = graph_files
     V = len(csr[0]) - 1
     starts = np.arange(V, dtype=np.int32)
@@ -155,17 +185,26 @@ def test_ablation_levels_and_park_threshold(gpu, graph_files, tmp_path):
     ref_wg, _, _ = orc.walk(og, orc.make_params(max_depth=11, seed=3, hub_threshold=1000), starts)
     ref_wave, _, _ = orc.walk(og, orc.make_params(max_depth=11, seed=3, hub_threshold=0x7FFFFFFF), starts)
     ref_zprs, _, _ = orc.walk(og, orc.make_params(sampler=2, max_depth=11, seed=3, hub_threshold=1000), starts)
-    ref_dprs, _, _ = orc.walk(og, orc.make_params(sampler=3, max_depth=11, seed=3, hub_threshold=1000), starts)
-    assert (ref_zprs != ref_wg).any() and (ref_dprs != ref_zprs).any()  # three samplers, three sets of walks
-    for mode, ref, note in ((9, ref_dprs, "DPRS samplers on 64-lane waves, static"), (10, ref_dprs, "DPRS"),
-                            (1, ref_zprs, "ZPRS samplers on 64-lane waves, static"),
-                            (6, ref_zprs, "ZPRS samplers on 64-lane waves, global query dispenser"),
+    assert (ref_zprs != ref_wg).any()
+    seen = {}
+    for mode, ref, note in ((9, None, "DPRS samplers on 64-lane waves, static query assignment, thread-owned generators in device memory"),
+                            (10, None, "DPRS samplers on 64-lane waves, static query assignment, thread-owned generators in LDS"),
+                            (1, None, "ZPRS samplers on 64-lane waves, static query assignment, thread-owned generators in LDS"),
+                            (6, ref_zprs, "ZPRS samplers on 64-lane waves, global query dispenser, draws addressed by"),
                             (20, ref_wave, "wave sampler only"), (21, ref_wg, "no parking"), (22, ref_wg, "full engine")):
         out = str(tmp_path / ("m%d.bin" % mode))
         text = _run("--input", prefix, "--deepwalk", "--all", "--d=10", "--seed=3", "--hub_threshold=1000",
                     "--walkmode=%d" % mode, "--savepaths", out)
         assert "ablation level %d" % mode in text and note in text
-        assert (np.fromfile(out, dtype=np.int32).reshape(V, 11) == ref).all(), mode
+        got = np.fromfile(out, dtype=np.int32).reshape(V, 11)
+        if ref is None:
+            launch = re.search(r"grid:(\d+),block:(\d+)", text)
+            ref, _, _ = orc.walk_ref_threads(og, orc.make_params(sampler=3 if mode in (9, 10) else 2, max_depth=11, seed=3,
+                                                                 hub_threshold=1000, wg_threads=int(launch.group(2))),
+                                             starts, int(launch.group(1)))
+        assert (got == ref).all(), mode
+        seen[mode] = got
+    assert (seen[9] == seen[10]).all() and (seen[10] != seen[1]).any() and (seen[1] != seen[6]).any()
     for park in (-1, 50):
         out = str(tmp_path / ("k%d.bin" % park))
         _run("--input", prefix, "--deepwalk", "--all", "--d=10", "--seed=3", "--hub_threshold=1000",

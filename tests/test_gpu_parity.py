@@ -68,6 +68,37 @@ def test_node2vec(gpu, hub):
     _check(gpu, hub, starts, app=gpu.APP_NODE2VEC, max_depth=16, p=2.0, q=0.5, hub_threshold=1000, seed=6)
 
 
+def test_node2vec_on_a_multigraph(gpu):
+    """Duplicate edges: neighbour lists that ascend with equal entries are accepted (fw_graph_is_sorted, the adjacency
+    test is a binary search), every copy of an edge is a candidate of its own, and the walks equal the oracle's; a
+    list that descends somewhere is still refused."""
+    rng = np.random.RandomState(77)
+    V = 3000
+    deg = rng.randint(1, 40, size=V)
+    deg[:3] = (2500, 900, 200)
+    xadj = np.zeros(V + 1, dtype=np.uint32)
+    np.cumsum(deg, out=xadj[1:])
+    adj = np.concatenate([np.sort(rng.randint(0, V // 4 if d > 100 else V, size=d)) for d in deg]).astype(np.int32)
+    assert any((np.diff(adj[xadj[v]:xadj[v + 1]]) == 0).any() for v in range(3))   # the hubs hold duplicates
+    w = (1.0 + 9.0 * rng.random_sample(len(adj))).astype(np.float32)
+    lab = rng.randint(0, 5, size=len(adj)).astype(np.int32)
+    starts = rng.randint(0, V, size=4000).astype(np.int32)
+    starts[:200] = 0
+    for park in (-1, 16):
+        for p, q in ((2.0, 0.5), (0.25, 4.0)):
+            _check(gpu, (xadj, adj, w, lab), starts, app=gpu.APP_NODE2VEC, max_depth=12, p=p, q=q, hub_threshold=1000,
+                   park_threshold=park, seed=31)
+    bad = adj.copy()
+    bad[[0, 1]] = bad[[1, 0]] if bad[0] != bad[1] else (bad[1] + 1, bad[1])
+    g = gpu.Graph.from_csr(xadj, bad, w, lab)
+    try:
+        with pytest.raises(gpu.FlowWalkerError) as e:
+            g.walk(gpu.default_params(app=gpu.APP_NODE2VEC, max_depth=3), starts[:10])
+        assert "ascending neighbour lists" in str(e.value)
+    finally:
+        g.destroy()
+
+
 def test_node2vec_on_lists_of_every_length(gpu):
     """node2vec proposes by weight and accepts with one search in N(prev): hubs of 30,000 / 20,000 / 5,000 / 600 / 70
     neighbours as cur and as prev, p < 1 < q and p > 1 > q (rejections on every kind of neighbour), wave and
@@ -373,6 +404,46 @@ def test_reference_engine_on_wave64(gpu, hub, sampler, static):
         assert st.launches == 1 and st.hub_steps == 0  # the reference's engine never parks
 
 
+@pytest.mark.parametrize("sampler", ["ref_zprs", "ref_dprs"])
+def test_reference_engine_with_thread_owned_generators(gpu, hub, sampler):
+    """FW_SAMPLER_REF_RNG_GLOBAL / _LDS with static assignment: the "FW" and "+ RNG" levels of the reference's ablation
+    (README.md:152-163), generators that belong to the threads with their state in device memory (cuRAND's place,
+    include/walker.cuh:1584-1696) or in LDS (include/myrand.cuh:83-86).  The walks are a function of the launch, which
+    the oracle replays thread by thread: bit-exact paths and counters for both placements, all four applications,
+    wave and workgroup granularity, several launch shapes; without static assignment the flags are refused."""
+    base = (gpu.SAMPLER_REF_ZPRS if sampler == "ref_zprs" else gpu.SAMPLER_REF_DPRS) | gpu.SAMPLER_REF_STATIC
+    starts = np.random.RandomState(8).randint(0, 12000, size=1500).astype(np.int32)
+    starts[:40] = 0
+    starts[40:60] = 1
+    xadj, adj, w, lab = hub
+    og = _oracle.Graph(xadj, adj, w, lab)
+    g = gpu.Graph.from_csr(xadj, adj, w, lab)
+    try:
+        for kw in (dict(app=gpu.APP_DEEPWALK, max_depth=21, hub_threshold=1024, wg_threads=512, grid=7),
+                   dict(app=gpu.APP_DEEPWALK, max_depth=11, hub_threshold=1 << 30, wg_threads=256, grid=24),
+                   dict(app=gpu.APP_DEEPWALK, max_depth=11, hub_threshold=100, wg_threads=1024, grid=3),
+                   dict(app=gpu.APP_PPR, max_depth=41, tp=0.15, hub_threshold=1024, grid=11),
+                   dict(app=gpu.APP_NODE2VEC, max_depth=9, p=2.0, q=0.5, hub_threshold=2000, wg_threads=256, grid=5),
+                   dict(app=gpu.APP_METAPATH, max_depth=7, schema=[1, 3, 0], hub_threshold=1024, grid=1000)):
+            got = []
+            for place in (gpu.SAMPLER_REF_RNG_LDS, gpu.SAMPLER_REF_RNG_GLOBAL):
+                p = gpu.default_params(sampler=base | place, seed=55, **kw)
+                paths, st = g.walk(p, starts)
+                assert st.launches == 1 and st.hub_steps == 0
+                ref, steps, edges = _oracle.walk_ref_threads(og, _oracle.from_walk_params(p), starts, st.grid)
+                bad = np.nonzero((paths != ref).any(axis=1))[0]
+                assert len(bad) == 0, "%s: first differing walk %d:\n gpu %s\n ref %s" % (kw, bad[0], paths[bad[0]], ref[bad[0]])
+                assert (st.steps, st.sampled_edges) == (steps, edges)
+                got.append(paths)
+            assert (got[0] == got[1]).all()  # where the state lives changes what a draw costs, not its value
+        p = gpu.default_params(sampler=(base & 0xFF) | gpu.SAMPLER_REF_RNG_LDS, max_depth=5, seed=1)
+        with pytest.raises(gpu.FlowWalkerError) as e:
+            g.walk(p, starts)
+        assert e.value.status == 1 and "FW_SAMPLER_REF_STATIC" in str(e.value)
+    finally:
+        g.destroy()
+
+
 def test_one_walk_call_at_a_time_per_graph(gpu):
     """The parking index, the parking lists and the launch record are cached in the fw_graph, so a second call on
     the same graph while one is running is refused with a status code (it used to race); afterwards the graph works
@@ -442,7 +513,7 @@ def test_random_access_calibration(gpu):
         assert L.fw_dev_random_access_rate(buf.ptr, (64 << 20) + 4, 0, C.byref(rate)) == 1  # not a multiple of a line
         assert L.fw_dev_random_access_rate(buf.ptr, 64 << 20, 7, C.byref(rate)) == 1    # unknown mode
         assert L.fw_dev_random_access_rate(None, 64 << 20, 0, C.byref(rate)) == 1
-        for mode in (0, 1, 3):
+        for mode in (0, 1, 3, 4, 5):
             gpu.check(L.fw_dev_random_access_rate(buf.ptr, 64 << 20, mode, C.byref(rate)))
             assert 1e9 < rate.value < 1e13
     finally:

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol(fw):
 def test_struct_layouts_match_the_header(fw):
     # fw_walk_params: 6 int32 + 64 int32 + 3 float + uint32 + uint64 + 2 int32
     assert C.sizeof(fw.WalkParams) == 6 * 4 + 64 * 4 + 3 * 4 + 4 + 8 + 8
-    assert C.sizeof(fw.WalkStats) == 8 + 8 + 8 + 8 + 4 + 4 + 8 + 8 + 8 + 8 + 8
+    assert C.sizeof(fw.WalkStats) == 8 + 8 + 8 + 8 + 4 + 4 + 8 + 8 + 8 + 8 + 8 + 4 * 8
     assert C.sizeof(fw.RmatParams) == 48
 
 
@@ -210,6 +210,21 @@ def test_sort_neighbours_moves_weights_and_labels_with_their_edges(fw):
     assert fw.csr_sort_neighbours(xadj, a2, w2, l2) == shuffled
     assert (a2 == adj).all() and (w2 == w).all() and (l2 == lab).all()   # uniform_graph's lists ascend, no duplicates
     assert fw.csr_sort_neighbours(xadj, a2, w2, l2) == 0
+
+
+def test_sort_neighbours_keeps_duplicate_edges_in_order(fw):
+    """A multigraph: a list with equal neighbours counts as ascending (the adjacency test is a binary search, which only
+    needs a non-decreasing list, include/gpu_graph.cuh:97-112), the sort keeps every copy of an edge with its own weight,
+    and a sorted list with duplicates is left alone."""
+    xadj = np.array([0, 6, 6, 9], dtype=np.uint32)
+    adj = np.array([2, 1, 2, 0, 1, 2, 0, 0, 1], dtype=np.int32)
+    w = np.arange(9, dtype=np.float32) + 1.0
+    lab = np.arange(9, dtype=np.int32)
+    assert fw.csr_sort_neighbours(xadj, adj, w, lab) == 1                 # the second list (0, 0, 1) already ascends
+    assert adj.tolist() == [0, 1, 1, 2, 2, 2, 0, 0, 1]
+    assert w.tolist() == [4.0, 2.0, 5.0, 1.0, 3.0, 6.0, 7.0, 8.0, 9.0]   # stable: copies keep their order
+    assert lab.tolist() == [3, 1, 4, 0, 2, 5, 6, 7, 8]
+    assert fw.csr_sort_neighbours(xadj, adj, w, lab) == 0
 
 
 def test_bench_measures_one_gpu_only():

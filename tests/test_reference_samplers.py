@@ -145,3 +145,136 @@ def test_wave64_restatements_follow_the_law_in_whole_walks():
             cnt = np.bincount(paths[:, 1], minlength=V)[:n].astype(np.float64)
             assert cnt.sum() == m and cnt[~pos].sum() == 0
             assert chisquare(cnt[pos], expect).pvalue > 0.01, (sampler, thr)
+
+
+def _thread_uniform(seed, gid, k):
+    """k-th uniform of the generator that thread `gid` owns: word k & 3 of Philox block (gid, k >> 2, 0x08000000, 0),
+    mapped to (0, 1]."""
+    out = orc.philox([gid, k >> 2, 0x08000000, 0], [seed & 0xFFFFFFFF, seed >> 32])
+    return np.float32(((int(out[k & 3]) >> 8) + 1) * 2.0 ** -24)
+
+
+def _replay_model(xadj, adj, w, starts, grid, W, thr, depth, seed, dprs):
+    """The launch of the reference's engine with thread-owned generators, written down independently of the C replay:
+    who owns which query, which slot is stepped when and by which threads, and which of its draws a thread spends on
+    which element.  The samplers themselves are the pinned fw_ref64_* (orc.ref_sample_many)."""
+    n = len(starts)
+    grid = min(grid, (n + 63) // 64)
+    per = (n + grid - 1) // grid
+    nw = W // 64
+    paths = np.full((n, depth), -1, dtype=np.int32)
+    for b in range(grid):
+        lo, hi = min(b * per, n), min(b * per + per, n)
+        count = [0] * W
+        nxt = lo
+        slots = [None] * 64
+
+        def take(s):
+            nonlocal nxt
+            if nxt < hi:
+                q = nxt
+                nxt += 1
+                paths[q, 0] = starts[q]
+                slots[s] = dict(q=q, cur=int(starts[q]), len=1)
+            else:
+                slots[s] = None
+
+        def step(sl, threads):
+            off, deg = int(xadj[sl["cur"]]), int(xadj[sl["cur"] + 1] - xadj[sl["cur"]])
+            if deg == 0:
+                return -1
+            Wg = len(threads)
+            u = np.zeros(deg, dtype=np.float32)
+            if dprs:
+                for base in range(0, deg + Wg - deg % Wg, Wg):
+                    for l, t in enumerate(threads):
+                        d = _thread_uniform(seed, b * W + t, count[t])
+                        count[t] += 1
+                        if base + l < deg:
+                            u[base + l] = d
+            else:
+                for l, t in enumerate(threads):
+                    for i in range(l, deg, Wg):
+                        u[i] = _thread_uniform(seed, b * W + t, count[t])
+                        count[t] += 1
+            kind = orc.REF64_DPRS if dprs else orc.REF64_ZPRS
+            return int(orc.ref_sample_many(kind, w[off:off + deg], u[None, :], Wg)[0])
+
+        for s in range(64):
+            take(s)
+        while any(sl is not None for sl in slots):
+            large = []
+            for v in range(nw):
+                for s in range(v, 64, nw):
+                    sl = slots[s]
+                    if sl is None or sl["len"] >= depth:
+                        continue
+                    if int(xadj[sl["cur"] + 1] - xadj[sl["cur"]]) > thr:
+                        large.append(s)
+                        continue
+                    sel = step(sl, list(range(64 * v, 64 * v + 64)))
+                    if sel < 0:
+                        sl["len"] = depth
+                    else:
+                        nv = int(adj[int(xadj[sl["cur"]]) + sel])
+                        paths[sl["q"], sl["len"]] = nv
+                        sl["cur"], sl["len"] = nv, sl["len"] + 1
+            for s in sorted(large):
+                sl = slots[s]
+                sel = step(sl, list(range(W)))
+                if sel < 0:
+                    sl["len"] = depth
+                else:
+                    nv = int(adj[int(xadj[sl["cur"]]) + sel])
+                    paths[sl["q"], sl["len"]] = nv
+                    sl["cur"], sl["len"] = nv, sl["len"] + 1
+            for s in range(64):
+                sl = slots[s]
+                if sl is not None and (sl["len"] >= depth or xadj[sl["cur"] + 1] == xadj[sl["cur"]]):
+                    take(s)
+    return paths
+
+
+@pytest.mark.parametrize("dprs", [False, True])
+def test_thread_owned_generators_replay_against_an_independent_model(dprs):
+    """fw_oracle_walk_ref_threads (the reference's engine with generators that belong to the threads, static assignment)
+    against a Python model of the same launch: a small graph with a list above the workgroup threshold, dead ends,
+    three workgroups with uneven shares, two waves per workgroup."""
+    import _graphs
+    xadj, adj, w, lab = _graphs.hub_graph(V=300, hub_degrees=(200,), base_degree=3, seed=4, symmetric=False)
+    rng = np.random.RandomState(5)
+    starts = rng.randint(0, 300, size=170).astype(np.int32)
+    starts[:6] = 0
+    for grid, W, thr in ((3, 128, 100), (2, 64, 1 << 30), (1, 256, 2)):
+        p = orc.make_params(sampler=3 if dprs else 2, max_depth=6, wg_threads=W, hub_threshold=thr, seed=91)
+        got, steps, edges = orc.walk_ref_threads(orc.Graph(xadj, adj, w, lab), p, starts, grid)
+        want = _replay_model(xadj, adj, w, starts, grid, W, thr, 6, 91, dprs)
+        assert (got == want).all(), (grid, W, thr)
+        deg = np.diff(xadj.astype(np.int64))
+        assert steps == int((got[:, 1:] >= 0).sum())
+        assert edges == int(sum(deg[row[j - 1]] for row in got for j in range(1, 6) if row[j] >= 0))
+
+
+def test_thread_owned_generators_follow_the_law():
+    """First steps from one vertex with thread-owned generators: chi-square against w / sum w for both samplers, wave and
+    workgroup granularity, and launches of different shape (the walks depend on the launch, the law does not)."""
+    rng = np.random.RandomState(99)
+    n, m = 900, 100000
+    w = (1.0 + 99.0 * rng.random_sample(n)).astype(np.float32)
+    w[rng.random_sample(n) < 0.1] = 0.0
+    pos = w > 0
+    expect = w[pos].astype(np.float64) / w.astype(np.float64).sum() * m
+    V = n + 2
+    xadj = np.zeros(V + 1, dtype=np.uint32)
+    xadj[2:] = n
+    g = orc.Graph(xadj, (np.arange(n) % V).astype(np.int32), w)
+    seen = []
+    for sampler in (2, 3):
+        for thr, grid, W in ((1 << 30, 40, 256), (500, 7, 128)):
+            p = orc.make_params(sampler=sampler, max_depth=2, hub_threshold=thr, wg_threads=W, seed=78)
+            paths, steps, _ = orc.walk_ref_threads(g, p, np.full(m, 1, dtype=np.int32), grid)
+            cnt = np.bincount(paths[:, 1], minlength=V)[:n].astype(np.float64)
+            assert steps == m and cnt.sum() == m and cnt[~pos].sum() == 0
+            assert chisquare(cnt[pos], expect).pvalue > 0.01, (sampler, thr)
+            seen.append(paths[:, 1].copy())
+    assert (seen[0] != seen[1]).any()  # another launch shape, other walks
