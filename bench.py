@@ -203,6 +203,8 @@ def main():
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the one-pass report of the other configurations after the timed region")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
+    ap.add_argument("--p", type=float, default=0.0, help="node2vec return parameter (0 = the library default 2.0)")
+    ap.add_argument("--q", type=float, default=0.0, help="node2vec in-out parameter (0 = the library default 0.5)")
     ap.add_argument("--hub-threshold", type=int, default=-1)
     ap.add_argument("--wg-threads", type=int, default=0)
     ap.add_argument("--park-threshold", type=int, default=0, help="0 = library default, -1 = hub parking off")
@@ -229,7 +231,7 @@ def main():
     if args.scale:
         wl["scale"] = args.scale
     defaults = (not args.scale and args.park_threshold == 0 and args.hub_threshold < 0 and args.wg_threads == 0
-                and args.sampler == "native")
+                and args.sampler == "native" and args.p == 0.0 and args.q == 0.0)
 
     t0 = time.time()
     g = make_graph(fw, wl)
@@ -244,6 +246,10 @@ def main():
     if args.wg_threads:
         params.wg_threads = args.wg_threads
     params.park_threshold = args.park_threshold
+    if args.p > 0.0:
+        params.p = args.p
+    if args.q > 0.0:
+        params.q = args.q
     if args.sampler != "native":
         params.sampler = fw.SAMPLER_REF_ZPRS if args.sampler == "ref_zprs" else fw.SAMPLER_REF_DPRS
         if args.hub_threshold < 0:
@@ -326,6 +332,7 @@ def main():
             "walk_steps_per_pass": int(last.steps), "sampled_edges_per_pass": int(last.sampled_edges),
             "wg_threads": params.wg_threads, "hub_threshold": params.hub_threshold,
             "park_threshold": params.park_threshold, "sampler": args.sampler, "launches_per_pass": last.launches,
+            "p": params.p, "q": params.q,
             "grid": last.grid,
             "graph_gen_s": round(gen_s, 2), "sources_sha": sources_sha,
         },

@@ -325,7 +325,7 @@ extern "C" int fw_graph_destroy(fw_graph* g) {
   }
   release_park_cache(g);
   for (hipEvent_t e : g->call_ev) if (e) (void)hipEventDestroy(e);
-  void* index_ptrs[3] = {g->hub_index, g->hub_info, g->call_scratch};
+  void* index_ptrs[4] = {g->hub_index, g->hub_info, g->call_scratch, g->adj_hub};
   for (void* p : index_ptrs) {
     if (p && hipFree(p) != hipSuccess) { (void)hipGetLastError(); rc = FW_ERR_HIP; }
   }
@@ -608,11 +608,24 @@ __global__ void fw_hub_index_kernel(const uint32_t* __restrict__ xadj, int32_t V
   }
 }
 
-// (Re)builds g->hub_index / hub_info for `threshold`; cached in the graph.
+// Every adjacency entry next to the parking index of the vertex it names.  A hub step needs both (the vertex for the
+// path, the index to park the walker again), and what the kernels pay for is the number of memory requests: the pair
+// sits in one 128-byte block, the entry and a look-up in hub_index are two.
+__global__ void fw_adj_hub_kernel(const int32_t* __restrict__ adjncy, const int32_t* __restrict__ hub_index, uint64_t E,
+                                  int2* __restrict__ adj_hub) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t e = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; e < E; e += stride) {
+    const int32_t v = adjncy[e];
+    adj_hub[e] = make_int2(v, hub_index[v]);
+  }
+}
+
+// (Re)builds g->hub_index / hub_info / adj_hub for `threshold`; cached in the graph.
 static int ensure_hub_index(fw_graph* g, int32_t threshold) {
   if (g->hub_index_threshold == threshold && g->hub_index) return FW_OK;
   if (g->hub_index) { (void)hipFree(g->hub_index); g->hub_index = nullptr; }
   if (g->hub_info) { (void)hipFree(g->hub_info); g->hub_info = nullptr; }
+  if (g->adj_hub) { (void)hipFree(g->adj_hub); g->adj_hub = nullptr; }
   g->hub_index_threshold = -1;
   g->n_hubs = 0;
   unsigned* d_cnt = nullptr;
@@ -634,6 +647,18 @@ static int ensure_hub_index(fw_graph* g, int32_t threshold) {
   if (rc == FW_OK) rc = fw_check_hip(hipMemcpy(&rows_taken, d_cnt + 2, sizeof(unsigned), hipMemcpyDeviceToHost), "hipMemcpy(hub rows)", __FILE__, __LINE__);
   (void)hipFree(d_cnt);
   if (rc != FW_OK) return rc;
+  // the annotated adjacency is an extra: without room for it (or with the edges in host memory, where it would be
+  // read over the bus) the hub kernels look the index up
+  if (n_hubs != 0u && !g->host_edges) {
+    if (hipMalloc(reinterpret_cast<void**>(&g->adj_hub), (size_t)g->E * sizeof(int2)) == hipSuccess) {
+      hipLaunchKernelGGL(fw_adj_hub_kernel, dim3(8192), dim3(256), 0, 0, g->adjncy, g->hub_index, g->E, g->adj_hub);
+      rc = fw_check_hip(hipDeviceSynchronize(), "adjacency with parking indices", __FILE__, __LINE__);
+      if (rc != FW_OK) return rc;
+    } else {
+      (void)hipGetLastError();
+      g->adj_hub = nullptr;
+    }
+  }
   g->n_hubs = (int32_t)n_hubs;
   g->hub_rows = rows_taken < kMaxHubRows ? rows_taken : kMaxHubRows;  // rows past the limit were not handed out
   g->hub_index_threshold = threshold;
@@ -1190,6 +1215,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   a.park_threshold = park_threshold;
   a.n_labels_per_hub = labels;
   a.hub_index = g->hub_index;
+  a.adj_hub = g->adj_hub;
   a.parked = pb->walked;
   a.parked_count = &pb->ctrs[0 * FW_CTR_STRIDE];
   fw_hub_args h;

@@ -37,6 +37,9 @@ struct fw_graph {
   int32_t n_hubs = 0;
   uint32_t hub_rows = 0;              // rows the hubs with rows need together, per label
   int32_t* hub_index = nullptr;       // int32[V]: position in hub_info, -1 (not parked on) or -2 (degree 0)
+  int2* adj_hub = nullptr;            // int2[E]: {adjncy[e], hub_index[adjncy[e]]}, so that a hub step learns its new
+                                      // vertex and that vertex's parking index with one memory request instead of two;
+                                      // NULL when the edge arrays live in host memory or there was no room
   struct fw_hub_info* hub_info = nullptr;  // [n_hubs]
   void* park_cache = nullptr;         // the parking lists of the last fw_walk_device call, kept for the next one
   void* call_scratch = nullptr;       // launch record (dispenser word + counters) of fw_walk_device, allocated once
@@ -79,6 +82,7 @@ struct fw_kargs {
   int32_t park_threshold;            // a walker that arrives on a vertex of larger degree is parked
   int32_t n_labels_per_hub;          // buckets per hub: 1, or schema_len for metapath (walkers wanting one label share a scan)
   const int32_t* hub_index;          // int32[V]: index of the vertex among the parked-on ones, -1, or -2 = degree 0
+  const int2* adj_hub;               // int2[E] or NULL: every adjacency entry with the parking index of its vertex
   fw_walker_rec* parked;             // out: parked[i] = the walker of entry i of the launch's input if it was parked, else a hole (q = -1)
   uint32_t* parked_count;            // += walkers parked (one update per workgroup)
   uint32_t* bucket_count;            // [n_hubs * n_labels_per_hub]

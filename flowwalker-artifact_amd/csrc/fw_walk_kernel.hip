@@ -1364,8 +1364,15 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
   bool retry = false;
   bool go_on = false;
   int32_t nv = -1;
+  int32_t nv_hidx = -1;  // the parking index of nv when it came with the adjacency entry
   if (moved) {
-    nv = a.adjncy[off + (uint32_t)pick];
+    if (a.adj_hub != nullptr) {
+      const int2 e = a.adj_hub[off + (uint32_t)pick];
+      nv = e.x;
+      nv_hidx = e.y;
+    } else {
+      nv = a.adjncy[off + (uint32_t)pick];
+    }
     if (kApp == FW_APP_NODE2VEC && rec.prev >= 0) {
       const N2vTest t = n2v_test(a, nv, rec.prev, walker, step, trial);
       bool common = false;
@@ -1404,7 +1411,7 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
   if (go_on) {
     // one look-up tells both what the step commit needs to know about the new vertex: parked on (index >= 0),
     // a dead end that finishes the walk (-2, include/walker.cuh:1373-1374), or neither
-    hidx = a.hub_index[nv];
+    hidx = a.adj_hub != nullptr ? nv_hidx : a.hub_index[nv];
     go_on = hidx != -2;
     park = hidx >= 0;
   }
