@@ -902,10 +902,14 @@ __global__ void fw_scatter_tagged_kernel(const fw_walker_rec* __restrict__ src, 
 // tagged_only (node2vec, whose records carry the previous vertex instead of a position): src is a batch launch's
 // output list, of which only the records tagged FW_REC_PARK take part.  whole (node2vec): the sorted list holds
 // fw_walker_rec, otherwise fw_parked_rec.
+// m_dev: when not NULL the number of entries is read there (m is an upper bound the grid was sized for): the launch
+// is queued before the host has seen the counters of the round that made the list.
 __global__ void fw_scatter_counted_kernel(const fw_walker_rec* __restrict__ src, uint32_t m,
+                                          const uint32_t* __restrict__ m_dev,
                                           const uint32_t* __restrict__ bucket_count,
                                           const uint32_t* __restrict__ bucket_offset, uint32_t* bucket_fill,
                                           void* __restrict__ sorted, int tagged_only, int whole) {
+  if (m_dev != nullptr) m = *m_dev < m ? *m_dev : m;
   const uint32_t stride = gridDim.x * blockDim.x;
   for (uint32_t i0 = blockIdx.x * blockDim.x; i0 < m; i0 += stride) {  // uniform in the wave: the ranks are taken together
     const uint32_t i = i0 + threadIdx.x;
@@ -1045,6 +1049,7 @@ struct ParkBuffers {
   hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};  // timing events of the walk and the hub launches
   hipStream_t side = nullptr;          // the quad launch of a round runs beside the batch launch
   hipEvent_t fork = nullptr, join = nullptr;
+  hipEvent_t copied = nullptr;         // the round's counters have reached the host
 
   uint32_t* count(int parity) const { return buckets + (size_t)parity * n_buckets; }
   uint32_t* offset() const { return buckets + (size_t)2 * n_buckets; }
@@ -1069,6 +1074,7 @@ struct ParkBuffers {
     FW_HIP(hipStreamCreateWithFlags(&side, hipStreamNonBlocking));
     FW_HIP(hipEventCreateWithFlags(&fork, hipEventDisableTiming));
     FW_HIP(hipEventCreateWithFlags(&join, hipEventDisableTiming));
+    FW_HIP(hipEventCreateWithFlags(&copied, hipEventDisableTiming));
     // the rows are an extra: without room for them every bucket is served by batch tasks
     if (rows_wanted != 0u) {
       // scan tasks: a list of G groups is cut into at most G / kScanRun + 1 runs, and no more lists are scanned in
@@ -1110,8 +1116,9 @@ struct ParkBuffers {
     if (side) (void)hipStreamDestroy(side);
     if (fork) (void)hipEventDestroy(fork);
     if (join) (void)hipEventDestroy(join);
+    if (copied) (void)hipEventDestroy(copied);
     side = nullptr;
-    fork = join = nullptr;
+    fork = join = copied = nullptr;
     walked = sorted = out = resume = nullptr;
     buckets = ctrs = h_ctrs = nullptr;
     tasks = wtasks = qtasks = nullptr;
@@ -1266,14 +1273,53 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     ++*launches;
     return FW_OK;
   };
-  auto read_back = [&]() -> int {
+  // The counters of a round go to the host once per round.  Behind the copy, before the host waits for it, the part of
+  // the next round that needs nothing from the host is queued already -- the bucket scan, the counting sort of the
+  // parked walkers and the reset of the round's counters -- so the device works through the host's round trip.
+  auto copy_counters = [&]() -> int {
     FW_HIP(hipMemcpyAsync(pb->h_ctrs, pb->ctrs, kParkCtrs * FW_CTR_STRIDE * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
-    FW_HIP(hipStreamSynchronize(stream));
+    FW_HIP(hipEventRecord(pb->copied, stream));
     return FW_OK;
+  };
+  auto wait_counters = [&]() -> int {
+    FW_HIP(hipEventSynchronize(pb->copied));
+    return FW_OK;
+  };
+  auto read_back = [&]() -> int {  // for the last launch of a call: nothing follows
+    int rc_ = copy_counters();
+    return rc_ != FW_OK ? rc_ : wait_counters();
   };
   unsigned rblocks = ((unsigned)pb->n_buckets + 255u) / 256u;
   if (rblocks > 2048u) rblocks = 2048u;
   if (rblocks == 0u) rblocks = 1u;
+  auto blocks_for = [](uint32_t cnt) {
+    unsigned blocks = (cnt + 255u) / 256u;
+    return blocks > 8192u ? 8192u : (blocks ? blocks : 1u);
+  };
+  // The sort of the walkers parked for the coming round (bucket counts in array `cnt`): n_tagged records of the last
+  // batch launch's output list (0: there was none) and the last walk launch's list of n_entries positions at most (the
+  // exact number on the device at entries_dev when not NULL); then the counters start the round at zero and array
+  // `nxt` is cleared for the walkers the round will park.
+  auto queue_sort = [&](int cnt, int nxt, uint32_t n_tagged, uint32_t n_entries, const uint32_t* entries_dev) -> int {
+    FW_HIP(rocprim::exclusive_scan(pb->tmp, pb->scan_bytes, pb->count(cnt), pb->offset(), 0u, (size_t)pb->n_buckets,
+                                   rocprim::plus<uint32_t>(), stream));
+    if (n_tagged != 0u) {
+      if (p->app == FW_APP_NODE2VEC)
+        hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_tagged)), dim3(256), 0, stream, pb->out, n_tagged,
+                           static_cast<const uint32_t*>(nullptr), pb->count(cnt), pb->offset(), pb->fill(), pb->sorted, 1, 1);
+      else
+        hipLaunchKernelGGL(fw_scatter_tagged_kernel, dim3(blocks_for(n_tagged)), dim3(256), 0, stream, pb->out, n_tagged,
+                           pb->offset(), reinterpret_cast<fw_parked_rec*>(pb->sorted));
+    }
+    if (n_entries != 0u)  // the walk launch's list has one position per entry of its input: parked walkers and holes
+      hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_entries)), dim3(256), 0, stream, pb->walked,
+                         n_entries, entries_dev, pb->count(cnt), pb->offset(), pb->fill(), pb->sorted, 0,
+                         p->app == FW_APP_NODE2VEC ? 1 : 0);
+    hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs * FW_CTR_STRIDE, pb->count(nxt),
+                       pb->fill(), pb->n_buckets, a.dispenser);
+    FW_HIP(hipGetLastError());
+    return FW_OK;
+  };
 
   if (two_pass_possible) {  // no bucket has rows yet
     hipLaunchKernelGGL(fw_fill_i32_kernel, dim3(rblocks), dim3(256), 0, stream, reinterpret_cast<int32_t*>(pb->rows_made()),
@@ -1291,7 +1337,9 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   entries_hint = hint_for((uint64_t)a.n);
   int rc = queue_walk(grid_used);
   if (rc != FW_OK) return rc;
-  if ((rc = read_back()) != FW_OK) return rc;
+  if ((rc = copy_counters()) != FW_OK) return rc;
+  if ((rc = queue_sort(0, 1, 0u, (uint32_t)a.n, nullptr)) != FW_OK) return rc;
+  if ((rc = wait_counters()) != FW_OK) return rc;
   tw.collect(&times->walk_ms);
   times->parked_records += pb->h_ctrs[0 * FW_CTR_STRIDE];
   uint32_t n_out = 0;  // records in `out` (the previous batch launch's input size)
@@ -1312,28 +1360,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     if (m == 0u) break;
     if (m > pb->cap) { fw_set_error("internal: %llu walkers parked, capacity %zu", (unsigned long long)m, pb->cap); return FW_ERR_INVALID; }
     const int nxt = cur ^ 1;
-    FW_HIP(rocprim::exclusive_scan(pb->tmp, pb->scan_bytes, pb->count(cur), pb->offset(), 0u, (size_t)pb->n_buckets,
-                                   rocprim::plus<uint32_t>(), stream));
-    auto blocks_for = [](uint32_t cnt) {
-      unsigned blocks = (cnt + 255u) / 256u;
-      return blocks > 8192u ? 8192u : blocks;
-    };
-    if (n_out != 0u) {
-      if (p->app == FW_APP_NODE2VEC)
-        hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
-                           pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 1, 1);
-      else
-        hipLaunchKernelGGL(fw_scatter_tagged_kernel, dim3(blocks_for(n_out)), dim3(256), 0, stream, pb->out, n_out,
-                           pb->offset(), reinterpret_cast<fw_parked_rec*>(pb->sorted));
-    }
-    if (n_walked != 0u)  // the walk launch's list has one position per entry of its input: parked walkers and holes
-      hipLaunchKernelGGL(fw_scatter_counted_kernel, dim3(blocks_for(walk_entries)), dim3(256), 0, stream, pb->walked,
-                         walk_entries, pb->count(cur), pb->offset(), pb->fill(), pb->sorted, 0,
-                         p->app == FW_APP_NODE2VEC ? 1 : 0);
-    FW_HIP(hipGetLastError());
-    hipLaunchKernelGGL(fw_round_reset_kernel, dim3(rblocks), dim3(256), 0, stream, pb->ctrs, kParkCtrs * FW_CTR_STRIDE, pb->count(nxt),
-                       pb->fill(), pb->n_buckets, a.dispenser);
-    FW_HIP(hipGetLastError());
+    // (the scan of this round's buckets, the sort of its walkers and the reset of its counters are queued already)
     if (p->park_threshold == 0 && m < kParkTail) {
       // default rule only (an explicit threshold keeps every round in the loop): too few walkers are left to
       // meet anywhere, so they finish in one walk launch that does not park
@@ -1403,7 +1430,11 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     a.bucket_count = pb->count(nxt);
     entries_hint = hint_for(n_out != 0u ? (uint64_t)resumed + 1u : m / 4u + 1u);  // about as many as a round ago
     if ((rc = queue_walk(nullptr)) != FW_OK) return rc;
-    if ((rc = read_back()) != FW_OK) return rc;
+    if ((rc = copy_counters()) != FW_OK) return rc;
+    // the next round: this round's m records of the batch launches' output list, and the walk launch's list (as many
+    // positions as walkers resumed, which the device knows)
+    if ((rc = queue_sort(nxt, cur, (uint32_t)m, (uint32_t)m, pb->ctrs + 6 * FW_CTR_STRIDE)) != FW_OK) return rc;
+    if ((rc = wait_counters()) != FW_OK) return rc;
     th.collect(&times->hub_ms);
     tw.collect(&times->walk_ms);
     times->hub_quartets += *reinterpret_cast<const uint64_t*>(pb->h_ctrs + 14 * FW_CTR_STRIDE);
@@ -1439,7 +1470,8 @@ struct TrafficModel {
   uint64_t total() const { return list_bytes + 128u * scattered_reads + 32u * scattered_writes + record_bytes; }
 };
 
-static TrafficModel traffic_model(const fw_walk_params* p, int32_t n, bool parked, int32_t park_threshold,
+// annotated: the hub kernels read the new vertex and its parking index from one annotated adjacency entry.
+static TrafficModel traffic_model(const fw_walk_params* p, int32_t n, bool parked, int32_t park_threshold, bool annotated,
                                   uint64_t walk_steps, uint64_t walk_edges, uint64_t hub_steps, const KernelTimes& t) {
   constexpr uint64_t kRec = 16;
   const bool n2v = p->app == FW_APP_NODE2VEC;
@@ -1451,7 +1483,7 @@ static TrafficModel traffic_model(const fw_walk_params* p, int32_t n, bool parke
   if (!short_lists) m.scattered_reads += walk_steps;             // adjncy[off + sel]
   m.scattered_reads += (parked ? 2u : 1u) * walk_steps;          // xadj pair, parking index
   m.scattered_writes += walk_steps;                              // path entry
-  if (n2v) m.scattered_reads += 8 * (walk_steps + hub_steps);    // about one search in N(prev) per step
+  if (n2v) m.scattered_reads += 4 * (walk_steps + hub_steps);    // the searches in N(prev): about four blocks per step
   m.record_bytes += 4 * (uint64_t)n;                             // start vertices
   m.scattered_reads += (parked ? 2u : 1u) * (uint64_t)n;         // xadj pair, parking index
   m.scattered_writes += (uint64_t)n;                             // path[0]
@@ -1463,7 +1495,7 @@ static TrafficModel traffic_model(const fw_walk_params* p, int32_t n, bool parke
     // the new vertex and the path entry
     m.list_bytes += 16 * t.hub_quartets;
     m.record_bytes += ((n2v ? kRec : kRec / 2) + kRec) * hub_steps;
-    m.scattered_reads += 2 * hub_steps;
+    m.scattered_reads += (annotated ? 1u : 2u) * hub_steps;
     m.scattered_writes += hub_steps;
     m.scattered_reads += 7 * t.table_walkers;                    // pivots, lane row, prefix, four quartets of one lane
     // counting sort (record in, scattered record out), compaction (in, out), task list, reset, bucket scan
@@ -1571,8 +1603,8 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
     stats->hub_kernel_ms = times.hub_ms;
     stats->hub_steps = h.counters[2];
     stats->hub_sampled_edges = h.counters[3];
-    const TrafficModel tm = traffic_model(p, n, launches > 1, park_threshold, h.counters[0], h.counters[1],
-                                          h.counters[2], times);
+    const TrafficModel tm = traffic_model(p, n, launches > 1, park_threshold, g->adj_hub != nullptr, h.counters[0],
+                                          h.counters[1], h.counters[2], times);
     stats->requested_bytes = tm.total();
     stats->list_bytes = tm.list_bytes;
     stats->scattered_reads = tm.scattered_reads;
@@ -1705,7 +1737,7 @@ extern "C" int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p
     stats->hub_kernel_ms = 0.0;
     stats->hub_steps = 0;
     stats->hub_sampled_edges = 0;
-    const TrafficModel tm = traffic_model(p, n, false, INT_MAX, h.counters[0], h.counters[1], 0, KernelTimes());
+    const TrafficModel tm = traffic_model(p, n, false, INT_MAX, false, h.counters[0], h.counters[1], 0, KernelTimes());
     stats->requested_bytes = tm.total();
     stats->list_bytes = tm.list_bytes;
     stats->scattered_reads = tm.scattered_reads;
@@ -1842,7 +1874,8 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     stats->grid = grid_used;
     stats->walk_kernel_ms = times.hub_ms == 0.0 && times.walk_ms == 0.0 ? kernel_ms : times.walk_ms;
     stats->hub_kernel_ms = times.hub_ms;
-    const TrafficModel tm = traffic_model(p, n, times.hub_ms != 0.0, park_threshold, stats->steps - stats->hub_steps,
+    const TrafficModel tm = traffic_model(p, n, times.hub_ms != 0.0, park_threshold, g->adj_hub != nullptr,
+                                          stats->steps - stats->hub_steps,
                                           stats->sampled_edges - stats->hub_sampled_edges, stats->hub_steps, times);
     stats->requested_bytes = tm.total();
     stats->list_bytes = tm.list_bytes;

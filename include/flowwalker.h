@@ -91,6 +91,15 @@ typedef struct {
                             list (by a workgroup above hub_threshold, by one wave below).  0 = library default (on
                             for batches >= 65536 queries), < 0 = off, > 0 = degree.  node2vec: the shared scan
                             proposes, each walker accepts with its own adjacency test (max_depth <= 65535). */
+  /* node2vec is sampled in two stages: a neighbour is proposed with probability w / sum w and accepted with
+   * probability f / F, f = 1/p (return edge), 1 (common neighbour of the previous vertex) or 1/q, F = max(1, 1/p,
+   * 1/q); a rejected walker proposes again.  The accepted neighbour has the reference's law w f / sum w f
+   * (include/app.cuh:97-127) exactly, but the work per step follows the parameters: the expected number of proposals
+   * is F * sum w / sum w f (1.3 at p = 2, q = 0.5 on the R-MAT benchmark graph, about 4 at p = q = 4, about 16 at
+   * p = 0.25, q = 4), where the reference's one pass over the biases costs the same whatever p and q.  After 16,383
+   * rejections of one step the next proposal is taken unconditionally (the trial count travels in 14 bits of a
+   * record): at acceptance probabilities this library is meant for that never happens (0.94^16383), and where it
+   * could (f / F below about 1e-3 for every neighbour) that step follows w / sum w instead of the node2vec law. */
 } fw_walk_params;
 
 /* What src/main.cu:82-113 (calculate_workload) and the timing code of src/walk.cu report. */
@@ -110,7 +119,7 @@ typedef struct {
    * quartets streamed): requested_bytes = list_bytes + 128 * scattered_reads + 32 * scattered_writes + record_bytes.
    * list_bytes: every list pass in 16-byte quartets (a list is read once per walker step by the walk kernel, once per
    * batch of up to 64 walkers or once per call by the hub kernels); scattered_reads: reads of one 128-byte block each
-   * (CSR offset pair, parking index, selected neighbour; node2vec: 8 per step for the search of its acceptance test);
+   * (CSR offset pair, parking index, selected neighbour; node2vec: 4 per step for the searches of its acceptance tests);
    * scattered_writes: stores of one 32-byte write request each (path entry, scattered record); record_bytes: walker
    * records, tasks and bucket tables that are streamed.  Tables that stay in the L2 are not priced.  This sits
    * between the algorithmic bytes of src/main.cu:93-111 (4 * sampled_edges + ...) and what a profiler's HBM counters
