@@ -1882,7 +1882,8 @@ int launch_hub_scan_app(const fw_kargs& a, const fw_hub_args& h, uint32_t tasks_
 }
 
 // quads_hint: about how many quad tasks to expect (the launch works through any number; 0 = no idea).  Four tasks per
-// wave and turn, about eight turns per wave, between one and eight resident sets (see launch_hub_one).
+// wave and turn, about kQuadTurns turns per wave, up to eight resident sets (see launch_hub_one).
+constexpr uint32_t kQuadTurns = 4;
 template <int kApp>
 int launch_hub_quad_app(const fw_kargs& a, const fw_hub_args& h, uint32_t quads_hint, hipStream_t stream) {
   int dev = 0, cus = 0;
@@ -1891,7 +1892,7 @@ int launch_hub_quad_app(const fw_kargs& a, const fw_hub_args& h, uint32_t quads_
   const uint32_t resident = (uint32_t)cus * 8u;  // workgroups of four waves, eight waves per SIMD
   uint32_t grid = resident;
   if (quads_hint != 0u) {
-    const uint32_t wanted = quads_hint / (4u * 4u * 8u) + 1u;
+    const uint32_t wanted = quads_hint / (4u * 4u * kQuadTurns) + 1u;
     grid = wanted < 8u * resident ? wanted : 8u * resident;
   }
   hipLaunchKernelGGL((fw_hub_quad<kApp>), dim3(grid), dim3(256), 0, stream, a, h);
@@ -1940,7 +1941,7 @@ int resident_set(Kernel kernel, int wg_threads, int* cus_out, int* per_cu_out) {
 // workgroup tasks; 0 = no idea).  All tasks are dealt out by position, so the grid may be larger than what is
 // resident: the hardware then starts a workgroup wherever one has finished, which evens out the uneven shares
 // without any counter.  About kTasksPerWave tasks per wave, between one and eight resident sets.
-constexpr uint32_t kTasksPerWave = 8;
+constexpr uint32_t kTasksPerWave = 4;
 
 template <int kApp, int kWGT>
 int launch_hub_one(const fw_kargs& a, const fw_hub_args& h, uint32_t tasks_hint, hipStream_t stream) {
@@ -1974,9 +1975,10 @@ int launch_hub_app(const fw_kargs& a, const fw_hub_args& h, int wg_threads, uint
 
 // entries_hint (launches of the parking pipeline; 0 otherwise): about how many entries the launch will find.  Their
 // walkers are short-lived (a step or two until they are parked again), so a launch is a few rounds of refills plus
-// a tail of sparse rounds that every workgroup pays; fewer workgroups with kEntriesPerWorkgroup entries each
-// (but at least one per compute unit) spend less on that tail than a full resident set with a few refills each.
-constexpr int kEntriesPerWorkgroup = 2432;
+// a tail of sparse rounds that every workgroup pays.  kEntriesPerWorkgroup entries per workgroup, at least one
+// workgroup per compute unit and at most a resident set: large launches fill the device, small ones (the later rounds,
+// the smaller batches) take as many workgroups as give each about a refill and a half of its task table.
+constexpr int kEntriesPerWorkgroup = 700;
 
 template <int kApp, int kWGT>
 int launch_one(fw_kargs a, int grid, uint32_t entries_hint, hipStream_t stream, int* grid_used) {
