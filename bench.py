@@ -357,6 +357,15 @@ def main():
         out["roofline"]["no_parking"] = nop
         configs = [config1(fw)]
         configs.append(one_config(fw, g, "node2vec_rmat24_sym", WORKLOADS["node2vec_rmat24_sym"], passes=3, warmup=1))
+        # node2vec's two-stage step (propose by weight, accept by the node2vec factor) costs trials in proportion to
+        # q * max(1, 1/p) where most proposals are not adjacent to the previous vertex; the reference's one-pass sampler
+        # costs the same at every (p, q).  Two points away from the benchmark's, one pass each.
+        n2v_points = []
+        for pp, qq in ((4.0, 0.25), (0.25, 4.0)):
+            c = one_config(fw, g, "node2vec_rmat24_sym", WORKLOADS["node2vec_rmat24_sym"], passes=1, warmup=0, p=pp, q=qq)
+            c["config"] = "C4 at p = %g, q = %g" % (pp, qq)
+            c["p"], c["q"] = pp, qq
+            n2v_points.append(c)
         cpu = None if args.no_cpu else cpu_baseline(fw, g, params, starts, args.cpu_seconds)
         g.destroy()
         g22 = make_graph(fw, WORKLOADS["deepwalk_rmat22"])
@@ -379,6 +388,7 @@ def main():
             "algorithmic_frac": roofline["algorithmic_frac"], "algorithmic_rate_GBs": roofline["algorithmic_rate"],
             "reuse_factor": roofline["reuse_factor"]})
         out["configs"] = configs
+        out["node2vec_other_parameters"] = n2v_points
         if cpu is not None:
             out["cpu_baseline"] = cpu
     else:

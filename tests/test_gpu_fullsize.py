@@ -91,7 +91,8 @@ def test_config3_ppr_rmat22(gpu):
 
 
 def test_config4_rmat24_symmetrised(gpu):
-    """Headline graph: DeepWalk and node2vec (p = 2, q = 0.5), one query per vertex each, library defaults."""
+    """Headline graph: DeepWalk and node2vec (p = 2, q = 0.5, then two points where the acceptance step rejects more
+    often), one query per vertex each, library defaults."""
     g = gpu.Graph.rmat(24, 16, symmetrise=True, seed=1)
     try:
         assert g.is_sorted()
@@ -113,6 +114,17 @@ def test_config4_rmat24_symmetrised(gpu):
         L = _check_paths(xadj, adj, paths, starts, st, 81, sample=50000)
         assert (L[deg > 0] == 81).all()
         _check_rows_against_oracle(xadj, adj, w, None, p, starts, paths, k=700)
+        # away from the benchmark's parameters the two-stage step takes more trials per step (about q * max(1, 1/p)
+        # where most proposals are not adjacent to the previous vertex): many more pipeline rounds, the same law
+        for pp, qq in ((4.0, 0.25), (0.25, 4.0)):
+            del paths
+            p = gpu.default_params(app=gpu.APP_NODE2VEC, max_depth=81, p=pp, q=qq, seed=1)
+            print("node2vec p = %g, q = %g, %d queries" % (pp, qq, g.V), flush=True)
+            paths, st = g.walk(p, starts)
+            print("node2vec done: %.0f ms, %d launches" % (st.kernel_ms, st.launches), flush=True)
+            L = _check_paths(xadj, adj, paths, starts, st, 81, sample=50000)
+            assert (L[deg > 0] == 81).all()
+            _check_rows_against_oracle(xadj, adj, w, None, p, starts, paths, k=200)
     finally:
         g.destroy()
 
