@@ -44,6 +44,7 @@ class WalkParams(C.Structure):
         ("hub_threshold", C.c_int32), ("schema_len", C.c_int32), ("schema", C.c_int32 * FW_MAX_SCHEMA),
         ("tp", C.c_float), ("p", C.c_float), ("q", C.c_float), ("walker_base", C.c_uint32),
         ("seed", C.c_uint64), ("grid", C.c_int32), ("park_threshold", C.c_int32),
+        ("time_kernels", C.c_int32), ("reserved", C.c_int32),
     ]
 
 

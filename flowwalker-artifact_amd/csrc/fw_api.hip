@@ -1195,13 +1195,18 @@ struct KernelTimes {
 // to the parking buffers (created once with them, not per launch).
 struct TimedLaunch {
   hipEvent_t e0 = nullptr, e1 = nullptr;
+  bool enabled = true;  // an event costs the stream about 5 us: the per-kernel split is measured on request only
   bool open = false;
   int begin(hipStream_t s) {
+    if (!enabled) return FW_OK;
     FW_HIP(hipEventRecord(e0, s));
     open = true;
     return FW_OK;
   }
-  int end(hipStream_t s) { FW_HIP(hipEventRecord(e1, s)); return FW_OK; }
+  int end(hipStream_t s) {
+    if (enabled) FW_HIP(hipEventRecord(e1, s));
+    return FW_OK;
+  }
   void collect(double* acc) {  // call after the stream has been synchronised
     float ms = 0.0f;
     if (open && hipEventElapsedTime(&ms, e0, e1) == hipSuccess) *acc += ms;
@@ -1257,6 +1262,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
   TimedLaunch tw;
   tw.e0 = pb->ev[0];
   tw.e1 = pb->ev[1];
+  tw.enabled = p->time_kernels != 0;
   uint32_t entries_hint = 0u;  // set before every queue_walk
   // the hint counts entries of the kind the grid rule was made for, lists of up to 124 neighbours (four or two to a
   // wave); with a higher parking threshold an entry is more work, about in proportion
@@ -1392,6 +1398,7 @@ static int run_walk_launches(const fw_graph* g, const fw_walk_params* p, fw_karg
     TimedLaunch th;
     th.e0 = pb->ev[2];
     th.e1 = pb->ev[3];
+    th.enabled = p->time_kernels != 0;
     if ((rc = th.begin(stream)) != FW_OK) return rc;
     if (plan.two_pass_walkers != 0xFFFFFFFFu) {
       // finds its task count on the device; sized by the round before (twice that many tasks still get a wave each)
@@ -1599,7 +1606,7 @@ extern "C" int fw_walk_device(const fw_graph* g, const fw_walk_params* p, const 
     stats->sampled_edges = h.counters[1] + h.counters[3];
     stats->launches = launches;
     stats->grid = grid_used;
-    stats->walk_kernel_ms = launches == 1 ? (double)ms : times.walk_ms;
+    stats->walk_kernel_ms = launches == 1 ? (double)ms : times.walk_ms;  // the split: with time_kernels only
     stats->hub_kernel_ms = times.hub_ms;
     stats->hub_steps = h.counters[2];
     stats->hub_sampled_edges = h.counters[3];
@@ -1872,9 +1879,9 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     }
     stats->launches = nbatch;
     stats->grid = grid_used;
-    stats->walk_kernel_ms = times.hub_ms == 0.0 && times.walk_ms == 0.0 ? kernel_ms : times.walk_ms;
+    stats->walk_kernel_ms = stats->hub_steps == 0 ? kernel_ms : times.walk_ms;  // the split: with time_kernels only
     stats->hub_kernel_ms = times.hub_ms;
-    const TrafficModel tm = traffic_model(p, n, times.hub_ms != 0.0, park_threshold, g->adj_hub != nullptr,
+    const TrafficModel tm = traffic_model(p, n, times.sorted_records != 0, park_threshold, g->adj_hub != nullptr,
                                           stats->steps - stats->hub_steps,
                                           stats->sampled_edges - stats->hub_sampled_edges, stats->hub_steps, times);
     stats->requested_bytes = tm.total();

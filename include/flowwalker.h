@@ -100,6 +100,10 @@ typedef struct {
    * rejections of one step the next proposal is taken unconditionally (the trial count travels in 14 bits of a
    * record): at acceptance probabilities this library is meant for that never happens (0.94^16383), and where it
    * could (f / F below about 1e-3 for every neighbour) that step follows w / sum w instead of the node2vec law. */
+  int32_t time_kernels;  /* != 0: fw_walk_stats.walk_kernel_ms / hub_kernel_ms are measured too (two more events on the
+                            stream per launch; an event costs the stream about 5 us, which is 3 - 5 % of a pass made of
+                            many short launches).  0 (default): they stay 0, kernel_ms is measured as always. */
+  int32_t reserved;      /* 0 */
 } fw_walk_params;
 
 /* What src/main.cu:82-113 (calculate_workload) and the timing code of src/walk.cu report. */
@@ -111,8 +115,9 @@ typedef struct {
   int32_t launches;       /* fw_walk_batch: batches; fw_walk_device: walk + hub-batch kernel launches */
   int32_t grid;           /* workgroups per launch actually used */
   /* per-kernel breakdown of kernel_ms / steps / sampled_edges (hub parking splits a pass over two kernels) */
-  double walk_kernel_ms;      /* sum over fw_walk_zprs launches */
-  double hub_kernel_ms;       /* sum over the hub launches of every round: fw_hub_scan, fw_hub_batch, fw_hub_quad */
+  double walk_kernel_ms;      /* sum over fw_walk_zprs launches (with fw_walk_params.time_kernels, else 0) */
+  double hub_kernel_ms;       /* sum over the hub launches of every round: fw_hub_scan, fw_hub_batch, fw_hub_quad
+                                 (with fw_walk_params.time_kernels, else 0) */
   uint64_t hub_steps;         /* steps taken in the hub launches (included in steps) */
   uint64_t hub_sampled_edges; /* their source degrees (included in sampled_edges) */
   /* What the call's kernels asked of the memory, MODELLED from the run's own counters (steps, records moved, list

@@ -444,6 +444,32 @@ def test_reference_engine_with_thread_owned_generators(gpu, hub, sampler):
         g.destroy()
 
 
+def test_kernel_times_on_request(gpu):
+    """fw_walk_params.time_kernels: the split of kernel_ms over the walk and the hub launches is measured on request
+    only (an event pair per launch costs the stream time); the walks and the counters are the same either way."""
+    csr = _graphs.hub_graph(V=30000, hub_degrees=(20000, 8000), base_degree=8, seed=5)
+    g = gpu.Graph.from_csr(*csr)
+    try:
+        starts = np.random.RandomState(2).randint(0, 30000, size=200000).astype(np.int32)
+        p = gpu.default_params(app=gpu.APP_DEEPWALK, max_depth=21, seed=9)
+        plain, st0 = g.walk(p, starts)
+        assert st0.launches > 1 and st0.hub_steps > 0                      # the parking pipeline ran
+        assert st0.kernel_ms > 0.0 and st0.walk_kernel_ms == 0.0 and st0.hub_kernel_ms == 0.0
+        assert st0.requested_bytes > 0 and st0.scattered_writes > 0
+        p.time_kernels = 1
+        timed, st1 = g.walk(p, starts)
+        assert (timed == plain).all()
+        assert (st1.steps, st1.sampled_edges, st1.hub_steps, st1.launches) == \
+               (st0.steps, st0.sampled_edges, st0.hub_steps, st0.launches)
+        assert st1.requested_bytes == st0.requested_bytes
+        assert st1.walk_kernel_ms > 0.0 and st1.hub_kernel_ms > 0.0
+        assert st1.walk_kernel_ms + st1.hub_kernel_ms <= st1.kernel_ms
+        paths_b, stb = g.walk_batch(p, starts, batch_size=0)
+        assert (paths_b == plain).all() and stb.hub_kernel_ms > 0.0
+    finally:
+        g.destroy()
+
+
 def test_one_walk_call_at_a_time_per_graph(gpu):
     """The parking index, the parking lists and the launch record are cached in the fw_graph, so a second call on
     the same graph while one is running is refused with a status code (it used to race); afterwards the graph works

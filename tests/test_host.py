@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol(fw):
 
 def test_struct_layouts_match_the_header(fw):
     # fw_walk_params: 6 int32 + 64 int32 + 3 float + uint32 + uint64 + 2 int32
-    assert C.sizeof(fw.WalkParams) == 6 * 4 + 64 * 4 + 3 * 4 + 4 + 8 + 8
+    assert C.sizeof(fw.WalkParams) == 6 * 4 + 64 * 4 + 3 * 4 + 4 + 8 + 8 + 8
     assert C.sizeof(fw.WalkStats) == 8 + 8 + 8 + 8 + 4 + 4 + 8 + 8 + 8 + 8 + 8 + 4 * 8
     assert C.sizeof(fw.RmatParams) == 48
 
