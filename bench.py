@@ -366,8 +366,9 @@ def main():
         configs = [config1(fw)]
         configs.append(one_config(fw, g, "node2vec_rmat24_sym", WORKLOADS["node2vec_rmat24_sym"], passes=3, warmup=1))
         # node2vec's two-stage step (propose by weight, accept by the node2vec factor) costs trials in proportion to
-        # q * max(1, 1/p) where most proposals are not adjacent to the previous vertex; the reference's one-pass sampler
-        # costs the same at every (p, q).  Two points away from the benchmark's, one pass each.
+        # max(1, q) where most proposals are not adjacent to the previous vertex (and nothing for a small p: the return
+        # edge's excess is a component of its own); the reference's one-pass sampler costs the same at every (p, q).
+        # Two points away from the benchmark's, one pass each.
         n2v_points = []
         for pp, qq in ((4.0, 0.25), (0.25, 4.0)):
             c = one_config(fw, g, "node2vec_rmat24_sym", WORKLOADS["node2vec_rmat24_sym"], passes=1, warmup=0, p=pp, q=qq)

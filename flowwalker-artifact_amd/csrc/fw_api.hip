@@ -544,8 +544,8 @@ static void fill_kargs(fw_kargs* a, const fw_graph* g, const fw_walk_params* p) 
   a->inv_p = 1.0f / p->p;
   a->inv_q = 1.0f / p->q;
   a->n2v_fmax = 1.0f;
-  if (a->inv_p > a->n2v_fmax) a->n2v_fmax = a->inv_p;
   if (a->inv_q > a->n2v_fmax) a->n2v_fmax = a->inv_q;
+  a->n2v_extra = a->inv_p > a->n2v_fmax ? a->inv_p - a->n2v_fmax : 0.0f;
   a->schema_len = p->schema_len;
   for (int i = 0; i < FW_MAX_SCHEMA; ++i) a->schema[i] = (i < p->schema_len) ? p->schema[i] : 0;
   a->park_threshold = INT_MAX;

@@ -75,7 +75,9 @@ struct fw_kargs {
   uint32_t seed_lo, seed_hi;
   uint32_t walker_base;
   float tp, inv_p, inv_q;
-  float n2v_fmax;                    // max(1, 1/p, 1/q): the envelope of node2vec's acceptance test
+  float n2v_fmax;                    // F = max(1, 1/q): the envelope of node2vec's acceptance test
+  float n2v_extra;                   // 1/p - F when positive, else 0: the return edge's excess over the envelope, a
+                                     // component of its own of the trial
   int32_t schema_len;
   int32_t schema[FW_MAX_SCHEMA];
   // hub parking (park_threshold = INT32_MAX switches it off)

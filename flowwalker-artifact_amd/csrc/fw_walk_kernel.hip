@@ -80,6 +80,23 @@ __device__ __forceinline__ bool sorted_contains(const int32_t* __restrict__ arr,
   return false;
 }
 
+// Sum of the weights of the entries of the ascending list adj[0, size) that equal `target`, added in list order
+// (0 when there is none): the return edges of a node2vec step.
+__device__ __forceinline__ float return_weight(const int32_t* __restrict__ adj, const float* __restrict__ w, uint32_t size,
+                                               int32_t target) {
+  uint32_t lo = 0u, hi = size;  // first entry that is not smaller
+  while (lo < hi) {
+    const uint32_t mid = (lo + hi) >> 1;
+    if (adj[mid] < target) lo = mid + 1u; else hi = mid;
+  }
+  float sum = 0.0f;
+  while (lo < size && adj[lo] == target) {
+    sum = sum + w[lo];
+    ++lo;
+  }
+  return sum;
+}
+
 // The same question answered by a whole wave for one (wave-uniform) list and target: 64 probes per round instead
 // of one, so a list of 100,000 entries takes three dependent loads instead of seventeen.  Lane l probes the last
 // entry of the l-th of 64 chunks; the entries ascend, so the lanes whose probe is smaller than the target form a
@@ -134,23 +151,35 @@ __device__ __forceinline__ bool segment_contains(const int32_t* __restrict__ arr
 
 // The acceptance test u * F < f of trial `trial` at (walker, step) in two halves, so that the search for the proposal
 // in N(prev) is only made when its answer matters: f is 1/p for the return edge, else 1 (common neighbour) or 1/q, so a
-// threshold u * F below both is accepted and one that reaches both is rejected whichever it is.
+// threshold u * F below both is accepted and one that reaches both is rejected whichever it is.  F = max(1, 1/q).
+// When 1/p is larger than that (a.n2v_extra = 1/p - F > 0) the return edge's excess is a component of its own: with T
+// the list's total as the sampler added it up and w_ret the weights of the entries that lead back to prev, the trial
+// takes the return edge outright when u0 (F T + extra w_ret) < extra w_ret (take_prev), and otherwise the return
+// edge among the proposals is always accepted.  The number of trials then does not depend on p.
 struct N2vTest {
   float uF;          // u * F
   bool decided;      // no search needed
   bool accept;       // the decision when decided
+  bool take_prev;    // the step goes back to the previous vertex whatever was proposed
 };
 
 __device__ __forceinline__ N2vTest n2v_test(const fw_kargs& a, int32_t post, int32_t prev, uint32_t walker, uint32_t step,
-                                            uint32_t trial) {
+                                            uint32_t trial, float T, float w_ret) {
   N2vTest t;
   t.uF = 0.0f;
   t.decided = true;
   t.accept = true;
+  t.take_prev = false;
   if (prev == -1 || trial == kMaxTrials - 1u) return t;
-  const uint32_t bits = philox4x32_10(walker, step, kStreamAccept | (trial << 8), 0u, a.seed_lo, a.seed_hi).x;
-  t.uF = u24(bits) * a.n2v_fmax;
-  if (post == prev) {
+  const uint4 bits = philox4x32_10(walker, step, kStreamAccept | (trial << 8), 0u, a.seed_lo, a.seed_hi);
+  t.uF = u24(bits.x) * a.n2v_fmax;
+  if (a.n2v_extra > 0.0f) {
+    const float gx = a.n2v_extra * w_ret;
+    const float gb = a.n2v_fmax * T;
+    const float lhs0 = u24(bits.y) * (gb + gx);
+    t.take_prev = lhs0 < gx;
+    if (t.take_prev || post == prev) return t;
+  } else if (post == prev) {
     t.accept = t.uF < a.inv_p;
     return t;
   }
@@ -384,10 +413,20 @@ __device__ __forceinline__ StepCtx load_ctx(const fw_kargs& a, const TaskTable<k
 
 // node2vec, all lanes of the wave: is the (wave-uniform) proposal v of the step accepted?  The lanes look it up in
 // N(prev) together when the answer matters.
+// T: the list's total as the step's sampler added it up.  v becomes the previous vertex when the trial takes the
+// return edge's own component.
 template <int kApp>
-__device__ __forceinline__ bool n2v_wave_accept(const fw_kargs& a, const StepCtx& c, int32_t v, bool ok, int lane) {
+__device__ __forceinline__ bool n2v_wave_accept(const fw_kargs& a, const StepCtx& c, int32_t& v, bool ok, int lane,
+                                                float T) {
   if (kApp != FW_APP_NODE2VEC || !ok) return true;
-  const N2vTest t = n2v_test(a, v, c.prev, c.walker, c.step, c.sbase >> 8);  // wave-uniform
+  float w_ret = 0.0f;
+  if (a.n2v_extra > 0.0f && c.prev >= 0)  // wave-uniform: every lane walks the same few entries
+    w_ret = return_weight(a.adjncy + c.off, a.weight + c.off, (uint32_t)c.deg, c.prev);
+  const N2vTest t = n2v_test(a, v, c.prev, c.walker, c.step, c.sbase >> 8, T, w_ret);  // wave-uniform
+  if (t.take_prev) {
+    v = c.prev;
+    return true;
+  }
   bool common = false;
   if (!t.decided) common = wave_contains(a.adjncy + c.prev_off, (uint32_t)c.prev_deg, v, lane);
   return n2v_finish(a, t, common);
@@ -535,16 +574,43 @@ __device__ __forceinline__ void packed_finish(const fw_kargs& a, TaskTable<kWGT,
   v = pick == 1 ? adj.y : v;
   v = pick == 2 ? adj.z : v;
   v = pick == 3 ? adj.w : v;
-  const int32_t selv = __builtin_amdgcn_ds_bpermute((seg_first + l) << 2, v);
+  int32_t selv = __builtin_amdgcn_ds_bpermute((seg_first + l) << 2, v);
   bool n2v_ok = true;
   if (kApp == FW_APP_NODE2VEC) {  // selv is a proposal: the acceptance test, its search made by the segment's lanes together
     N2vTest t;
-    t.uF = 0.0f; t.decided = true; t.accept = true;
+    t.uF = 0.0f; t.decided = true; t.accept = true; t.take_prev = false;
     uint32_t psize = 0u;
     const int32_t* plist = a.adjncy;
+    float w_ret = 0.0f;
+    if (a.n2v_extra > 0.0f) {
+      // The weights of the entries that lead back to the previous vertex, added in list order.  The entries are in
+      // the lanes' registers (lane k of the segment holds quartet k); they follow each other in the list, so they sit
+      // in one lane or in a few neighbouring ones, which are visited in order.
+      const int32_t pv = active ? tt.prev[slot] : -1;
+      uint32_t mine = 0u;  // which of this lane's four entries lead back
+      mine |= (li < lim && adj.x == pv) ? 1u : 0u;
+      mine |= (li + 1u < lim && adj.y == pv) ? 2u : 0u;
+      mine |= (li + 2u < lim && adj.z == pv) ? 4u : 0u;
+      mine |= (li + 3u < lim && adj.w == pv) ? 8u : 0u;
+      uint32_t rest = (uint32_t)(__ballot(mine != 0u) >> seg_first) & seg_mask;
+      while (__ballot(rest != 0u) != 0ull) {
+        const int from = (seg_first + (rest != 0u ? __builtin_ctz(rest) : 0)) << 2;
+        const uint32_t their = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)mine);
+        const float y0 = bperm_f(from, x[0]), y1 = bperm_f(from, x[1]);
+        const float y2 = bperm_f(from, x[2]), y3 = bperm_f(from, x[3]);
+        if (rest != 0u) {
+          if (their & 1u) w_ret = w_ret + y0;
+          if (their & 2u) w_ret = w_ret + y1;
+          if (their & 4u) w_ret = w_ret + y2;
+          if (their & 8u) w_ret = w_ret + y3;
+          rest &= rest - 1u;
+        }
+      }
+    }
     if (active && accept) {
       t = n2v_test(a, selv, tt.prev[slot], a.walker_base + (uint32_t)tt.walker[slot], (uint32_t)(len - 1),
-                   (uint32_t)tt.trial[slot]);  // the same in every lane of the segment
+                   (uint32_t)tt.trial[slot], T, w_ret);  // the same in every lane of the segment
+      if (t.take_prev) selv = tt.prev[slot];
       if (!t.decided) {
         plist = a.adjncy + tt.prev_off[slot];
         psize = (uint32_t)tt.prev_deg[slot];
@@ -690,7 +756,7 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
           }
           int32_t v = -1;
           if (pick >= 0) v = a.adjncy[c.off + (uint32_t)pick];  // wave-uniform
-          const bool accepted = n2v_wave_accept<kApp>(a, c, v, pick >= 0, lane);
+          const bool accepted = n2v_wave_accept<kApp>(a, c, v, pick >= 0, lane, total);
           if (lane == 0) commit(a, tt, slot, c, v, pick >= 0, accepted, n_steps, n_edges);
         }
         if (hb + kHubChunk < nh) __syncthreads();  // the partial buffers are reused by the next chunk
@@ -757,7 +823,7 @@ __global__ __launch_bounds__(kWGT, kPackedInFlight == 1 ? 8 : 4) void fw_walk_zp
           wave_stream<kApp, kGroupQuartets, false>(a, c, lane, 0u, 1u, dq0, W, sel, selv);
           if (sel >= 0) v = a.adjncy[c.off + (uint32_t)sel];
         }
-        const bool accepted = n2v_wave_accept<kApp>(a, c, v, sel >= 0, lane);
+        const bool accepted = n2v_wave_accept<kApp>(a, c, v, sel >= 0, lane, W);
         if (lane == 0) commit(a, tt, slot, c, v, sel >= 0, accepted, n_steps, n_edges);
       }
       __syncthreads();
@@ -1256,7 +1322,8 @@ __device__ __forceinline__ int32_t resolve_pick(const uint32_t* __restrict__ bia
 // test that failed on S fails again.
 __device__ __forceinline__ void table_reservoir(const fw_kargs& a, const float* totals, const uint32_t ngroups,
                                                 const uint32_t seq, const uint32_t nw, const uint32_t walker,
-                                                const uint32_t step, const uint32_t sbase, int32_t& gsel, float& tsel) {
+                                                const uint32_t step, const uint32_t sbase, int32_t& gsel, float& tsel,
+                                                float& S_out) {
   float S = 0.0f, Sj = 0.0f, u = 1.0f;
   LaneDraw dq;
   gsel = -1;
@@ -1280,6 +1347,7 @@ __device__ __forceinline__ void table_reservoir(const fw_kargs& a, const float* 
       S = Snew;
     }
   }
+  S_out = S;
 }
 
 // A step of up to 64 walkers (lane i = walker i) on a hub whose rows are made: returns each walker's local index
@@ -1289,12 +1357,13 @@ __device__ __forceinline__ int32_t table_sample(const fw_kargs& a, const uint32_
                                                 const uint32_t deg, const int32_t want, const bool wg, const bool have,
                                                 const uint32_t walker, const uint32_t step, const uint32_t sbase,
                                                 const int lane, const float* totals, const float* rows,
-                                                const int32_t* lastpos) {
+                                                const int32_t* lastpos, float& total_out) {
   constexpr uint32_t kG = 64u * kGroupQuartets;
   const uint32_t nq = (off + deg - (off & ~3u) + 3u) >> 2;
   const uint32_t ngroups = (nq + kG - 1u) / kG;
   const uint32_t nw = wg ? (uint32_t)kNW : 1u;
   int wsel = 0;
+  total_out = 0.0f;
   if (wg) {
     // the sequences' totals, each added up in its own order by one lane, then the inverse transform over them
     float Wl = 0.0f;
@@ -1312,6 +1381,7 @@ __device__ __forceinline__ int32_t table_sample(const fw_kargs& a, const uint32_
     }
     const float J = row_scan(Wl);
     const float total = readlane_f(J, kNW - 1);
+    total_out = total;
     const float target = u24(philox4x32_10(walker, step, kStreamWave | sbase, 0u, a.seed_lo, a.seed_hi).x) * total;
     int wlast = -1;
     wsel = -1;
@@ -1329,7 +1399,9 @@ __device__ __forceinline__ int32_t table_sample(const fw_kargs& a, const uint32_
   // only the sequence the walker ends up in needs running: the draws of a sequence are addressed by the sequence
   int32_t gsel = -1;
   float tsel = 0.0f;
-  if (have && wsel >= 0) table_reservoir(a, totals, ngroups, (uint32_t)wsel, nw, walker, step, sbase, gsel, tsel);
+  float S_seq = 0.0f;  // the total of the sequence the reservoir ran over: the list's total at wave granularity
+  if (have && wsel >= 0) table_reservoir(a, totals, ngroups, (uint32_t)wsel, nw, walker, step, sbase, gsel, tsel, S_seq);
+  if (!wg) total_out = S_seq;
   int32_t pick = -1;
   if (gsel >= 0) pick = resolve_pick<kApp>(bias, off, deg, want, rows, lastpos, gsel, tsel);
   return pick;
@@ -1353,13 +1425,14 @@ __device__ __forceinline__ fw_walker_rec load_parked(const void* sorted, uint32_
 
 // v, off, deg: the list the lane's walker stands on (the same in every lane, or one list per 16-lane row with
 // kPerLane, where every lane then counts its own step); out_at: the walker's position in the output list.
+// T (node2vec): the list's total as the step's sampler added it up.
 template <int kApp, bool kPerLane = false>
 __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_args& h, const int32_t v,
                                              const uint32_t off, const uint32_t deg, const uint32_t out_at,
                                              const fw_walker_rec rec, const uint32_t trial, const bool have,
                                              const int32_t pick, const uint32_t walker, const uint32_t step,
                                              const int lane, unsigned long long& n_steps,
-                                             unsigned long long& n_edges, uint32_t (&n_out)[2]) {
+                                             unsigned long long& n_edges, uint32_t (&n_out)[2], const float T = 0.0f) {
   bool moved = have && pick >= 0;
   bool retry = false;
   bool go_on = false;
@@ -1374,15 +1447,22 @@ __device__ __forceinline__ void batch_commit(const fw_kargs& a, const fw_hub_arg
       nv = a.adjncy[off + (uint32_t)pick];
     }
     if (kApp == FW_APP_NODE2VEC && rec.prev >= 0) {
-      const N2vTest t = n2v_test(a, nv, rec.prev, walker, step, trial);
-      bool common = false;
-      if (!t.decided) {
-        const uint32_t po = a.xadj[rec.prev];
-        common = sorted_contains(a.adjncy + po, (int32_t)(a.xadj[rec.prev + 1] - po), nv);
-      }
-      if (!n2v_finish(a, t, common)) {
-        moved = false;
-        retry = true;
+      float w_ret = 0.0f;  // T: the list's total as the step's sampler added it up
+      if (a.n2v_extra > 0.0f) w_ret = return_weight(a.adjncy + off, a.weight + off, deg, rec.prev);
+      const N2vTest t = n2v_test(a, nv, rec.prev, walker, step, trial, T, w_ret);
+      if (t.take_prev) {  // the return edge's own component: back to the previous vertex
+        nv = rec.prev;
+        if (a.adj_hub != nullptr) nv_hidx = a.hub_index[nv];
+      } else {
+        bool common = false;
+        if (!t.decided) {
+          const uint32_t po = a.xadj[rec.prev];
+          common = sorted_contains(a.adjncy + po, (int32_t)(a.xadj[rec.prev + 1] - po), nv);
+        }
+        if (!n2v_finish(a, t, common)) {
+          moved = false;
+          retry = true;
+        }
       }
     }
   }
@@ -1527,11 +1607,12 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     const uint32_t walker = a.walker_base + (uint32_t)rec.q;
     const uint32_t step = (uint32_t)(rec.len - 1);
 
+    float T = 0.0f;
     const int32_t sel = table_sample<kApp, kNW>(a, bias, off, deg, want, (int32_t)deg > a.hub_threshold, have, walker,
                                                step, trial << 8, lane, h.totals + row_base,
-                                               h.rows + (size_t)row_base * 128u, h.lastpos + row_base);
+                                               h.rows + (size_t)row_base * 128u, h.lastpos + row_base, T);
     batch_commit<kApp>(a, h, v, off, deg, rec_base + (uint32_t)lane, rec, trial, have, sel, walker, step, lane, n_steps,
-                       n_edges, n_out);
+                       n_edges, n_out, T);
   }
 
   // ---- then wave tasks: lists up to hub_threshold, sampled at wave granularity, one batch per wave; the tasks are
@@ -1561,7 +1642,7 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
     int32_t sel;
     batch_stream<kApp>(a, bias, off, deg, want, 0u, 1u, have, walker, step, trial << 8, lane, S, sel);
     batch_commit<kApp>(a, h, v, off, deg, rec_base + (uint32_t)lane, rec, trial, have, sel, walker, step, lane, n_steps,
-                       n_edges, n_out);
+                       n_edges, n_out, S);
   }
 
   // ---- then workgroup tasks: lists above hub_threshold, sampled at workgroup granularity.  They are few, long and
@@ -1623,7 +1704,7 @@ __global__ __launch_bounds__(kWGT, 8) void fw_hub_batch(const fw_kargs a, const 
         if (wsel >= 0) pick = s_sel[wsel][lane];
       }
       batch_commit<kApp>(a, h, task.v, task.off, task.deg, task.rec_base + (uint32_t)lane, rec, trial, have, pick, walker,
-                         step, lane, n_steps, n_edges, n_out);
+                         step, lane, n_steps, n_edges, n_out, total);
     }
   }
 
@@ -1813,7 +1894,7 @@ __global__ __launch_bounds__(256, 8) void fw_hub_quad(const fw_kargs a, const fw
       }
       __builtin_amdgcn_wave_barrier();  // the rows are rewritten by the wave's next four tasks
       batch_commit<kApp, true>(a, h, task.v, task.off, task.deg, task.rec_base + (uint32_t)rl, rec, trial, have, sel, walker,
-                               step, lane, n_steps, n_edges, n_out);
+                               step, lane, n_steps, n_edges, n_out, T);
     }
   }
 

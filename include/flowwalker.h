@@ -92,14 +92,17 @@ typedef struct {
                             for batches >= 65536 queries), < 0 = off, > 0 = degree.  node2vec: the shared scan
                             proposes, each walker accepts with its own adjacency test (max_depth <= 65535). */
   /* node2vec is sampled in two stages: a neighbour is proposed with probability w / sum w and accepted with
-   * probability f / F, f = 1/p (return edge), 1 (common neighbour of the previous vertex) or 1/q, F = max(1, 1/p,
-   * 1/q); a rejected walker proposes again.  The accepted neighbour has the reference's law w f / sum w f
-   * (include/app.cuh:97-127) exactly, but the work per step follows the parameters: the expected number of proposals
-   * is F * sum w / sum w f (1.3 at p = 2, q = 0.5 on the R-MAT benchmark graph, about 4 at p = q = 4, about 16 at
-   * p = 0.25, q = 4), where the reference's one pass over the biases costs the same whatever p and q.  After 16,383
-   * rejections of one step the next proposal is taken unconditionally (the trial count travels in 14 bits of a
-   * record): at acceptance probabilities this library is meant for that never happens (0.94^16383), and where it
-   * could (f / F below about 1e-3 for every neighbour) that step follows w / sum w instead of the node2vec law. */
+   * probability f / F, f = 1 (common neighbour of the previous vertex) or 1/q, F = max(1, 1/q); a rejected walker
+   * proposes again.  The return edge (f = 1/p) is accepted with probability (1/p) / F when that is at most 1; when 1/p
+   * is larger, a trial first takes the return edge outright with the probability its excess (1/p - F) w has in the
+   * envelope F sum w + (1/p - F) w, and otherwise accepts it whenever it is proposed.  The accepted neighbour has the
+   * reference's law w f / sum w f (include/app.cuh:97-127) exactly.  The work per step does not depend on p, but it
+   * follows q: the expected number of proposals is about F sum w / sum w f (1.3 at p = 2, q = 0.5 on the R-MAT
+   * benchmark graph, where few proposals are common neighbours; about q for q > 1: 4 at q = 4), where the reference's
+   * one pass over the biases costs the same whatever p and q.  After 16,383 rejections of one step the next proposal
+   * is taken unconditionally (the trial count travels in 14 bits of a record): at acceptance probabilities this library
+   * is meant for that never happens (0.94^16383), and where it could (q above about 1000) that step follows w / sum w
+   * instead of the node2vec law. */
   int32_t time_kernels;  /* != 0: fw_walk_stats.walk_kernel_ms / hub_kernel_ms are measured too (two more events on the
                             stream per launch; an event costs the stream about 5 us, which is 3 - 5 % of a pass made of
                             many short launches).  0 (default): they stay 0, kernel_ms is measured as always. */

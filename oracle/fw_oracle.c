@@ -45,13 +45,20 @@
  *       common neighbour of prev and cur, 1/q otherwise; include/app.cuh:108-123) of EVERY neighbour, one binary
  *       search each, inside its one-pass sampler.  Here a trial proposes a neighbour with probability w_i / sum w
  *       through the same sampler DeepWalk uses (no adjacency test at all) and accepts it with probability f_i / F,
- *       F = max(1, 1/p, 1/q), which takes ONE adjacency test (include/gpu_graph.cuh:97-118); a rejected trial is
+ *       F = max(1, 1/q), which takes ONE adjacency test (include/gpu_graph.cuh:97-118); a rejected trial is
  *       followed by another with its own draws.  P(i) = (w_i / sum w)(f_i / F) / sum_j (w_j / sum w)(f_j / F) =
  *       w_i f_i / sum_j w_j f_j: the reference's law exactly (its own rejection sampler has the same structure,
- *       include/sampler.cuh:202-266).  Draws of trial t use the streams of a plain step offset by t << 8; the
- *       acceptance uniform is word 0 of block 0 of stream FW_STREAM_ACCEPT | t << 8; trial FW_MAX_TRIALS - 1 is accepted
- *       unconditionally (never reached in practice: the acceptance probability is at least min(f) / F).
- *       f uses host-computed f32 reciprocals 1/p and 1/q; the test is u * F < f, no division.
+ *       include/sampler.cuh:202-266).  When 1/p exceeds F, the return edge is the one neighbour the envelope w F does
+ *       not cover, and raising F to 1/p would make every other proposal 1/(p F) times less likely to be accepted.
+ *       Its excess is a component of its own instead: with T the list's total as the sampler adds it up and R the
+ *       weights of the entries that lead back to prev (f32, list order), a trial takes the return edge outright when
+ *       u0 (F T + (1/p - F) R) < (1/p - F) R, and otherwise runs as above with the return edge always accepted
+ *       (envelope w F for every entry plus (1/p - F) w for the return entries: total mass of an entry w f, as above).
+ *       So the number of trials does not depend on p.  Draws of trial t use the streams of a plain step offset by
+ *       t << 8; the acceptance uniform is word 0 and u0 word 1 of block 0 of stream FW_STREAM_ACCEPT | t << 8; trial
+ *       FW_MAX_TRIALS - 1 is accepted unconditionally (never reached in practice: the acceptance probability is at
+ *       least min(1, 1/q) / F).  f uses host-computed f32 reciprocals 1/p and 1/q; the tests are u * F < f and the
+ *       one above, no division.
  *   - --dprs selects nothing different: the one sampler already has DPRS's property (one bias
  *       evaluation per neighbour, include/sampler.cuh:129-200), so FW_SAMPLER_DPRS is an alias.
  *
@@ -266,7 +273,8 @@ static int pick_by_prefix(const float* v, const float* prefix, int n, float targ
  * Waves are combined by one more inverse transform on the row scan of the wave totals.
  */
 static int32_t group_sample(const bias_ctx* c, uint32_t off, int32_t deg, int nw, uint32_t walker,
-                            uint32_t step) {
+                            uint32_t step, float* total_out) {
+  if (total_out) *total_out = 0.0f;
   if (deg <= 0) return -1;
   enum { U = FW_GROUP_QUARTETS, EL = FW_EL, G = FW_WAVE * FW_GROUP_QUARTETS };
   const uint64_t a0 = (uint64_t)off & ~(uint64_t)(FW_QUAD - 1);
@@ -328,11 +336,15 @@ static int32_t group_sample(const bias_ctx* c, uint32_t off, int32_t deg, int nw
     W[wv] = S;
     wsel[wv] = sel;
   }
-  if (nw == 1) return wsel[0];
+  if (nw == 1) {
+    if (total_out) *total_out = W[0];
+    return wsel[0];
+  }
 
   float J[16];
   for (int wv = 0; wv < nw; ++wv) J[wv] = W[wv];
   row_scan(J, nw);
+  if (total_out) *total_out = J[nw - 1];
   const float u3 = step_draw(c, walker, step, FW_STREAM_WAVE, 0u);
   const float target = u3 * J[nw - 1];
   const int wv = pick_by_prefix(W, J, nw, target);
@@ -370,17 +382,37 @@ int32_t fw_oracle_sample(const fw_oracle_graph* g, const fw_oracle_params* p, in
     free(u);
     return sel;
   }
-  if (p->app != FW_APP_NODE2VEC || prev < 0) return group_sample(&c, off, deg, nw, walker, step);
-  /* node2vec after the first step: propose by weight, accept by f / F (include/app.cuh:108-123 for f) */
+  if (p->app != FW_APP_NODE2VEC || prev < 0) return group_sample(&c, off, deg, nw, walker, step, NULL);
+  /* node2vec after the first step: propose by weight, accept by f / F (include/app.cuh:108-123 for f).  F covers the
+   * common neighbours and the others; the return edge's excess over it is a component of its own (header). */
   float F = 1.0f;
-  if (p->inv_p > F) F = p->inv_p;
   if (p->inv_q > F) F = p->inv_q;
+  const float extra = p->inv_p > F ? p->inv_p - F : 0.0f;
+  float w_ret = 0.0f;     /* weights of the entries of N(cur) that lead back to prev, in list order */
+  int32_t first_ret = -1;
+  if (extra > 0.0f) {
+    for (int32_t i = 0; i < deg; ++i) {
+      if (g->adjncy[(uint64_t)off + (uint32_t)i] == prev) {
+        if (first_ret < 0) first_ret = i;
+        w_ret = w_ret + bias_at(&c, (uint64_t)off + (uint32_t)i);
+      }
+    }
+  }
   for (uint32_t trial = 0;; ++trial) {
     c.stream_base = trial << 8;
-    const int32_t sel = group_sample(&c, off, deg, nw, walker, step);
+    float T = 0.0f;
+    const int32_t sel = group_sample(&c, off, deg, nw, walker, step, &T);
     if (sel < 0) return -1; /* no positive weight: dead end, whatever the trial */
     if (trial == FW_MAX_TRIALS - 1u) return sel;
     const int32_t post = g->adjncy[(uint64_t)off + (uint32_t)sel];
+    if (extra > 0.0f) {
+      const float u0 = u24(draw_bits(p->seed, walker, step, FW_STREAM_ACCEPT | (trial << 8), 1u));
+      const float gx = extra * w_ret;
+      const float gb = F * T;
+      const float lhs0 = u0 * (gb + gx);
+      if (lhs0 < gx) return first_ret; /* the return edge's own component (gx > 0: there is such an entry) */
+      if (post == prev) return sel;    /* its share of the proposals is never turned down */
+    }
     float f;
     if (post == prev) f = p->inv_p;
     else if (sorted_contains(g->adjncy + c.prev_off, c.prev_deg, post)) f = 1.0f;
@@ -706,7 +738,7 @@ int fw_oracle_enumerate_draw(const float* bias, int32_t deg, uint32_t off, int32
 #pragma omp for schedule(static)
       for (int64_t v = 0; v < (1 << 24); ++v) {
         c.force_value = (float)v * 0x1p-24f;
-        const int32_t s = group_sample(&c, off, deg, nw, walker, step);
+        const int32_t s = group_sample(&c, off, deg, nw, walker, step, NULL);
         mine[s + 1] += 1;
       }
 #pragma omp critical
@@ -737,7 +769,7 @@ int32_t fw_oracle_sample_forced(const float* bias, int32_t deg, uint32_t off, in
   memset(&c, 0, sizeof(c));
   c.g = &g; c.p = &p; c.prev = -1;
   c.force = 1; c.force_stream = stream; c.force_index = index; c.force_value = value;
-  const int32_t sel = group_sample(&c, off, deg, nw, walker, step);
+  const int32_t sel = group_sample(&c, off, deg, nw, walker, step, NULL);
   free(padded);
   return sel;
 }

@@ -67,9 +67,12 @@ def test_ppr_lengths(gpu, hub_graph):
     assert abs(L[ok].mean() - 1 / tp) < 0.2
 
 
-def test_node2vec_second_step_frequencies(gpu):
+@pytest.mark.parametrize("pp,qq", [(2.0, 0.5), (0.25, 4.0), (0.02, 1.0), (0.4, 0.5)])
+def test_node2vec_second_step_frequencies(gpu, pp, qq):
     """Vertex P hangs on hub H with a heavy edge and shares 60 neighbours with it.  From P the first step goes to H
-    almost surely; the second step must follow w/p (back to P), w (common neighbours), w/q (others)."""
+    almost surely; the second step must follow w/p (back to P), w (common neighbours), w/q (others).  With 1/p above
+    max(1, 1/q) the return edge's excess is a component of its own of the trial (the last three points; at p = 0.02 a
+    good part of the steps goes back)."""
     rng = np.random.RandomState(3)
     V, H, P = 20000, 0, 1
     hub_nb = rng.choice(np.arange(2, V), size=6000, replace=False)
@@ -84,7 +87,6 @@ def test_node2vec_second_step_frequencies(gpu):
     w = wu[inv]
     w[(pair == min(H, P) * V + max(H, P))] = 1.0e6
     g = gpu.Graph.from_csr(xadj, adj, w)
-    pp, qq = 2.0, 0.5
     try:
         for thr in (1 << 30, 1024):
             prm = gpu.default_params(app=gpu.APP_NODE2VEC, max_depth=3, p=pp, q=qq, hub_threshold=thr, seed=thr % 97)

@@ -114,8 +114,9 @@ def test_config4_rmat24_symmetrised(gpu):
         L = _check_paths(xadj, adj, paths, starts, st, 81, sample=50000)
         assert (L[deg > 0] == 81).all()
         _check_rows_against_oracle(xadj, adj, w, None, p, starts, paths, k=700)
-        # away from the benchmark's parameters the two-stage step takes more trials per step (about q * max(1, 1/p)
-        # where most proposals are not adjacent to the previous vertex): many more pipeline rounds, the same law
+        # away from the benchmark's parameters: q > 1 takes about q trials per step where most proposals are not
+        # adjacent to the previous vertex (more pipeline rounds), and 1/p > max(1, 1/q) makes the return edge's excess a
+        # component of its own of every trial; the same law
         for pp, qq in ((4.0, 0.25), (0.25, 4.0)):
             del paths
             p = gpu.default_params(app=gpu.APP_NODE2VEC, max_depth=81, p=pp, q=qq, seed=1)

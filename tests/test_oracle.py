@@ -209,14 +209,16 @@ def test_node2vec_reduces_to_deepwalk_for_p_q_one(hub_csr):
     assert (a == b).all()
 
 
-def test_node2vec_second_step_distribution(hub_csr):
-    """From a fixed (prev, cur): weights w/p for the return edge, w for common neighbours, w/q otherwise."""
+@pytest.mark.parametrize("pp,qq", [(2.0, 0.5), (0.25, 4.0), (0.25, 1.0), (0.4, 0.5), (0.05, 0.5)])
+def test_node2vec_second_step_distribution(hub_csr, pp, qq):
+    """From a fixed (prev, cur): weights w/p for the return edge, w for common neighbours, w/q otherwise.  With 1/p
+    above max(1, 1/q) the return edge's excess is a component of its own (the last four points; at p = 0.05 it takes
+    most of the steps)."""
     xadj, adj, w, lab = hub_csr
     g = orc.Graph(xadj, adj, w, lab)
     prev = 1                                    # the 900-degree hub
     nb = adj[xadj[prev]:xadj[prev + 1]]
     cur = int(nb[np.argmax(np.diff(xadj.astype(np.int64))[nb])])
-    pp, qq = 2.0, 0.5
     p = orc.make_params(app=2, max_depth=3, p=pp, q=qq, seed=31)
     lo, hi = int(xadj[cur]), int(xadj[cur + 1])
     prev_set = set(nb.tolist())
@@ -229,6 +231,32 @@ def test_node2vec_second_step_distribution(hub_csr):
     for walker in range(n):
         s = orc.sample(g, p, cur, prev, walker, 1)
         cnt[adj[lo + s]] += 1
+    m = exp > 0
+    assert cnt[~m].sum() == 0
+    assert chisquare(cnt[m], exp[m] * n / exp.sum()).pvalue > 0.01
+
+
+@pytest.mark.parametrize("pp,qq", [(0.25, 4.0), (0.3, 0.7), (3.0, 2.0)])
+def test_node2vec_return_edges_of_a_multigraph(pp, qq):
+    """Several entries of N(cur) lead back to prev, with weights of their own: every one of them carries w / p, so the
+    vertex prev is taken in proportion to their sum (brute force over the entries)."""
+    # vertex 0 = cur: three edges to 1 (prev), one each to 2 (common neighbour of prev), 3, 4, 5; vertex 1: 0, 2, 6
+    lists = {0: [1, 1, 1, 2, 3, 4, 5], 1: [0, 2, 6], 2: [0, 1], 3: [0], 4: [0], 5: [0], 6: [1]}
+    V = 7
+    xadj = np.zeros(V + 1, dtype=np.uint32)
+    np.cumsum([len(lists[v]) for v in range(V)], out=xadj[1:])
+    adj = np.concatenate([lists[v] for v in range(V)]).astype(np.int32)
+    w = (1.0 + 9.0 * np.random.RandomState(8).random_sample(len(adj))).astype(np.float32)
+    g = orc.Graph(xadj, adj, w, None)
+    p = orc.make_params(app=2, max_depth=3, p=pp, q=qq, seed=77)
+    exp = np.zeros(V)
+    for i in range(int(xadj[0]), int(xadj[1])):
+        t = int(adj[i])
+        exp[t] += w[i] / pp if t == 1 else (w[i] if t in (0, 2, 6) else w[i] / qq)
+    n = 200000
+    cnt = np.zeros(V)
+    for walker in range(n):
+        cnt[adj[orc.sample(g, p, 0, 1, walker, 1)]] += 1
     m = exp > 0
     assert cnt[~m].sum() == 0
     assert chisquare(cnt[m], exp[m] * n / exp.sum()).pvalue > 0.01
