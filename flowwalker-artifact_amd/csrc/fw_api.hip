@@ -312,6 +312,7 @@ static int alloc_edge_array(T** out, uint64_t E, const T* h_src, int host_pinned
 }
 
 static void release_park_cache(fw_graph* g);  // defined with the parking buffers below
+static void release_batch_cache(fw_graph* g);
 
 extern "C" int fw_graph_destroy(fw_graph* g) {
   if (!g) return FW_OK;
@@ -324,6 +325,7 @@ extern "C" int fw_graph_destroy(fw_graph* g) {
     }
   }
   release_park_cache(g);
+  release_batch_cache(g);
   for (hipEvent_t e : g->call_ev) if (e) (void)hipEventDestroy(e);
   void* index_ptrs[4] = {g->hub_index, g->hub_info, g->call_scratch, g->adj_hub};
   for (void* p : index_ptrs) {
@@ -1154,6 +1156,57 @@ static ParkBuffers* cached_park_buffers(fw_graph* g, size_t n, int n_buckets, ui
   return c;
 }
 
+struct Scratch {  // dispenser word + workload counters of the two kernels, 48 bytes per launch slot
+  uint32_t dispenser;
+  uint32_t pad;
+  unsigned long long counters[4];
+  unsigned long long pad2;
+};
+
+// The device side of fw_walk_batch: start vertices and path matrices of the batches in flight, their parking lists,
+// launch records, streams and events.  Kept with the graph from one call to the next and only ever grown.  A call that
+// allocated and freed them itself would cost the NEXT call's copy of the path matrix half its rate: memory that was
+// just freed keeps the device's copy engines busy for a few hundred milliseconds (measured: the 5.4 GB path matrix
+// of the largest benchmark configuration crosses the bus in 95 ms, and in 178 ms when 14 GB were freed 125 ms before).
+struct BatchCache {
+  int32_t* d_starts = nullptr;
+  int32_t* d_paths = nullptr;
+  Scratch* d_scr = nullptr;
+  size_t starts_cap = 0, paths_cap = 0, scr_cap = 0;  // elements
+  ParkBuffers pbs[2];
+  hipStream_t streams[2] = {nullptr, nullptr};
+  std::vector<hipEvent_t> events;
+  size_t bytes() const {
+    size_t b = starts_cap * sizeof(int32_t) + paths_cap * sizeof(int32_t) + scr_cap * sizeof(Scratch);
+    for (const ParkBuffers& pb : pbs) b += pb.cap * 72u;  // about what the lists of a query take
+    return b;
+  }
+  void release() {
+    if (d_starts) (void)hipFree(d_starts);
+    if (d_paths) (void)hipFree(d_paths);
+    if (d_scr) (void)hipFree(d_scr);
+    d_starts = d_paths = nullptr;
+    d_scr = nullptr;
+    starts_cap = paths_cap = scr_cap = 0;
+    for (ParkBuffers& pb : pbs) pb.release();
+    for (hipStream_t& s : streams) {
+      if (s) (void)hipStreamDestroy(s);
+      s = nullptr;
+    }
+    for (hipEvent_t e : events) (void)hipEventDestroy(e);
+    events.clear();
+  }
+};
+
+static void release_batch_cache(fw_graph* g) {
+  BatchCache* c = static_cast<BatchCache*>(g->batch_cache);
+  if (c) {
+    c->release();
+    delete c;
+  }
+  g->batch_cache = nullptr;
+}
+
 // Rows the two-pass steps of a call need: every hub that has rows, once per label a walker can want.
 static uint64_t two_pass_rows(const fw_graph* g, int labels) {
   const uint64_t rows = (uint64_t)g->hub_rows * (uint64_t)labels;
@@ -1513,12 +1566,6 @@ static TrafficModel traffic_model(const fw_walk_params* p, int32_t n, bool parke
   return m;
 }
 
-struct Scratch {  // dispenser word + workload counters of the two kernels, 48 bytes per launch slot
-  uint32_t dispenser;
-  uint32_t pad;
-  unsigned long long counters[4];
-  unsigned long long pad2;
-};
 
 // One walk call at a time per graph: the parking index, the parking lists and the launch record are cached in the
 // graph, so a second call that started while one is running would rebuild or overwrite them under it.
@@ -1760,10 +1807,15 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
   if (rc != FW_OK) return rc;
   BusyGuard busy(g);
   if (!busy.ok()) return FW_ERR_INVALID;
+  fw_graph* const mg = const_cast<fw_graph*>(g);
+  if (!mg->batch_cache) mg->batch_cache = new (std::nothrow) BatchCache;
+  BatchCache* const bc = static_cast<BatchCache*>(mg->batch_cache);
+  if (!bc) { fw_set_error("fw_walk_batch: out of host memory"); return FW_ERR_NOMEM; }
   if (batch_size == 0) {  // autobatch, src/main.cu:259-271 with the default 512 MB headroom
     size_t free_b = 0, total_b = 0;
     rc = fw_device_mem_info(&free_b, &total_b);
     if (rc != FW_OK) return rc;
+    free_b += bc->bytes();  // what the last call left with the graph is this call's to use
     batch_size = fw_autobatch_size(free_b, 512, p->max_depth, sync, (uint32_t)n);
     if (batch_size == 0) { fw_set_error("autobatch: not enough free device memory"); return FW_ERR_NOMEM; }
     if (resolve_park_threshold(g, p, (int32_t)batch_size) != INT_MAX) {
@@ -1775,54 +1827,71 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
     }
   }
   if (batch_size > (uint32_t)n) batch_size = (uint32_t)n;
-  const int nbuf = sync ? 1 : 2;
   const size_t bs = batch_size;
   const size_t md = (size_t)p->max_depth;
+  const int nbatch = (int)(((size_t)n + bs - 1) / bs);
+  const int nbuf = sync || nbatch == 1 ? 1 : 2;  // buffers in flight
 
   const int32_t park_threshold = resolve_park_threshold(g, p, (int32_t)bs);
   bool use_pb = false;
   if (park_threshold != INT_MAX) {
-    rc = ensure_hub_index(const_cast<fw_graph*>(g), park_threshold);
+    rc = ensure_hub_index(mg, park_threshold);
     if (rc != FW_OK) return rc;
     // buckets = parked-on vertices x labels must stay a 30-bit count (bucket ids travel in 32-bit record fields)
     use_pb = g->n_hubs > 0 &&
              (int64_t)g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1) <= ((int64_t)1 << 30);
   }
-  ParkBuffers pbs[2];
-  int32_t* d_starts = nullptr;
-  int32_t* d_paths = nullptr;
-  Scratch* d_scr = nullptr;
-  hipStream_t streams[2] = {nullptr, nullptr};
-  std::vector<hipEvent_t> events;
-  auto cleanup = [&]() {
-    for (hipEvent_t e : events) (void)hipEventDestroy(e);
-    for (int i = 0; i < 2; ++i) if (streams[i]) (void)hipStreamDestroy(streams[i]);
-    if (d_starts) (void)hipFree(d_starts);
-    if (d_paths) (void)hipFree(d_paths);
-    if (d_scr) (void)hipFree(d_scr);
-    pbs[0].release();
-    pbs[1].release();
-  };
-  FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_starts), bs * nbuf * sizeof(int32_t)));
-  FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_paths), bs * nbuf * md * sizeof(int32_t)));
+  // The buffers stay with the graph (see BatchCache); a failed call gives them up.
+  auto cleanup = [&]() { release_batch_cache(mg); };
+  if (bc->starts_cap < bs * (size_t)nbuf) {
+    if (bc->d_starts) (void)hipFree(bc->d_starts);
+    bc->d_starts = nullptr;
+    bc->starts_cap = 0;
+    FW_TRY(hipMalloc(reinterpret_cast<void**>(&bc->d_starts), bs * (size_t)nbuf * sizeof(int32_t)));
+    bc->starts_cap = bs * (size_t)nbuf;
+  }
+  if (bc->paths_cap < bs * (size_t)nbuf * md) {
+    if (bc->d_paths) (void)hipFree(bc->d_paths);
+    bc->d_paths = nullptr;
+    bc->paths_cap = 0;
+    FW_TRY(hipMalloc(reinterpret_cast<void**>(&bc->d_paths), bs * (size_t)nbuf * md * sizeof(int32_t)));
+    bc->paths_cap = bs * (size_t)nbuf * md;
+  }
   if (use_pb) {
+    const int n_buckets = g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1);
+    const uint64_t rows = two_pass_rows(g, p->app == FW_APP_METAPATH ? p->schema_len : 1);
     for (int i = 0; i < nbuf && use_pb; ++i) {
-      rc = pbs[i].alloc(bs, g->n_hubs * (p->app == FW_APP_METAPATH ? p->schema_len : 1),
-                        two_pass_rows(g, p->app == FW_APP_METAPATH ? p->schema_len : 1));
-      if (rc != FW_OK) {  // no room for the parking lists: walk without parking (same results)
-        pbs[0].release();
-        pbs[1].release();
+      ParkBuffers& pb = bc->pbs[i];
+      if (pb.cap >= bs && pb.n_buckets == n_buckets && pb.rows_cap >= rows) continue;
+      pb.release();
+      if (pb.alloc(bs, n_buckets, rows) != FW_OK) {  // no room for the parking lists: walk without parking (same results)
+        bc->pbs[0].release();
+        bc->pbs[1].release();
         use_pb = false;
         (void)hipGetLastError();
       }
     }
   }
-  const int nbatch = (int)(((size_t)n + bs - 1) / bs);
-  FW_TRY(hipMalloc(reinterpret_cast<void**>(&d_scr), sizeof(Scratch) * (size_t)nbatch));
-  FW_TRY(hipMemset(d_scr, 0, sizeof(Scratch) * (size_t)nbatch));
-  for (int i = 0; i < nbuf; ++i) FW_TRY(hipStreamCreate(&streams[i]));
-  events.resize((size_t)nbatch * 2, nullptr);
-  for (auto& e : events) FW_TRY(hipEventCreate(&e));
+  if (bc->scr_cap < (size_t)nbatch) {
+    if (bc->d_scr) (void)hipFree(bc->d_scr);
+    bc->d_scr = nullptr;
+    bc->scr_cap = 0;
+    FW_TRY(hipMalloc(reinterpret_cast<void**>(&bc->d_scr), sizeof(Scratch) * (size_t)nbatch));
+    bc->scr_cap = (size_t)nbatch;
+  }
+  FW_TRY(hipMemset(bc->d_scr, 0, sizeof(Scratch) * (size_t)nbatch));
+  for (int i = 0; i < nbuf; ++i) if (!bc->streams[i]) FW_TRY(hipStreamCreate(&bc->streams[i]));
+  while (bc->events.size() < (size_t)nbatch * 2) {
+    hipEvent_t e = nullptr;
+    FW_TRY(hipEventCreate(&e));
+    bc->events.push_back(e);
+  }
+  ParkBuffers* const pbs = bc->pbs;
+  int32_t* const d_starts = bc->d_starts;
+  int32_t* const d_paths = bc->d_paths;
+  Scratch* const d_scr = bc->d_scr;
+  hipStream_t* const streams = bc->streams;
+  std::vector<hipEvent_t>& events = bc->events;
 
   fw_kargs a;
   fill_kargs(&a, g, p);
@@ -1863,7 +1932,6 @@ extern "C" int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const i
   }
   std::vector<Scratch> h((size_t)nbatch);
   FW_TRY(hipMemcpy(h.data(), d_scr, sizeof(Scratch) * (size_t)nbatch, hipMemcpyDeviceToHost));
-  cleanup();
   if (stats) {
     stats->kernel_ms = kernel_ms;
     stats->total_ms = total;

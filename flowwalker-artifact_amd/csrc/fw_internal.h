@@ -42,6 +42,7 @@ struct fw_graph {
                                       // NULL when the edge arrays live in host memory or there was no room
   struct fw_hub_info* hub_info = nullptr;  // [n_hubs]
   void* park_cache = nullptr;         // the parking lists of the last fw_walk_device call, kept for the next one
+  void* batch_cache = nullptr;        // the device buffers of the last fw_walk_batch call, kept for the next one
   void* call_scratch = nullptr;       // launch record (dispenser word + counters) of fw_walk_device, allocated once
   hipEvent_t call_ev[2] = {nullptr, nullptr};  // and its two timing events
   std::atomic<int> busy{0};           // a walk call is running on this graph (the caches above are per graph)

@@ -301,6 +301,10 @@ int fw_walk_device_noalloc(const fw_graph* g, const fw_walk_params* p, const int
  * sync != 0, timing_batch_sync (:468-523).  h_starts: int32[n]; h_paths: int32[n][max_depth],
  * caller-owned (pinned memory gives overlap, pageable works).  batch_size = 0: autobatch.
  * Walker ids are walker_base + query index, whatever the batch size.
+ * The device buffers of a call (start vertices, the path matrices of the one or two batches in flight, their parking
+ * lists) stay with the graph for the next call and are freed by fw_graph_destroy (the reference allocates and frees
+ * them per call, src/walk.cu:586-649): memory that was freed a moment ago keeps the device's copy engines busy, and
+ * the next call's path matrix would cross the bus at half its rate.  Autobatch counts them as free memory.
  */
 int fw_walk_batch(const fw_graph* g, const fw_walk_params* p, const int32_t* h_starts, int32_t n,
                   uint32_t batch_size, int sync, int32_t* h_paths, fw_walk_stats* stats);

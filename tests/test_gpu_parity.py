@@ -470,6 +470,27 @@ def test_kernel_times_on_request(gpu):
         g.destroy()
 
 
+def test_batch_calls_reuse_their_buffers(gpu):
+    """fw_walk_batch keeps its device buffers with the graph: calls of growing and shrinking size, other batch sizes,
+    another application (other parking lists) and a fw_walk_device call in between all give the walks of one plain call."""
+    csr = _graphs.hub_graph(V=30000, hub_degrees=(20000, 8000), base_degree=8, seed=5)
+    g = gpu.Graph.from_csr(*csr)
+    try:
+        rng = np.random.RandomState(4)
+        for app, n, bs, sync, extra in ((gpu.APP_DEEPWALK, 90000, 0, False, {}), (gpu.APP_DEEPWALK, 200000, 70001, False, {}),
+                                        (gpu.APP_METAPATH, 150000, 0, False, {"schema": [0, 1, 2]}),
+                                        (gpu.APP_DEEPWALK, 1000, 0, True, {}), (gpu.APP_PPR, 200000, 50000, True, {}),
+                                        (gpu.APP_NODE2VEC, 120000, 60000, False, {"p": 0.5, "q": 2.0})):
+            starts = rng.randint(0, 30000, size=n).astype(np.int32)
+            p = gpu.default_params(app=app, max_depth=13, seed=n, **extra)
+            want, st0 = g.walk(p, starts)
+            got, st = g.walk_batch(p, starts, batch_size=bs, sync=sync)
+            assert (got == want).all(), (app, n, bs)
+            assert (st.steps, st.sampled_edges) == (st0.steps, st0.sampled_edges)
+    finally:
+        g.destroy()
+
+
 def test_one_walk_call_at_a_time_per_graph(gpu):
     """The parking index, the parking lists and the launch record are cached in the fw_graph, so a second call on
     the same graph while one is running is refused with a status code (it used to race); afterwards the graph works
