@@ -491,6 +491,36 @@ def test_batch_calls_reuse_their_buffers(gpu):
         g.destroy()
 
 
+def test_graph_destroy_returns_the_cached_buffers(gpu):
+    """What the walk calls keep with a graph (parking lists, annotated adjacency, the batch call's buffers) goes with
+    fw_graph_destroy: a dozen create / walk / destroy cycles leave the free device memory where it was."""
+    import ctypes as C
+    csr = _graphs.hub_graph(V=30000, hub_degrees=(20000, 8000), base_degree=8, seed=5)
+    starts = np.random.RandomState(1).randint(0, 30000, size=300000).astype(np.int32)
+    p = gpu.default_params(app=gpu.APP_DEEPWALK, max_depth=41, seed=3)
+
+    def free_bytes():
+        f, t = C.c_size_t(0), C.c_size_t(0)
+        gpu.check(gpu.lib().fw_device_mem_info(C.byref(f), C.byref(t)))
+        return f.value
+
+    def cycle():
+        g = gpu.Graph.from_csr(*csr)
+        try:
+            a, st = g.walk_batch(p, starts, batch_size=100000)
+            assert st.hub_steps > 0
+            b, _ = g.walk(p, starts)
+            assert (a == b).all()
+        finally:
+            g.destroy()
+
+    cycle()  # what the runtime itself keeps after first use is allocated now
+    before = free_bytes()
+    for _ in range(12):
+        cycle()
+    assert abs(free_bytes() - before) <= 64 << 20  # a leak of the buffers would be 12 x 120 MB
+
+
 def test_one_walk_call_at_a_time_per_graph(gpu):
     """The parking index, the parking lists and the launch record are cached in the fw_graph, so a second call on
     the same graph while one is running is refused with a status code (it used to race); afterwards the graph works
